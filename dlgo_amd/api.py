@@ -1,0 +1,97 @@
+"""The Python entry point, in the manner of computerex/dlgo's dlgo.go: LoadLLM
+(:37) -> load_llm, (*LLM).Generate (:51) -> LLM.generate, GenerateStream (:79) ->
+LLM.generate_stream, Benchmark (:93) -> LLM.benchmark, ModelInfo (:117) ->
+LLM.model_info, and the With* options (:209-240).  Token ids go in and come out;
+tokenizers and chat templates are not part of this library.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, List, Optional, Sequence, Union
+
+import torch
+
+from .config import ModelConfig, load_config
+from .engine.engine import Engine
+from .engine.generate import Result, Stats, generate
+from .sampling import GenerateConfig, Option, Sampler, apply_options
+
+Prompt = Sequence[int]
+
+
+@dataclass
+class GenerateResult:
+    """dlgo.go:187-207: the output with the timings of the call."""
+    tokens: List[int]
+    finish_reason: str
+    tokens_per_sec: float
+    prefill_ms: float
+    generate_ms: float
+    output_tokens: int
+    prompt_tokens: int
+
+    def __str__(self) -> str:
+        return (f"{self.tokens_per_sec:.1f} tok/s | prefill: {self.prefill_ms:.0f}ms | gen: {self.generate_ms:.0f}ms | "
+                f"{self.output_tokens} tokens | {self.finish_reason}")
+
+
+class LLM:
+    def __init__(self, engine: Engine, max_batch: int = 64):
+        self.engine = engine
+        self.config: ModelConfig = engine.model.config
+        self.max_seq_len = engine.max_ctx
+        self.max_batch = max_batch
+        self.sampler = Sampler(engine.vocab, engine.device, max_rows=max_batch)
+        eos = getattr(self.config, "eos_token_ids", ())
+        self.stop_tokens = tuple(eos)
+
+    def _run(self, prompts: Sequence[Prompt], opts: Sequence[Option], on_token=None):
+        cfg = apply_options(opts)
+        results, stats = generate(self.engine, self.sampler, prompts, [cfg] * len(prompts), self.stop_tokens, on_token,
+                                  self.max_batch, sync=torch.cuda.synchronize)
+        return results, stats
+
+    @staticmethod
+    def _wrap(r: Result, s: Stats) -> GenerateResult:
+        return GenerateResult(r.tokens, r.finish_reason, s.tokens_per_sec, s.prefill_ms, s.generate_ms, len(r.tokens),
+                              r.prompt_tokens)
+
+    def generate(self, prompt: Union[Prompt, Sequence[Prompt]], *opts: Option):
+        """One prompt (a list of token ids) -> GenerateResult; a list of prompts -> a list of them, run as
+        batches of unequal lengths."""
+        many = len(prompt) > 0 and not isinstance(prompt[0], int)
+        prompts = list(prompt) if many else [prompt]
+        results, stats = self._run(prompts, opts)
+        out = [self._wrap(r, stats) for r in results]
+        return out if many else out[0]
+
+    def generate_stream(self, prompt: Prompt, on_token: Callable[[int], None], *opts: Option) -> GenerateResult:
+        """on_token(token id) is called for every token as it is generated (dlgo.go:79-90)."""
+        results, stats = self._run([prompt], opts, on_token=lambda i, t: on_token(t))
+        return self._wrap(results[0], stats)
+
+    def benchmark(self, prompt: Prompt, *opts: Option) -> GenerateResult:
+        """A run with separate prefill and generation timings (dlgo.go:93-114)."""
+        return self.generate(prompt, *opts)
+
+    def model_info(self) -> str:
+        """dlgo.go:170-185."""
+        c = self.config
+        g = lambda k: getattr(c, k, "?")
+        return (f"{c.architecture} | {g('num_hidden_layers')} layers | {g('hidden_size')} dim | "
+                f"{g('num_attention_heads')} heads ({g('num_key_value_heads')} KV) | {g('intermediate_size')} FFN | "
+                f"vocab {g('vocab_size')} | ctx {self.max_seq_len} | {str(self.engine.dtype).replace('torch.', '')}")
+
+
+def load_llm(path: str, max_seq_len: int = 0, dtype: str = "bfloat16", device: str = "cuda:0", max_batch: int = 64,
+             max_tokens: Optional[int] = None, **engine_options) -> LLM:
+    """Load a model folder (config.json, model.safetensors).  max_seq_len <= 0 or beyond the model's
+    context means the model's context (models/llm/generate.go:56-58).  The cache is sized for
+    `max_tokens` tokens over all live sequences (default: max_batch sequences of max_seq_len, at most 2^20)."""
+    config = load_config(path)
+    limit = getattr(config, "max_position_embeddings", None)
+    ctx = max_seq_len if max_seq_len > 0 and (limit is None or max_seq_len <= limit) else limit
+    if max_tokens is None:
+        max_tokens = min(max_batch * ctx, 1 << 20)
+    engine = Engine.from_folder(path, dtype, device, max_tokens=max_tokens, max_ctx=ctx, **engine_options)
+    return LLM(engine, max_batch)

@@ -1,0 +1,300 @@
+"""The cache: a slot for each live sequence, paged keys and values for each run
+of a layer, and fixed-size per-sequence state beside them.
+
+computerex/dlgo keeps one sequence: per layer `Keys, Vals [maxPos][kvDim]` and a
+length (memory/kvcache.go:5-36), reset by setting the length to zero without
+clearing (kvcache.go:25-27,74-78), and for recurrent layers a fixed-size state
+that is zero-filled on reset (memory/ssmstate.go:4-69).  Here:
+
+* a *slot* is one live sequence: its length and, per group, the pages it holds;
+* cache units (one per run of a layer that keeps keys/values) with equal needs
+  (kv heads, head size, window) form a *group* with storage of its own: a pool of
+  pages of 64 tokens, one page id covering all units of the group, and a page
+  table [slot, page index] the kernels read.  A windowed group gives pages back
+  as soon as no later token can see them and has a smaller pool;
+* giving a slot back returns its pages at once; data is never cleared, because
+  attention reads positions below the length only;
+* fixed-size state lives in [slot, ...] tensors per unit and is zeroed when a
+  slot is handed out.
+
+The bookkeeping is plain host code and runs without a GPU.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..parts.base import CacheNeed
+
+PAGE = 64
+
+
+class CacheError(RuntimeError):
+    pass
+
+
+class OutOfPages(CacheError):
+    pass
+
+
+class PagePool:
+    """Free list of page ids with double-free and foreign-id checks."""
+
+    def __init__(self, n_pages: int):
+        self.n_pages = n_pages
+        self._free = list(range(n_pages - 1, -1, -1))   # pop() hands out low ids first
+        self._held = np.zeros(n_pages, dtype=bool)
+
+    @property
+    def n_free(self) -> int:
+        return len(self._free)
+
+    def take(self, n: int) -> List[int]:
+        if n > len(self._free):
+            raise OutOfPages(f"cache full: {n} pages wanted, {len(self._free)} of {self.n_pages} free")
+        out = [self._free.pop() for _ in range(n)]
+        self._held[out] = True
+        return out
+
+    def give(self, pages: Sequence[int]) -> None:
+        for p in pages:
+            if not (0 <= p < self.n_pages) or not self._held[p]:
+                raise CacheError(f"page {p} given back but not held")
+            self._held[p] = False
+            self._free.append(p)
+
+
+@dataclass
+class GroupSpec:
+    kv_heads: int
+    head_dim: int
+    window: Optional[int]
+    units: List[int] = field(default_factory=list)     # cache unit ids, in storage order
+
+
+class KVGroup:
+    def __init__(self, spec: GroupSpec, n_pages: int, max_slots: int, max_pages_per_seq: int,
+                 dtype: torch.dtype, device: torch.device):
+        self.spec = spec
+        self.pool = PagePool(n_pages)
+        self.unit_elems = 2 * spec.kv_heads * PAGE * spec.head_dim     # keys then values of one unit in a page
+        self.page_stride = self.unit_elems * len(spec.units)
+        self.v_off = spec.kv_heads * PAGE * spec.head_dim
+        # never cleared and never read beyond a sequence's length
+        self.storage = torch.empty(n_pages * self.page_stride, dtype=dtype, device=device)
+        self.table_host = np.full((max_slots, max_pages_per_seq), -1, dtype=np.int32)
+        self.table = torch.full((max_slots, max_pages_per_seq), -1, dtype=torch.int32, device=device)
+        self.dirty: set = set()
+
+    def unit_view(self, index_in_group: int) -> torch.Tensor:
+        """Storage from the first element of this unit's part of page 0."""
+        return self.storage[index_in_group * self.unit_elems:]
+
+    def first_needed_page(self, length: int) -> int:
+        """Lowest page index that a token at position >= length can still see."""
+        if self.spec.window is None:
+            return 0
+        lo = length - self.spec.window + 1
+        return max(0, lo) // PAGE
+
+
+class Cache:
+    def __init__(self, unit_needs: Sequence[Sequence[CacheNeed]], max_tokens: int, max_ctx: int, dtype: torch.dtype,
+                 device, max_slots: Optional[int] = None, max_step_tokens: Optional[int] = None):
+        """unit_needs[u]: what cache unit u asks for.  max_tokens: the most tokens live sequences hold together,
+        each sequence rounded up to whole pages.  max_ctx: the longest sequence."""
+        self.device = torch.device(device)
+        self.dtype = dtype
+        if max_tokens < 1 or max_ctx < 1:
+            raise CacheError("cache: max_tokens and max_ctx must be positive")
+        self.n_pages = (max_tokens + PAGE - 1) // PAGE
+        self.max_ctx = min(max_ctx, self.n_pages * PAGE)
+        self.max_pages_per_seq = (self.max_ctx + PAGE - 1) // PAGE
+        self.max_slots = max_slots if max_slots is not None else min(self.n_pages, 4096)
+        self.max_step_tokens = max_step_tokens or self.max_ctx
+
+        self.groups: List[KVGroup] = []
+        self.unit_group: Dict[int, Tuple[int, int]] = {}     # unit -> (group index, index in group)
+        self.state: Dict[int, torch.Tensor] = {}            # unit -> [max_slots, *shape]
+        specs: Dict[Tuple[int, int, Optional[int]], GroupSpec] = {}
+        for u, needs in enumerate(unit_needs):
+            for need in needs:
+                if need.kind == "kv":
+                    key = (need.kv_heads, need.head_dim, need.window)
+                    if need.kv_heads < 1 or need.head_dim < 1 or (need.window is not None and need.window < 1):
+                        raise CacheError(f"cache unit {u}: bad key/value need {need}")
+                    spec = specs.setdefault(key, GroupSpec(*key))
+                    if u in self.unit_group:
+                        raise CacheError(f"cache unit {u} asks for keys/values twice")
+                    self.unit_group[u] = (list(specs).index(key), len(spec.units))
+                    spec.units.append(u)
+                elif need.kind == "state":
+                    if u in self.state:
+                        raise CacheError(f"cache unit {u} asks for state twice")
+                    self.state[u] = torch.zeros((self.max_slots, *need.state_shape), dtype=need.state_dtype, device=self.device)
+                elif need.kind != "none":
+                    raise CacheError(f"cache unit {u}: unknown need kind {need.kind!r}")
+        for spec in specs.values():
+            n_pages = self.n_pages
+            if spec.window is not None:
+                per_seq = (spec.window + min(self.max_step_tokens, self.max_ctx) + PAGE - 1) // PAGE + 1
+                n_pages = min(n_pages, self.max_slots * per_seq)
+            self.groups.append(KVGroup(spec, n_pages, self.max_slots, self.max_pages_per_seq, dtype, self.device))
+
+        self._free_slots = list(range(self.max_slots - 1, -1, -1))
+        self._live = np.zeros(self.max_slots, dtype=bool)
+        self.lengths = np.zeros(self.max_slots, dtype=np.int64)
+        # pages held per slot and group: page index -> page id
+        self._held: List[List[Dict[int, int]]] = [[{} for _ in self.groups] for _ in range(self.max_slots)]
+
+    # -- slots ---------------------------------------------------------------
+    @property
+    def n_free_slots(self) -> int:
+        return len(self._free_slots)
+
+    def live_slots(self) -> List[int]:
+        return [int(s) for s in np.nonzero(self._live)[0]]
+
+    def alloc_slot(self) -> int:
+        if not self._free_slots:
+            raise CacheError(f"no free slot: all {self.max_slots} are in use")
+        slot = self._free_slots.pop()
+        self._live[slot] = True
+        self.lengths[slot] = 0
+        for t in self.state.values():
+            t[slot].zero_()
+        return slot
+
+    def free_slot(self, slot: int) -> None:
+        self._check_live(slot)
+        for gi, g in enumerate(self.groups):
+            held = self._held[slot][gi]
+            g.pool.give(list(held.values()))
+            if held:
+                g.table_host[slot, list(held.keys())] = -1
+                g.dirty.add(slot)
+            held.clear()
+        self._live[slot] = False
+        self.lengths[slot] = 0
+        self._free_slots.append(slot)
+
+    def _check_live(self, slot: int) -> None:
+        if not (0 <= slot < self.max_slots) or not self._live[slot]:
+            raise CacheError(f"slot {slot} is not in use")
+
+    def length(self, slot: int) -> int:
+        self._check_live(slot)
+        return int(self.lengths[slot])
+
+    # -- pages ---------------------------------------------------------------
+    def pages_wanted(self, slot: int, new_len: int, group: int) -> List[int]:
+        """Page indices the slot lacks in `group` to hold positions below new_len."""
+        g = self.groups[group]
+        held = self._held[slot][group]
+        first = g.first_needed_page(int(self.lengths[slot]))
+        last = (new_len - 1) // PAGE
+        return [i for i in range(first, last + 1) if i not in held]
+
+    def can_reserve(self, wants: Sequence[Tuple[int, int]]) -> Optional[str]:
+        """None if every (slot, new_len) fits, else the reason."""
+        for slot, new_len in wants:
+            self._check_live(slot)
+            if new_len > self.max_ctx:
+                return f"slot {slot}: {new_len} tokens exceed the context of {self.max_ctx}"
+        for gi, g in enumerate(self.groups):
+            if g.spec.window is not None:
+                continue   # bounded by construction: steps are cut to max_step_tokens
+            need = sum(len(self.pages_wanted(s, n, gi)) for s, n in wants)
+            if need > g.pool.n_free:
+                return f"cache full: the step needs {need} more pages of {PAGE} tokens, {g.pool.n_free} of {g.pool.n_pages} are free"
+        return None
+
+    def reserve(self, wants: Sequence[Tuple[int, int]]) -> None:
+        """Make room so that each slot can hold positions below its new length."""
+        why = self.can_reserve(wants)
+        if why:
+            raise OutOfPages(why)
+        for gi, g in enumerate(self.groups):
+            for slot, new_len in wants:
+                idx = self.pages_wanted(slot, new_len, gi)
+                if not idx:
+                    continue
+                pages = g.pool.take(len(idx))
+                for i, p in zip(idx, pages):
+                    self._held[slot][gi][i] = p
+                    g.table_host[slot, i] = p
+                g.dirty.add(slot)
+
+    def advance(self, slot: int, n_tokens: int) -> None:
+        """The slot now holds n_tokens more; pages no later token can see go back to their pool."""
+        self._check_live(slot)
+        self.lengths[slot] += n_tokens
+        for gi, g in enumerate(self.groups):
+            if g.spec.window is None:
+                continue
+            first = g.first_needed_page(int(self.lengths[slot]))
+            held = self._held[slot][gi]
+            gone = [i for i in held if i < first]
+            if gone:
+                g.pool.give([held.pop(i) for i in gone])
+                g.table_host[slot, gone] = -1
+                g.dirty.add(slot)
+
+    def sync_tables(self) -> None:
+        """Bring the device page tables up to date (rows of slots that changed)."""
+        for g in self.groups:
+            if not g.dirty:
+                continue
+            rows = sorted(g.dirty)
+            g.dirty.clear()
+            idx = torch.as_tensor(rows, dtype=torch.int64)
+            host = torch.from_numpy(g.table_host[rows])
+            if self.device.type == "cuda":
+                g.table.index_copy_(0, idx.to(self.device), host.to(self.device))
+            else:
+                g.table.index_copy_(0, idx, host)
+
+    # -- views for the parts --------------------------------------------------
+    def kv_view(self, unit: int) -> "KVView":
+        gi, ui = self.unit_group[unit]
+        g = self.groups[gi]
+        return KVView(g.unit_view(ui), g.page_stride, g.v_off, g.table, g.spec.kv_heads, g.spec.head_dim, g.spec.window)
+
+    def state_of(self, unit: int) -> torch.Tensor:
+        return self.state[unit]
+
+    def held_pages(self, slot: int, group: int = 0) -> Dict[int, int]:
+        return dict(self._held[slot][group])
+
+    def check_consistent(self) -> None:
+        """No page lost, none held twice (used by tests and cheap enough to call anywhere)."""
+        for gi, g in enumerate(self.groups):
+            seen: Dict[int, int] = {}
+            for slot in range(self.max_slots):
+                for i, p in self._held[slot][gi].items():
+                    if not self._live[slot]:
+                        raise CacheError(f"free slot {slot} holds page {p}")
+                    if p in seen:
+                        raise CacheError(f"page {p} held by slots {seen[p]} and {slot}")
+                    seen[p] = slot
+                    if g.table_host[slot, i] != p:
+                        raise CacheError(f"page table of slot {slot} disagrees at index {i}")
+            if len(seen) + g.pool.n_free != g.pool.n_pages:
+                raise CacheError(f"group {gi}: {len(seen)} held + {g.pool.n_free} free != {g.pool.n_pages} pages")
+        if len(self._free_slots) + int(self._live.sum()) != self.max_slots or len(set(self._free_slots)) != len(self._free_slots):
+            raise CacheError("slot accounting broken")
+
+
+@dataclass
+class KVView:
+    """What an attention kernel needs of one cache unit."""
+    cache: torch.Tensor        # flat storage starting at this unit's part of page 0
+    page_stride: int           # elements from a page to the next
+    v_off: int                 # elements from a page's keys to its values
+    page_table: torch.Tensor   # [max_slots, max_pages] int32 on the device
+    kv_heads: int
+    head_dim: int
+    window: Optional[int]

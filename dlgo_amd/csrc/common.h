@@ -1,0 +1,83 @@
+// Shared by every kernel file: element types, conversions, wave reductions and
+// the error convention (an exported function returns nullptr on success, else a
+// message that names what was refused).  Everything here is written for gfx950:
+// 64-lane waves, MFMA, 160 KB of LDS per CU.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#define DLGO_DTYPE_F32 0
+#define DLGO_DTYPE_BF16 1
+
+#define WAVE 64
+
+typedef uint16_t bf16_t;   // storage only; arithmetic is always float
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+  static constexpr int code = DLGO_DTYPE_F32;
+  __device__ static __forceinline__ float load(const float* p) { return *p; }
+  __device__ static __forceinline__ void store(float* p, float v) { *p = v; }
+};
+template <> struct Elem<bf16_t> {
+  static constexpr int code = DLGO_DTYPE_BF16;
+  __device__ static __forceinline__ float load(const bf16_t* p) { return bf16_to_f32(*p); }
+  __device__ static __forceinline__ void store(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+  return v;
+}
+
+// Sum over a block of NW waves; every thread gets the result.  `red` holds NW floats.
+template <int NW>
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  v = wave_sum(v);
+  if (NW == 1) return v;
+  const int w = threadIdx.x / WAVE;
+  __syncthreads();
+  if ((threadIdx.x & (WAVE - 1)) == 0) red[w] = v;
+  __syncthreads();
+  float t = 0.f;
+#pragma unroll
+  for (int i = 0; i < NW; ++i) t += red[i];
+  return t;
+}
+
+static thread_local char dlgo_errbuf[512];
+#define DLGO_FAIL(...)                                        \
+  do {                                                        \
+    snprintf(dlgo_errbuf, sizeof(dlgo_errbuf), __VA_ARGS__);  \
+    return dlgo_errbuf;                                       \
+  } while (0)
+#define DLGO_REQUIRE(cond, ...) \
+  do {                          \
+    if (!(cond)) DLGO_FAIL(__VA_ARGS__); \
+  } while (0)
+#define DLGO_LAUNCH_CHECK(what)                                             \
+  do {                                                                      \
+    hipError_t e_ = hipGetLastError();                                      \
+    if (e_ != hipSuccess) DLGO_FAIL("%s: launch failed: %s", what, hipGetErrorString(e_)); \
+  } while (0)

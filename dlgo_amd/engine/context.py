@@ -1,0 +1,65 @@
+"""What the parts see of one step: the rows' token ids, positions and sequences as
+device arrays, the cache, and scratch buffers that keep their addresses (so that
+a captured step can be replayed)."""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+
+class Workspace:
+    """Named scratch buffers with room for `max_rows` rows each; a buffer is allocated
+    at its first use and never moves afterwards."""
+
+    def __init__(self, device: torch.device, max_rows: int):
+        self.device = device
+        self.max_rows = max_rows
+        self._bufs: Dict[Tuple[str, int, torch.dtype], torch.Tensor] = {}
+
+    def get(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
+        rows, cols = int(shape[0]), int(np.prod(shape[1:], dtype=np.int64)) if len(shape) > 1 else 1
+        if rows > self.max_rows:
+            raise RuntimeError(f"workspace {name}: {rows} rows asked, room for {self.max_rows}")
+        key = (name, cols, dtype)
+        buf = self._bufs.get(key)
+        if buf is None:
+            buf = torch.empty((self.max_rows, cols), dtype=dtype, device=self.device)
+            self._bufs[key] = buf
+        return buf[:rows].view(rows, *shape[1:]) if len(shape) > 1 else buf[:rows, 0]
+
+    def bytes(self) -> int:
+        return sum(b.numel() * b.element_size() for b in self._bufs.values())
+
+
+class StepContext:
+    """Device arrays of a step (or of one piece of a step that was cut along its rows).
+
+    token_ids, positions, tok_seq: one entry per row (int32); tok_seq is the index of the row's
+    sequence in this step.  slots, start_pos, cu_q: one entry per sequence (cu_q one more): the
+    sequence's slot, the length it had before this step, and the offset of its first row.
+    The same numbers are kept on the host (`*_host`) for parts that plan launches.
+    """
+
+    def __init__(self, engine, n_seq: int, n_tokens: int, arrays: Dict[str, torch.Tensor], host: Dict[str, np.ndarray]):
+        self.engine = engine
+        self.cache = engine.cache
+        self.dtype: torch.dtype = engine.dtype
+        self.device: torch.device = engine.device
+        self.n_seq, self.n_tokens = n_seq, n_tokens
+        self.token_ids = arrays["token_ids"]
+        self.positions = arrays["positions"]
+        self.tok_seq = arrays["tok_seq"]
+        self.slots = arrays["slots"]
+        self.start_pos = arrays["start_pos"]
+        self.cu_q = arrays["cu_q"]
+        self.arrays = arrays
+        self.host = host
+        q_lens = host["q_lens"]
+        self.max_q_len = int(q_lens.max()) if n_seq else 0
+        self.is_decode = bool(n_seq) and self.max_q_len == 1
+        self.max_kv_len = int((host["start_pos"] + q_lens).max()) if n_seq else 0
+
+    def buffer(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
+        return self.engine.workspace.get(name, shape, dtype)

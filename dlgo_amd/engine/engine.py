@@ -1,0 +1,335 @@
+"""The step function: a batch of sequences, each bringing its next tokens (a whole
+prompt, a piece of one, or a single token), run as one flat batch of rows from
+the cache; logits come back for the rows that were asked for.
+
+computerex/dlgo has two functions for one sequence, Forward(token, pos)
+(models/llm/forward.go:123) and ForwardBatch(tokens, startPos)
+(models/llm/forward_batch.go:78), the latter returning the last position's
+logits only (:221-235).  Both write the new keys and values first and then attend
+over cache rows [0, startPos+p] (:143-207), which is why a continuation is the
+same computation as a prompt; the one function here relies on the same order.
+
+There is no padding: rows of all sequences lie one after another, each with its
+own position and sequence index.  A step with more rows than the workspace holds
+is cut along the rows into pieces, exact by the same argument.  A step of single
+tokens is captured once per batch size as a HIP graph and replayed.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from .. import models as _models  # noqa: F401  (registers the architectures)
+from ..cache import PAGE, Cache
+from ..config import ModelConfig, build_model, load_config
+from ..kernels import build as kernel_build
+from ..weights import load_state, load_weights, random_tensors
+from .context import StepContext, Workspace
+
+_RUN_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+               "f32": torch.float32}
+
+
+class EngineError(RuntimeError):
+    pass
+
+
+def run_dtype(name) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        if name not in (torch.bfloat16, torch.float32):
+            raise EngineError(f"the engine runs in bfloat16 or float32, not {name}")
+        return name
+    try:
+        return _RUN_DTYPES[str(name).lower()]
+    except KeyError:
+        raise EngineError(f"unknown dtype {name!r}: bfloat16 or float32") from None
+
+
+@dataclass
+class Entry:
+    """One sequence's part of a step: its slot, its next tokens, and the places among
+    these tokens whose logits are wanted."""
+    slot: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+
+
+@dataclass
+class _Graph:
+    graph: "torch.cuda.CUDAGraph"
+    batch: int
+    ctx: StepContext
+
+
+class Engine:
+    def __init__(self, model, dtype="bfloat16", device="cuda:0", max_tokens: int = 8192, max_ctx: Optional[int] = None,
+                 max_slots: Optional[int] = None, max_step_tokens: int = 8192, logits_rows: int = 1024,
+                 use_graphs: bool = True, graph_max_batch: int = 128):
+        """`model` holds its weights already (see from_folder / from_random)."""
+        if not torch.cuda.is_available():
+            raise EngineError("no HIP device: dlgo_amd runs on an AMD GPU only and has no CPU path")
+        self.model = model
+        self.dtype = run_dtype(dtype)
+        self.device = torch.device(device)
+        torch.cuda.set_device(self.device)
+        limit = getattr(model.config, "max_position_embeddings", None)
+        pages_tokens = ((max_tokens + PAGE - 1) // PAGE) * PAGE
+        self.max_ctx = min(x for x in (max_ctx, limit, pages_tokens) if x)
+        self.max_step_tokens = max(1, min(max_step_tokens, pages_tokens))
+        self.logits_rows = max(1, min(logits_rows, self.max_step_tokens))
+        kernel_build.ensure_built(model.kernel_variants(self.dtype))
+        self.cache = Cache(model.unit_needs, max_tokens, self.max_ctx, self.dtype, self.device, max_slots,
+                           self.max_step_tokens)
+        self.workspace = Workspace(self.device, self.max_step_tokens)
+        model.prepare(self.max_ctx, self.device)
+        self.vocab = model.vocab
+        self.use_graphs = use_graphs
+        self.graph_max_batch = min(graph_max_batch, self.max_step_tokens)
+        self._graphs: Dict[int, _Graph] = {}
+        self._graph_seen: Dict[int, int] = {}
+        self._static: Optional[Dict[str, torch.Tensor]] = None
+        self._static_logits: Optional[torch.Tensor] = None
+        self._meta_dev = torch.empty(0, dtype=torch.int32, device=self.device)
+        self._staging: List[Tuple[torch.Tensor, Optional[torch.cuda.Event]]] = []
+        self._staging_next = 0
+        self._logits_piece: Optional[torch.Tensor] = None
+        self.steps_run = 0
+
+    # -- construction ------------------------------------------------------------
+    @classmethod
+    def from_folder(cls, folder: str, dtype="bfloat16", device="cuda:0", **kw) -> "Engine":
+        config = load_config(folder)
+        model = build_model(config)
+        load_weights(model, folder, device, run_dtype(dtype))
+        return cls(model, dtype, device, **kw)
+
+    @classmethod
+    def from_random(cls, config: ModelConfig, seed: int, dtype="bfloat16", device="cuda:0", std: Optional[float] = None,
+                    norm_jitter: float = 0.0, **kw) -> "Engine":
+        """Random weights drawn on the device and never written (benchmarks)."""
+        model = build_model(config)
+        rd = run_dtype(dtype)
+        tensors = random_tensors(config, seed, rd, std, norm_jitter, device=device)
+        load_state(model, tensors, device, rd, where="random weights")
+        del tensors
+        return cls(model, dtype, device, **kw)
+
+    # -- slots -------------------------------------------------------------------
+    def open(self, n: int = 1) -> List[int]:
+        """Slots for n new sequences (all or none)."""
+        if n > self.cache.n_free_slots:
+            raise EngineError(f"{n} sequences asked, {self.cache.n_free_slots} slots free")
+        return [self.cache.alloc_slot() for _ in range(n)]
+
+    def close(self, slots: Sequence[int]) -> None:
+        for s in slots:
+            self.cache.free_slot(s)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    def free_slots(self) -> int:
+        return self.cache.n_free_slots
+
+    def free_pages(self) -> int:
+        """Pages (of 64 tokens) that new sequences can still take."""
+        full = [g.pool.n_free for g in self.cache.groups if g.spec.window is None]
+        return min(full) if full else self.cache.n_pages
+
+    # -- uploads -----------------------------------------------------------------
+    def _stage(self, n_ints: int) -> torch.Tensor:
+        """A pinned host buffer that no copy in flight still reads."""
+        if not self._staging:
+            self._staging = [(torch.empty(max(4096, n_ints), dtype=torch.int32, pin_memory=True), None) for _ in range(4)]
+        i = self._staging_next
+        self._staging_next = (i + 1) % len(self._staging)
+        buf, ev = self._staging[i]
+        if ev is not None:
+            ev.synchronize()
+        if buf.numel() < n_ints:
+            buf = torch.empty(n_ints * 2, dtype=torch.int32, pin_memory=True)
+        self._staging[i] = (buf, None)
+        return buf
+
+    def _upload(self, fields: Dict[str, np.ndarray], dest: Optional[torch.Tensor] = None) -> Dict[str, torch.Tensor]:
+        """One host-to-device copy for all the int32 arrays of a step."""
+        offs, total = {}, 0
+        for k, v in fields.items():
+            offs[k] = total
+            total += (len(v) + 3) // 4 * 4
+        host = self._stage(total)
+        hv = host.numpy()
+        for k, v in fields.items():
+            hv[offs[k]:offs[k] + len(v)] = v
+        if dest is None:
+            if self._meta_dev.numel() < total:
+                self._meta_dev = torch.empty(total * 2, dtype=torch.int32, device=self.device)
+            dest = self._meta_dev
+        dest[:total].copy_(host[:total], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        idx = (self._staging_next - 1) % len(self._staging)
+        self._staging[idx] = (self._staging[idx][0], ev)
+        return {k: dest[offs[k]:offs[k] + len(v)] for k, v in fields.items()}
+
+    # -- the step ----------------------------------------------------------------
+    def step(self, entries: Sequence[Entry], sink: Optional[Callable[[int, torch.Tensor], None]] = None) -> Optional[torch.Tensor]:
+        """Run the entries' tokens from the cache, as one batch; return float32 logits [wanted, vocab] in the
+        order of the entries and of their `want` lists.  With `sink`, logits are handed over in pieces as
+        sink(first_output_row, tensor) and nothing is returned (for outputs too large to keep)."""
+        entries = list(entries)
+        if not entries:
+            raise EngineError("step: no entries")
+        seen = set()
+        q_lens, starts = [], []
+        for e in entries:
+            if e.slot in seen:
+                raise EngineError(f"step: slot {e.slot} appears twice")
+            seen.add(e.slot)
+            try:
+                start = self.cache.length(e.slot)
+            except Exception as ex:
+                raise EngineError(f"step: {ex}") from None
+            n = len(e.tokens)
+            if n < 1:
+                raise EngineError(f"step: slot {e.slot} brings no tokens")
+            if start + n > self.max_ctx:
+                raise EngineError(f"step: slot {e.slot} would hold {start + n} tokens, the context is {self.max_ctx}")
+            for w in e.want:
+                if not 0 <= w < n:
+                    raise EngineError(f"step: slot {e.slot} wants logits at place {w} of {n} tokens")
+            q_lens.append(n)
+            starts.append(start)
+        tokens = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=sum(q_lens))
+        if tokens.min() < 0 or tokens.max() >= self.vocab:
+            bad = int(tokens[(tokens < 0) | (tokens >= self.vocab)][0])
+            raise EngineError(f"step: token id {bad} is outside the vocabulary of {self.vocab}")
+        why = self.cache.can_reserve([(e.slot, s + n) for e, s, n in zip(entries, starts, q_lens)])
+        if why:
+            raise EngineError(f"step: {why}")
+        self.steps_run += 1
+
+        if (self.use_graphs and sink is None and len(entries) <= self.graph_max_batch
+                and all(n == 1 for n in q_lens) and all(list(e.want) == [0] for e in entries)):
+            return self._decode_step(entries, tokens, starts)
+
+        # wanted rows: (output row, flat row), in output order
+        cu = np.concatenate([[0], np.cumsum(q_lens)])
+        wanted = [(int(cu[i]) + w) for i, e in enumerate(entries) for w in e.want]
+        n_out = len(wanted)
+        out = None
+        if sink is None:
+            out = torch.empty((n_out, self.vocab), dtype=torch.float32, device=self.device)
+        wanted_arr = np.asarray(wanted, dtype=np.int64)
+
+        total = int(cu[-1])
+        seq_of = np.repeat(np.arange(len(entries)), q_lens)
+        pos_all = np.concatenate([np.arange(s, s + n) for s, n in zip(starts, q_lens)])
+        for c0 in range(0, total, self.max_step_tokens):
+            c1 = min(total, c0 + self.max_step_tokens)
+            seqs = np.unique(seq_of[c0:c1])                     # sequences with rows in this piece, ascending
+            local_seq = np.searchsorted(seqs, seq_of[c0:c1])
+            piece_q = np.bincount(local_seq, minlength=len(seqs))
+            first_row = np.concatenate([[0], np.cumsum(piece_q)[:-1]])
+            piece_start = pos_all[c0:c1][first_row]
+            slots = np.array([entries[int(s)].slot for s in seqs], dtype=np.int64)
+            self.cache.reserve([(int(sl), int(st + q)) for sl, st, q in zip(slots, piece_start, piece_q)])
+            self.cache.sync_tables()
+            sel = np.nonzero((wanted_arr >= c0) & (wanted_arr < c1))[0]      # output rows served by this piece
+            fields = {
+                "token_ids": tokens[c0:c1].astype(np.int32),
+                "positions": pos_all[c0:c1].astype(np.int32),
+                "tok_seq": local_seq.astype(np.int32),
+                "slots": slots.astype(np.int32),
+                "start_pos": piece_start.astype(np.int32),
+                "cu_q": np.concatenate([[0], np.cumsum(piece_q)]).astype(np.int32),
+                "rows": (wanted_arr[sel] - c0).astype(np.int32),
+            }
+            arrays = self._upload(fields)
+            host = {"q_lens": piece_q, "start_pos": piece_start, "slots": slots}
+            ctx = StepContext(self, len(seqs), c1 - c0, arrays, host)
+            x = self.model.hidden(ctx, ctx.token_ids)
+            # runs of consecutive output rows, at most logits_rows each
+            i = 0
+            while i < len(sel):
+                j = i + 1
+                while j < len(sel) and sel[j] == sel[j - 1] + 1 and j - i < self.logits_rows:
+                    j += 1
+                o0 = int(sel[i])
+                if out is not None:
+                    self.model.logits(ctx, x, arrays["rows"][i:j], out[o0:o0 + (j - i)])
+                else:
+                    if self._logits_piece is None:
+                        self._logits_piece = torch.empty((self.logits_rows, self.vocab), dtype=torch.float32, device=self.device)
+                    piece = self._logits_piece[:j - i]
+                    self.model.logits(ctx, x, arrays["rows"][i:j], piece)
+                    sink(o0, piece)
+                i = j
+            for sl, q in zip(slots, piece_q):
+                self.cache.advance(int(sl), int(q))
+        return out
+
+    # -- single tokens, captured ---------------------------------------------------
+    def _static_arrays(self) -> Dict[str, torch.Tensor]:
+        if self._static is None:
+            b = self.graph_max_batch
+            meta = torch.zeros(4 * b + 8, dtype=torch.int32, device=self.device)
+            self._static = {"meta": meta}
+            self._static_logits = torch.empty((b, self.vocab), dtype=torch.float32, device=self.device)
+        return self._static
+
+    def _decode_fields(self, tokens: np.ndarray, starts: Sequence[int], slots: Sequence[int]) -> Dict[str, np.ndarray]:
+        b = len(slots)
+        return {
+            "token_ids": tokens.astype(np.int32),
+            "positions": np.asarray(starts, dtype=np.int32),
+            "slots": np.asarray(slots, dtype=np.int32),
+            "start_pos": np.asarray(starts, dtype=np.int32),
+            "tok_seq": np.arange(b, dtype=np.int32),
+            "cu_q": np.arange(b + 1, dtype=np.int32),
+        }
+
+    def _decode_step(self, entries: Sequence[Entry], tokens: np.ndarray, starts: Sequence[int]) -> torch.Tensor:
+        b = len(entries)
+        slots = [e.slot for e in entries]
+        self.cache.reserve([(s, st + 1) for s, st in zip(slots, starts)])
+        self.cache.sync_tables()
+        st = self._static_arrays()
+        # a fixed layout per batch size inside the static buffer: one copy brings all arrays
+        fields = self._decode_fields(tokens, starts, slots)
+        width = sum((len(v) + 3) // 4 * 4 for v in fields.values())
+        if st["meta"].numel() < width:
+            raise EngineError("decode step: static arrays too small")   # cannot happen: sized for graph_max_batch
+        arrays = self._upload(fields, dest=st["meta"])
+        logits = self._static_logits[:b]
+        g = self._graphs.get(b)
+        if g is not None:
+            g.graph.replay()
+        else:
+            host = {"q_lens": np.ones(b, dtype=np.int64), "start_pos": np.asarray(starts, dtype=np.int64),
+                    "slots": np.asarray(slots, dtype=np.int64)}
+            ctx = StepContext(self, b, b, arrays, host)
+            ctx.is_decode = True
+            x = self.model.hidden(ctx, ctx.token_ids)
+            self.model.logits(ctx, x, None, logits)
+            # the second time a batch size is seen it is worth capturing
+            self._graph_seen[b] = self._graph_seen.get(b, 0) + 1
+            if self._graph_seen[b] >= 2:
+                self._capture(b, ctx, logits)
+        for s in slots:
+            self.cache.advance(s, 1)
+        return logits
+
+    def _capture(self, b: int, ctx: StepContext, logits: torch.Tensor) -> None:
+        """Record the step for this batch size.  Recording runs nothing; the arrays the recorded kernels
+        read (token ids, positions, slots, page tables) live at fixed addresses and are refreshed before
+        each replay."""
+        graph = torch.cuda.CUDAGraph()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph):
+            x = self.model.hidden(ctx, ctx.token_ids)
+            self.model.logits(ctx, x, None, logits)
+        self._graphs[b] = _Graph(graph, b, ctx)

@@ -1,0 +1,241 @@
+"""Python faces of the HIP kernels: each checks on the host what its kernel and
+grid assume (device, dtype, contiguity, shapes), then launches on torch's current
+stream.  There is no other implementation behind these: on a machine without the
+GPU or the compiler they raise.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import Optional, Sequence
+
+import torch
+
+from . import build
+
+PAGE = 64   # tokens per cache page; the kernels are compiled with the same number
+
+EPI_STORE, EPI_ACCUM_F32, EPI_SWIGLU, EPI_STORE_F32 = 0, 1, 2, 3
+GEMM_AUTO, GEMM_STREAM, GEMM_TILE128, GEMM_TILE64, GEMM_TILE32 = 0, 1, 2, 3, 4
+
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise KernelError(f"kernels run in float32 or bfloat16, not {dtype}") from None
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> ctypes.c_void_p:
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def _need(t: torch.Tensor, name: str, dtype: Optional[torch.dtype] = None, dims: Optional[int] = None) -> None:
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise KernelError(f"{name}: expected a tensor on the GPU")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: expected {dtype}, found {t.dtype}")
+    if dims is not None and t.dim() != dims:
+        raise KernelError(f"{name}: expected {dims} dimensions, found shape {tuple(t.shape)}")
+
+
+def _rows(t: torch.Tensor, name: str) -> int:
+    """Row stride (elements) of a 2-d tensor whose rows are contiguous."""
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise KernelError(f"{name}: expected rows that are contiguous in memory, found shape {tuple(t.shape)} strides {t.stride()}")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+def _check(err: Optional[bytes]) -> None:
+    if err:
+        raise KernelError(err.decode())
+
+
+_protos_done: set = set()
+
+
+def _lib(module: str, defines=()):
+    lib = build.load(module, defines)
+    key = (module, tuple(defines))
+    if key not in _protos_done:
+        for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_attention_rows",
+                     "dlgo_attention_prefill", "dlgo_attention_decode", "dlgo_argmax", "dlgo_sample"):
+            if hasattr(lib, name):
+                getattr(lib, name).restype = ctypes.c_char_p
+        _protos_done.add(key)
+    return lib
+
+
+# ---------------------------------------------------------------------------
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, :] = table[ids[t], :] as float32."""
+    _need(table, "embed table", dims=2)
+    _need(ids, "token ids", torch.int32, 1)
+    _need(out, "embed output", torch.float32, 2)
+    n, d = ids.shape[0], table.shape[1]
+    if not table.is_contiguous() or not out.is_contiguous() or tuple(out.shape) != (n, d):
+        raise KernelError(f"embed: output {tuple(out.shape)} does not fit {n} tokens of width {d}")
+    _check(_lib("embed").dlgo_embed(_ptr(table), dtype_code(table.dtype), _ptr(ids), _ptr(out), n, d, table.shape[0], _stream()))
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+            rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[r] = rmsnorm(x[rows[r]] if rows is given else x[r]) * weight; x float32, out in its own dtype."""
+    _need(x, "rmsnorm input", torch.float32, 2)
+    _need(weight, "rmsnorm weight", torch.float32, 1)
+    _need(out, "rmsnorm output", dims=2)
+    d = x.shape[1]
+    n = out.shape[0]
+    if rows is not None:
+        _need(rows, "rmsnorm rows", torch.int32, 1)
+        if rows.shape[0] != n:
+            raise KernelError("rmsnorm: one output row per gathered row")
+    elif x.shape[0] != n:
+        raise KernelError(f"rmsnorm: {x.shape[0]} input rows, {n} output rows")
+    if weight.shape[0] != d or out.shape[1] != d or not x.is_contiguous() or not out.is_contiguous():
+        raise KernelError(f"rmsnorm: width mismatch or strided operands (x {tuple(x.shape)}, w {tuple(weight.shape)}, out {tuple(out.shape)})")
+    _check(_lib("rmsnorm").dlgo_rmsnorm(_ptr(x), _ptr(rows), _ptr(weight), _ptr(out), dtype_code(out.dtype), n, d,
+                                        ctypes.c_float(eps), _stream()))
+    return out
+
+
+def gemm(weight: torch.Tensor, x: torch.Tensor, out: torch.Tensor, epilogue: int = EPI_STORE,
+         kind: int = GEMM_AUTO) -> torch.Tensor:
+    """out (epilogue)= x @ weight.T with weight [N, K], x [T, K].
+
+    EPI_STORE: out [T, N] in the run dtype.  EPI_ACCUM_F32: out float32 [T, N], added to.
+    EPI_SWIGLU: weight rows are (gate_0, up_0, gate_1, up_1, ...), out [T, N/2] = silu(gate) * up.
+    EPI_STORE_F32: out float32 [T, N].
+    """
+    _need(weight, "gemm weight", dims=2)
+    _need(x, "gemm input", weight.dtype, 2)
+    n, k = weight.shape
+    t = x.shape[0]
+    if x.shape[1] != k:
+        raise KernelError(f"gemm: input width {x.shape[1]} does not match weight {tuple(weight.shape)}")
+    want_dtype = torch.float32 if epilogue in (EPI_ACCUM_F32, EPI_STORE_F32) else weight.dtype
+    _need(out, "gemm output", want_dtype, 2)
+    cols = n // 2 if epilogue == EPI_SWIGLU else n
+    if tuple(out.shape) != (t, cols):
+        raise KernelError(f"gemm: output {tuple(out.shape)}, expected {(t, cols)}")
+    _check(_lib("gemm").dlgo_gemm(_ptr(weight), _ptr(x), _ptr(out), dtype_code(weight.dtype), n, t, k,
+                                  _rows(weight, "gemm weight"), _rows(x, "gemm input"), _rows(out, "gemm output"),
+                                  epilogue, kind, _stream()))
+    return out
+
+
+def rope_kv(qkv: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, rot: int, interleaved: bool,
+            cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
+            tok_seq: Optional[torch.Tensor], slots: Optional[torch.Tensor], page_table: Optional[torch.Tensor],
+            cache: Optional[torch.Tensor], page_stride: int, v_off: int, write_kv: bool = True) -> None:
+    """Rotate the query heads of qkv [T, (H+2KV)*hd] in place; rotate the key heads and copy the value heads
+    into the cache page of each token (cache: the first element of this layer's pages)."""
+    _need(qkv, "qkv rows", dims=2)
+    _need(positions, "positions", torch.int32, 1)
+    t = qkv.shape[0]
+    if positions.shape[0] != t:
+        raise KernelError("rope_kv: one position per row")
+    table_rows = 0
+    if cos is not None:
+        _need(cos, "cos table", torch.float32, 2)
+        _need(sin, "sin table", torch.float32, 2)
+        if cos.shape != sin.shape or cos.shape[1] != rot // 2 or not cos.is_contiguous() or not sin.is_contiguous():
+            raise KernelError(f"rope_kv: tables {tuple(cos.shape)} do not fit a rotated width of {rot}")
+        table_rows = cos.shape[0]
+    max_pages = 0
+    if write_kv:
+        _need(tok_seq, "token->sequence", torch.int32, 1)
+        _need(slots, "slots", torch.int32, 1)
+        _need(page_table, "page table", torch.int32, 2)
+        _need(cache, "cache", qkv.dtype)
+        if tok_seq.shape[0] != t or not page_table.is_contiguous():
+            raise KernelError("rope_kv: one sequence index per row and a contiguous page table")
+        max_pages = page_table.shape[1]
+    _check(_lib("rope_kv").dlgo_rope_kv(_ptr(qkv), dtype_code(qkv.dtype), t, _rows(qkv, "qkv rows"), n_heads, n_kv, head_dim,
+                                        rot, int(interleaved), _ptr(cos), _ptr(sin), table_rows, _ptr(positions),
+                                        _ptr(tok_seq), _ptr(slots), _ptr(page_table), max_pages, _ptr(cache),
+                                        ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(write_kv), _stream()))
+
+
+def attention_rows(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
+                   positions: torch.Tensor, tok_seq: torch.Tensor, slots: torch.Tensor, page_table: torch.Tensor,
+                   cache: torch.Tensor, page_stride: int, v_off: int, window: int = 0,
+                   scale: Optional[float] = None) -> torch.Tensor:
+    """One wave per (row, head): the general kernel, every dtype, every step shape."""
+    _need(q, "query rows", dims=2)
+    _need(out, "attention output", q.dtype, 2)
+    for name, v in (("positions", positions), ("token->sequence", tok_seq), ("slots", slots)):
+        _need(v, name, torch.int32, 1)
+    _need(page_table, "page table", torch.int32, 2)
+    _need(cache, "cache", q.dtype)
+    t = q.shape[0]
+    if out.shape[0] != t or positions.shape[0] != t or tok_seq.shape[0] != t or not page_table.is_contiguous():
+        raise KernelError("attention: one position, sequence index and output row per query row")
+    if scale is None:
+        scale = 1.0 / math.sqrt(head_dim)
+    lib = _lib("attention", (("HEAD_DIM", head_dim),))
+    _check(lib.dlgo_attention_rows(_ptr(q), _rows(q, "query rows"), _ptr(out), _rows(out, "attention output"),
+                                   dtype_code(q.dtype), t, n_heads, n_kv, head_dim, _ptr(positions), _ptr(tok_seq),
+                                   _ptr(slots), _ptr(page_table), page_table.shape[1], _ptr(cache),
+                                   ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(window),
+                                   ctypes.c_float(scale), _stream()))
+    return out
+
+
+def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, positions: torch.Tensor,
+              tok_seq: torch.Tensor, slots: torch.Tensor, page_table: torch.Tensor, cache: torch.Tensor, page_stride: int,
+              v_off: int, q_lens: Sequence[int], start_pos: Sequence[int], window: int = 0,
+              scale: Optional[float] = None) -> torch.Tensor:
+    """Attention of a step's query rows over the cache, with the kernel chosen by the step's shape
+    (q_lens, start_pos: per sequence, on the host).  All kernels compute the same thing."""
+    return attention_rows(q, out, n_heads, n_kv, head_dim, positions, tok_seq, slots, page_table, cache, page_stride,
+                          v_off, window, scale)
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _need(logits, "logits", torch.float32, 2)
+    _need(out, "argmax output", torch.int32, 1)
+    if out.shape[0] != logits.shape[0]:
+        raise KernelError("argmax: one output per row")
+    _check(_lib("sampling").dlgo_argmax(_ptr(logits), _rows(logits, "logits"), logits.shape[0], logits.shape[1], _ptr(out),
+                                        _stream()))
+    return out
+
+
+def sample(logits: torch.Tensor, work: torch.Tensor, e: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
+           top_p: torch.Tensor, min_p: torch.Tensor, penalty: torch.Tensor, recent: Optional[torch.Tensor],
+           uniform: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _need(logits, "logits", torch.float32, 2)
+    n, v = logits.shape
+    for name, t, dt in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
+                        ("top_p", top_p, torch.float32), ("min_p", min_p, torch.float32),
+                        ("penalty", penalty, torch.float32), ("uniform", uniform, torch.float32),
+                        ("sample output", out, torch.int32)):
+        _need(t, name, dt, 1)
+        if t.shape[0] != n:
+            raise KernelError(f"sample: {name} has {t.shape[0]} entries for {n} rows")
+    for name, t in (("work", work), ("e", e)):
+        _need(t, name, torch.float32, 2)
+        if t.shape[0] < n or t.shape[1] != v or not t.is_contiguous():
+            raise KernelError(f"sample: scratch {name} {tuple(t.shape)} too small for {(n, v)}")
+    n_recent = 0
+    if recent is not None:
+        _need(recent, "recent tokens", torch.int32, 2)
+        if recent.shape[0] != n or not recent.is_contiguous():
+            raise KernelError("sample: one row of recent tokens per row of logits")
+        n_recent = recent.shape[1]
+    _check(_lib("sampling").dlgo_sample(_ptr(logits), _rows(logits, "logits"), n, v, _ptr(work), _ptr(e), _ptr(temperature),
+                                        _ptr(top_k), _ptr(top_p), _ptr(min_p), _ptr(penalty), _ptr(recent), n_recent,
+                                        _ptr(uniform), _ptr(out), _stream()))
+    return out

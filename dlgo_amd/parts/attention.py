@@ -1,0 +1,107 @@
+"""The attention mixer: grouped-query attention over the paged cache.
+
+Per token (computerex/dlgo, models/llm/forward.go:207-290): q, k, v projections
+without bias (:224), rotation of each q and k head (:246-252), keys (rotated) and
+values stored at the token's position (:257), then for query head h the softmax
+over the scores against keys 0..p of KV head h // (H/KV), scaled by 1/sqrt(hd)
+(:258-278), and the output projection (:286).  The three projections are one
+matrix product against the fused [q|k|v] rows, the rotation and the cache write
+are one kernel, and the output projection adds into the float32 residual stream.
+
+The mixer's sizes are its parameters; `window` limits each token to the last
+`window` keys (layers/gqa.go:98-132).  A run of the layer that reads another
+run's cache computes queries only and stores nothing.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import CacheNeed, Part, TensorSpec, stored
+from .position import PositionEncoding
+
+
+class Mixer(Part):
+    """Interface of a sequence mixer.
+
+    cache_needs(): what one run of the layer keeps per sequence.
+    forward(xn, ctx, unit, residual, owns_cache): xn are the normed rows of the step (run dtype, [T, width]);
+    the result is added into `residual` (float32 [T, width]).  `unit` is the cache unit this run reads;
+    `owns_cache` is False when the unit belongs to another run (then nothing is stored).
+    A mixer with state must treat the rows of a sequence in order: ctx.cu_q gives each sequence's rows.
+    """
+
+    def cache_needs(self) -> List[CacheNeed]:
+        return []
+
+    def prepare(self, max_positions: int, device: torch.device) -> None:
+        pass
+
+    def forward(self, xn: torch.Tensor, ctx, unit: int, residual: torch.Tensor, owns_cache: bool = True) -> None:
+        raise NotImplementedError
+
+
+class Attention(Mixer):
+    kernel_modules = ("gemm", "rope_kv")
+
+    def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PositionEncoding,
+                 window: Optional[int] = None, scale: Optional[float] = None):
+        if n_heads % n_kv_heads:
+            raise ValueError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} kv heads")
+        if head_dim % 16:
+            raise ValueError(f"attention: head size {head_dim} is not a multiple of 16 (the kernels take steps of 16)")
+        self.width, self.n_heads, self.n_kv_heads, self.head_dim = width, n_heads, n_kv_heads, head_dim
+        self.q_dim, self.kv_dim = n_heads * head_dim, n_kv_heads * head_dim
+        self.position = position
+        self.window = window
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.w_qkv: Optional[torch.Tensor] = None
+        self.w_o: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {
+            "q_proj.weight": TensorSpec((self.q_dim, self.width)),
+            "k_proj.weight": TensorSpec((self.kv_dim, self.width)),
+            "v_proj.weight": TensorSpec((self.kv_dim, self.width)),
+            "o_proj.weight": TensorSpec((self.width, self.q_dim)),
+        }
+
+    def kernel_variants(self, dtype):
+        return (("gemm", ()), ("rope_kv", ()), ("attention", (("HEAD_DIM", self.head_dim),)))
+
+    def cache_needs(self) -> List[CacheNeed]:
+        return [CacheNeed(kind="kv", kv_heads=self.n_kv_heads, head_dim=self.head_dim, window=self.window)]
+
+    def prepare(self, max_positions: int, device: torch.device) -> None:
+        self.position.prepare(max_positions, device)
+
+    def load(self, tensors, device, dtype) -> None:
+        spec = self.tensor_specs()
+        fused = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], dim=0)
+        self.w_qkv = stored(fused, spec["q_proj.weight"], device, dtype)
+        self.w_o = stored(tensors["o_proj.weight"], spec["o_proj.weight"], device, dtype)
+
+    def forward(self, xn, ctx, unit, residual, owns_cache=True) -> None:
+        t = xn.shape[0]
+        n_kv = self.n_kv_heads if owns_cache else 0
+        cols = self.q_dim + 2 * n_kv * self.head_dim
+        qkv = ctx.buffer("attention.qkv", (t, self.q_dim + 2 * self.kv_dim), xn.dtype)
+        ops.gemm(self.w_qkv[:cols], xn, qkv[:, :cols])
+        kv = ctx.cache.kv_view(unit)
+        rot = self.position.rotation()
+        ops.rope_kv(qkv, self.n_heads, n_kv, self.head_dim, rot.width if rot else 0, rot.interleaved if rot else False,
+                    rot.cos if rot else None, rot.sin if rot else None, ctx.positions,
+                    ctx.tok_seq, ctx.slots, kv.page_table, kv.cache, kv.page_stride, kv.v_off, write_kv=owns_cache)
+        out = ctx.buffer("attention.out", (t, self.q_dim), xn.dtype)
+        self.attend(qkv, out, ctx, kv)
+        ops.gemm(self.w_o, out, residual, ops.EPI_ACCUM_F32)
+
+    def attend(self, q, out, ctx, kv) -> None:
+        """Attention of the step's (rotated) query rows over the cache; the kernel is chosen by the
+        step's shape and the run dtype, the arithmetic is the same."""
+        ops.attention(q, out, self.n_heads, self.n_kv_heads, self.head_dim, ctx.positions, ctx.tok_seq, ctx.slots,
+                      kv.page_table, kv.cache, kv.page_stride, kv.v_off, ctx.host["q_lens"], ctx.host["start_pos"],
+                      window=self.window or 0, scale=self.scale)

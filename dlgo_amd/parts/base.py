@@ -1,0 +1,80 @@
+"""What every part of a model has in common.
+
+A part owns tensors (declared by name and shape, relative to the prefix under
+which the model mounts it), is given them once at load time, and runs on the
+rows of a step.  It knows its own sizes and constants, never the model it sits
+in.  computerex/dlgo keeps the same independence through per-layer enum choices
+(models/llm/model.go:12-55) switched on in the forward pass
+(models/llm/forward.go:142-182); here each choice is an object with one
+interface per kind.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """A tensor a part expects: its shape, how it is stored, and how random
+    weights are drawn for it.
+
+    kind "matrix": operand of a matrix product, kept in the run dtype.
+    kind "vector": per-channel weights (norms), kept in float32 (exact from bfloat16).
+    kind "table":  integers, kept as int32.
+    init "normal": N(0, std) with std the configuration's initializer range;
+    init "ones":   1, or 1 + N(0, jitter) when the caller asks for jitter.
+    """
+    shape: Tuple[int, ...]
+    kind: str = "matrix"
+    init: str = "normal"
+
+
+class Part:
+    """Base of everything that may own tensors."""
+
+    #: kernel modules (names under csrc/) this part launches; built before first use
+    kernel_modules: Tuple[str, ...] = ()
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {}
+
+    def load(self, tensors: Dict[str, torch.Tensor], device: torch.device, dtype: torch.dtype) -> None:
+        """Take the tensors named in tensor_specs() (CPU, as stored) and keep them on
+        `device` the way the kernels want them."""
+
+    def kernel_variants(self, dtype: torch.dtype) -> Tuple[Tuple[str, Tuple[Tuple[str, int], ...]], ...]:
+        """(module, defines) pairs to compile for this part at `dtype`."""
+        return tuple((m, ()) for m in self.kernel_modules)
+
+
+def stored(t: torch.Tensor, spec: TensorSpec, device: torch.device, dtype: torch.dtype) -> torch.Tensor:
+    """The storage rule: matrices in the run dtype, vectors in float32, tables in int32."""
+    if spec.kind == "matrix":
+        return t.to(device=device, dtype=dtype).contiguous()
+    if spec.kind == "vector":
+        return t.to(device=device, dtype=torch.float32).contiguous()
+    if spec.kind == "table":
+        return t.to(device=device, dtype=torch.int32).contiguous()
+    raise ValueError(f"unknown tensor kind {spec.kind!r}")
+
+
+@dataclass
+class CacheNeed:
+    """What a mixer asks of the cache for one run of a layer.
+
+    kind "kv":    keys and values of every token (window None) or of the last
+                  `window` tokens; kv_heads x head_dim each.
+    kind "state": a fixed-size tensor per sequence (`state_shape`, `state_dtype`),
+                  zero when a sequence starts.
+    kind "none":  nothing.
+    A mixer may ask for both keys/values and state by returning two needs.
+    """
+    kind: str = "none"
+    kv_heads: int = 0
+    head_dim: int = 0
+    window: Optional[int] = None
+    state_shape: Tuple[int, ...] = ()
+    state_dtype: torch.dtype = torch.float32

@@ -1,0 +1,53 @@
+"""Token embedding and output head.  The embedding copies a table row per token,
+unscaled (computerex/dlgo, models/llm/forward.go:132-135); the head multiplies the
+normed rows by the output matrix, which is the embedding table when the model
+ties them (models/llm/loader.go:74-76; forward.go:193-201), into float32 logits."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import Part, TensorSpec, stored
+
+
+class Embedding(Part):
+    kernel_modules = ("embed",)
+
+    def __init__(self, vocab: int, width: int):
+        self.vocab, self.width = vocab, width
+        self.weight: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {"weight": TensorSpec((self.vocab, self.width))}
+
+    def load(self, tensors, device, dtype) -> None:
+        self.weight = stored(tensors["weight"], self.tensor_specs()["weight"], device, dtype)
+
+    def __call__(self, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        return ops.embed(self.weight, ids, out)
+
+
+class OutputHead(Part):
+    kernel_modules = ("gemm",)
+
+    def __init__(self, vocab: int, width: int, tied_to: Optional[Embedding] = None):
+        self.vocab, self.width = vocab, width
+        self.tied_to = tied_to
+        self._weight: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {} if self.tied_to is not None else {"weight": TensorSpec((self.vocab, self.width))}
+
+    def load(self, tensors, device, dtype) -> None:
+        if self.tied_to is None:
+            self._weight = stored(tensors["weight"], self.tensor_specs()["weight"], device, dtype)
+
+    @property
+    def weight(self) -> torch.Tensor:
+        return self.tied_to.weight if self.tied_to is not None else self._weight
+
+    def __call__(self, xn: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """xn: normed rows (run dtype); out: float32 [rows, vocab]."""
+        return ops.gemm(self.weight, xn, out, ops.EPI_STORE_F32)

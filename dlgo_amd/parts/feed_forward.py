@@ -1,0 +1,50 @@
+"""Feed-forward parts.  The gated one is SwiGLU as computerex/dlgo computes it
+(models/llm/forward.go:295-298; ops/activation.go:8-19,36-38): hid = silu(gate x) * (up x),
+out = down hid, no biases.  Gate and up rows are interleaved at load, so one matrix
+product yields both and its epilogue writes `hid` once; the down projection adds
+into the float32 residual stream."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..kernels import ops
+from .base import Part, TensorSpec, stored
+
+
+class FeedForward(Part):
+    """Interface: forward(xn, ctx, residual) adds the result for the step's rows into `residual`."""
+
+    def forward(self, xn: torch.Tensor, ctx, residual: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class GatedFeedForward(FeedForward):
+    kernel_modules = ("gemm",)
+
+    def __init__(self, width: int, inner: int, activation: str = "silu"):
+        if activation != "silu":
+            raise ValueError(f"gated feed-forward: activation {activation!r} has no kernel (silu has)")
+        self.width, self.inner = width, inner
+        self.w_gate_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        return {
+            "gate_proj.weight": TensorSpec((self.inner, self.width)),
+            "up_proj.weight": TensorSpec((self.inner, self.width)),
+            "down_proj.weight": TensorSpec((self.width, self.inner)),
+        }
+
+    def load(self, tensors, device, dtype) -> None:
+        spec = self.tensor_specs()
+        gate, up = tensors["gate_proj.weight"], tensors["up_proj.weight"]
+        inter = torch.stack([gate, up], dim=1).reshape(2 * self.inner, self.width)   # rows g0,u0,g1,u1,...
+        self.w_gate_up = stored(inter, spec["gate_proj.weight"], device, dtype)
+        self.w_down = stored(tensors["down_proj.weight"], spec["down_proj.weight"], device, dtype)
+
+    def forward(self, xn, ctx, residual) -> None:
+        hid = ctx.buffer("feed_forward.hidden", (xn.shape[0], self.inner), xn.dtype)
+        ops.gemm(self.w_gate_up, xn, hid, ops.EPI_SWIGLU)
+        ops.gemm(self.w_down, hid, residual, ops.EPI_ACCUM_F32)

@@ -1,0 +1,71 @@
+import copy
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs an AMD GPU (run on the MI355X box)")
+
+
+# Two tiny configurations of the architecture that differ in every size and option.
+TINY_A = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "vocab_size": 256, "hidden_size": 64, "num_hidden_layers": 2, "intermediate_size": 160,
+    "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 16,
+    "rms_norm_eps": 1e-5, "rope_theta": 10000.0, "rope_scaling": None,
+    "max_position_embeddings": 128, "tie_word_embeddings": True, "initializer_range": 0.02,
+    "hidden_act": "silu", "torch_dtype": "float32", "bos_token_id": 1, "eos_token_id": 2,
+}
+TINY_B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "vocab_size": 384, "hidden_size": 128, "num_hidden_layers": 3, "intermediate_size": 352,
+    "num_attention_heads": 4, "num_key_value_heads": 1, "head_dim": 32,
+    "rms_norm_eps": 1e-6, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 4.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 64},
+    "max_position_embeddings": 512, "tie_word_embeddings": False, "initializer_range": 0.02,
+    "hidden_act": "silu", "torch_dtype": "float32", "bos_token_id": 0, "eos_token_id": [3, 5],
+}
+# a third one with a head size that is neither a power of two nor hidden/heads, and more heads than fit one wave's tile
+TINY_C = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "vocab_size": 515, "hidden_size": 96, "num_hidden_layers": 2, "intermediate_size": 136,
+    "num_attention_heads": 6, "num_key_value_heads": 3, "head_dim": 48,
+    "rms_norm_eps": 3e-6, "rope_theta": 20000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 2.0,
+                     "original_max_position_embeddings": 32},
+    "max_position_embeddings": 640, "tie_word_embeddings": True, "initializer_range": 0.05,
+    "hidden_act": "silu", "torch_dtype": "bfloat16", "eos_token_id": 7,
+}
+
+
+@pytest.fixture
+def tiny_a():
+    return copy.deepcopy(TINY_A)
+
+
+@pytest.fixture
+def tiny_b():
+    return copy.deepcopy(TINY_B)
+
+
+@pytest.fixture
+def tiny_c():
+    return copy.deepcopy(TINY_C)
+
+
+def make_folder(raw, seed, path, dtype=None, std=None, norm_jitter=0.0):
+    """Write a random model folder for a raw config dict with the library's own writer."""
+    import torch
+    from dlgo_amd import models  # noqa: F401
+    from dlgo_amd.config import config_from_dict
+    from dlgo_amd.weights import write_random_model
+    dt = {None: None, "float32": torch.float32, "bfloat16": torch.bfloat16}[dtype]
+    return write_random_model(config_from_dict(raw), seed, str(path), dtype=dt, std=std, norm_jitter=norm_jitter)

@@ -1,0 +1,182 @@
+"""The engine against the plain implementation: each request alone and whole; with its last
+tokens one by one; in batches of unequal lengths whose shorter requests end earlier, one batch
+after another so that slots are used again; in float32 and in bfloat16."""
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as plain
+from conftest import TINY_A, TINY_B, TINY_C, make_folder
+
+pytestmark = pytest.mark.gpu
+
+CONFIGS = {"A": (TINY_A, dict()), "B": (TINY_B, dict(norm_jitter=0.1)), "C": (TINY_C, dict(norm_jitter=0.1, std=0.12))}
+# float32: the engine against float64 arithmetic on the same weights; bfloat16: against the same,
+# with the rounding of activations to 8 bits of mantissa at every layer
+TOL = {"float32": 2e-5, "bfloat16": 3e-2}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    out = {}
+    for name, (raw, kw) in CONFIGS.items():
+        for wdtype in ("float32", "bfloat16"):
+            d = tmp_path_factory.mktemp(f"tiny{name}_{wdtype}")
+            make_folder(raw, seed=11 + len(out), path=d, dtype=wdtype, **kw)
+            out[name, wdtype] = str(d)
+    return out
+
+
+@pytest.fixture(scope="module")
+def oracle(folders):
+    cache = {}
+
+    def get(name, wdtype, tokens):
+        key = (name, wdtype, tuple(tokens))
+        if key not in cache:
+            cfg, w = plain.read_model(folders[name, wdtype])
+            cache[key] = plain.forward(cfg, w, tokens)
+        return cache[key]
+    return get
+
+
+def engine_for(folder, dtype, **kw):
+    from dlgo_amd.engine import Engine
+    kw.setdefault("max_tokens", 2048)
+    return Engine.from_folder(folder, dtype, **kw)
+
+
+def rel_err(got, want):
+    got = np.asarray(got, dtype=np.float64)
+    return np.abs(got - want).max() / (np.abs(want).max() + 1e-30)
+
+
+def prompts_for(raw, lens, seed):
+    rng = np.random.default_rng(seed)
+    return [rng.integers(0, raw["vocab_size"], size=n).tolist() for n in lens]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole_prompt(folders, oracle, name, dtype):
+    from dlgo_amd.engine import Entry
+    raw = CONFIGS[name][0]
+    wdtype = dtype
+    eng = engine_for(folders[name, wdtype], dtype)
+    for tokens in prompts_for(raw, [1, 5, 70, 127], seed=3):
+        (slot,) = eng.open(1)
+        logits = eng.step([Entry(slot, tokens, list(range(len(tokens))))]).cpu().numpy()
+        eng.close([slot])
+        want = oracle(name, wdtype, tokens)
+        assert logits.shape == want.shape
+        assert np.isfinite(logits).all()
+        assert rel_err(logits, want) <= TOL[dtype], (name, dtype, len(tokens))
+    eng.cache.check_consistent()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("graphs", [False, True])
+def test_last_tokens_one_by_one(folders, oracle, name, dtype, graphs):
+    from dlgo_amd.engine import Entry
+    raw = CONFIGS[name][0]
+    eng = engine_for(folders[name, dtype], dtype, use_graphs=graphs)
+    (tokens,) = prompts_for(raw, [100], seed=5)
+    want = oracle(name, dtype, tokens)
+    (slot,) = eng.open(1)
+    head = len(tokens) - 32
+    rows = [eng.step([Entry(slot, tokens[:head], list(range(head)))]).cpu().numpy()]
+    for t in tokens[head:]:
+        rows.append(eng.step([Entry(slot, [t], [0])]).cpu().numpy().copy())
+    got = np.concatenate(rows)
+    assert rel_err(got, want) <= TOL[dtype]
+    # whole against one-by-one: the same numbers beyond rounding, also where the plain one is further away
+    eng.close([slot])
+    (slot,) = eng.open(1)
+    whole = eng.step([Entry(slot, tokens, list(range(len(tokens))))]).cpu().numpy()
+    assert rel_err(got, whole.astype(np.float64)) <= (1e-5 if dtype == "float32" else TOL[dtype])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_unequal_batches_with_slot_reuse(folders, oracle, name, dtype):
+    """Three batches one after another in a cache that holds one batch at a time; each batch's requests
+    start together with unequal prompts, go on one token per step, and end at different times."""
+    from dlgo_amd.engine import Entry
+    raw = CONFIGS[name][0]
+    eng = engine_for(folders[name, dtype], dtype, max_tokens=6 * 64, max_slots=4)
+    batches = [[(5, 8), (9, 3), (1, 12)], [(17, 12), (3, 1), (40, 6), (1, 9)], [(64, 2), (63, 3), (65, 1)]]
+    seed = 0
+    for batch in batches:
+        seed += 1
+        seqs = prompts_for(raw, [p + d for p, d in batch], seed=seed)
+        want = [oracle(name, dtype, s) for s in seqs]
+        slots = eng.open(len(batch))
+        got = [[] for _ in batch]
+        out = eng.step([Entry(slots[i], seqs[i][:p], list(range(p))) for i, (p, d) in enumerate(batch)]).cpu().numpy()
+        o = 0
+        for i, (p, d) in enumerate(batch):
+            got[i].append(out[o:o + p])
+            o += p
+        step = 0
+        live = list(range(len(batch)))
+        while live:
+            live = [i for i in live if step < batch[i][1]]
+            for i in range(len(batch)):
+                if i not in live and slots[i] is not None and step >= batch[i][1]:
+                    eng.close([slots[i]])
+                    slots[i] = None
+            if not live:
+                break
+            out = eng.step([Entry(slots[i], [seqs[i][batch[i][0] + step]], [0]) for i in live]).cpu().numpy()
+            for r, i in enumerate(live):
+                got[i].append(out[r:r + 1].copy())
+            step += 1
+        eng.cache.check_consistent()
+        assert eng.cache.n_free_slots == 4
+        for i in range(len(batch)):
+            g = np.concatenate(got[i])
+            assert g.shape == want[i].shape
+            assert rel_err(g, want[i]) <= TOL[dtype], (name, dtype, batch[i])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_step_cut_into_pieces_and_batch_mates(folders, oracle, dtype):
+    """A step with more rows than the workspace holds is cut along the rows; a request's logits do not
+    depend on that nor on what else is in the batch."""
+    from dlgo_amd.engine import Entry
+    raw = TINY_B
+    seqs = prompts_for(raw, [150, 33, 70], seed=9)
+    big = engine_for(folders["B", dtype], dtype, max_step_tokens=4096)
+    small = engine_for(folders["B", dtype], dtype, max_step_tokens=48)
+    outs = []
+    for eng in (big, small):
+        slots = eng.open(3)
+        outs.append(eng.step([Entry(s, t, list(range(len(t)))) for s, t in zip(slots, seqs)]).cpu().numpy())
+    tol = 1e-5 if dtype == "float32" else TOL[dtype]
+    assert rel_err(outs[1], outs[0].astype(np.float64)) <= tol
+    o = 0
+    for t in seqs:
+        assert rel_err(outs[0][o:o + len(t)], oracle("B", dtype, t)) <= TOL[dtype]
+        o += len(t)
+
+
+def test_errors_before_anything_runs(folders):
+    from dlgo_amd.engine import EngineError, Entry
+    eng = engine_for(folders["A", "float32"], "float32", max_tokens=128)
+    (slot,) = eng.open(1)
+    with pytest.raises(EngineError, match="vocabulary"):
+        eng.step([Entry(slot, [1, 256], [0])])
+    with pytest.raises(EngineError, match="no tokens"):
+        eng.step([Entry(slot, [], [])])
+    with pytest.raises(EngineError, match="twice"):
+        eng.step([Entry(slot, [1], []), Entry(slot, [2], [])])
+    with pytest.raises(EngineError, match="context"):
+        eng.step([Entry(slot, [1] * 129, [])])
+    with pytest.raises(EngineError, match="place"):
+        eng.step([Entry(slot, [1, 2], [2])])
+    with pytest.raises(EngineError):
+        eng.step([Entry(99, [1], [])])
+    assert eng.length(slot) == 0
+    eng.step([Entry(slot, [1, 2, 3], [])])
+    assert eng.length(slot) == 3

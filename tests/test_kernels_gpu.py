@@ -1,0 +1,386 @@
+"""Each kernel alone against a plain float64 reference of the same operation, at sizes
+other than the models' (tails, widths that are no power of two)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _ops():
+    from dlgo_amd.kernels import ops
+    return ops
+
+
+def close(got, want, rel, what=""):
+    got = got.double().cpu()
+    want = want.double().cpu()
+    scale = want.abs().max().item() + 1e-30
+    err = (got - want).abs().max().item()
+    assert err <= rel * scale, f"{what}: max error {err:.3e} against scale {scale:.3e} (allowed {rel:.1e} of it)"
+
+
+DT = [(torch.float32, 2e-6, 1e-5), (torch.bfloat16, 1.0, 1.2e-2)]   # dtype, -, relative tolerance
+
+
+@pytest.mark.parametrize("dtype,_,rel", DT)
+def test_embed(dtype, _, rel):
+    ops = _ops()
+    g = torch.Generator().manual_seed(1)
+    table = torch.randn(37, 24, generator=g).to(dtype).to(DEV)
+    ids = torch.tensor([0, 36, 5, 5, 17], dtype=torch.int32, device=DEV)
+    out = torch.empty(5, 24, dtype=torch.float32, device=DEV)
+    ops.embed(table, ids, out)
+    assert torch.equal(out.cpu(), table.float().cpu()[ids.cpu().long()])
+
+
+@pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("d", [4, 7, 96, 1024, 1500, 4096])
+def test_rmsnorm(dtype, _, rel, d):
+    ops = _ops()
+    g = torch.Generator().manual_seed(d)
+    x = (torch.randn(9, d, generator=g) * 3).to(DEV)
+    w = (1 + 0.3 * torch.randn(d, generator=g)).to(DEV)
+    eps = 1e-3
+    out = torch.empty(9, d, dtype=dtype, device=DEV)
+    ops.rmsnorm(x, w, eps, out)
+    xd = x.double()
+    want = xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + eps) * w.double()
+    close(out, want, rel, f"rmsnorm d={d}")
+    rows = torch.tensor([8, 0, 3], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(3, d, dtype=dtype, device=DEV)
+    ops.rmsnorm(x, w, eps, out2, rows)
+    assert torch.equal(out2, out[rows.long()])
+
+
+def test_rmsnorm_reference_vectors():
+    """The reference's own vectors (ops/norm_test.go:8-52)."""
+    ops = _ops()
+    x = torch.tensor([[1., 2., 3., 4.]], device=DEV)
+    out = torch.empty_like(x)
+    ops.rmsnorm(x, torch.ones(4, device=DEV), 1e-5, out)
+    close(out, x.double() / math.sqrt(7.5 + 1e-5), 1e-6)
+    ones = torch.ones(1, 4, device=DEV)
+    w = torch.tensor([2., 3., 4., 5.], device=DEV)
+    ops.rmsnorm(ones, w, 1e-5, out)
+    close(out, w.double()[None] / math.sqrt(1 + 1e-5), 1e-6)
+
+
+GEMM_SHAPES = [(200, 37, 96), (130, 5, 40), (64, 1, 64), (388, 130, 352), (34, 8, 160), (512, 257, 128), (6, 3, 8)]
+
+
+@pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("n,t,k", GEMM_SHAPES)
+def test_gemm_store_and_accumulate(dtype, _, rel, kind, n, t, k):
+    ops = _ops()
+    if kind == 1 and t > 8:
+        pytest.skip("the streaming kernel takes at most 8 rows")
+    if dtype == torch.bfloat16 and k % 8:
+        pytest.skip("bfloat16 rows come in 16-byte pieces")
+    g = torch.Generator().manual_seed(n * 1000 + t)
+    w = torch.randn(n, k, generator=g).to(dtype).to(DEV)
+    x = torch.randn(t, k, generator=g).to(dtype).to(DEV)
+    want = x.double() @ w.double().T
+    out = torch.empty(t, n, dtype=dtype, device=DEV)
+    ops.gemm(w, x, out, ops.EPI_STORE, kind)
+    close(out, want, rel, f"gemm store kind={kind}")
+    out32 = torch.empty(t, n, dtype=torch.float32, device=DEV)
+    ops.gemm(w, x, out32, ops.EPI_STORE_F32, kind)
+    close(out32, want, 1e-5 if dtype == torch.float32 else 1e-5, f"gemm store f32 kind={kind}")
+    res = torch.randn(t, n, generator=g).to(DEV)
+    res0 = res.clone()
+    ops.gemm(w, x, res, ops.EPI_ACCUM_F32, kind)
+    close(res, res0.double() + want, 1e-5, f"gemm accumulate kind={kind}")
+
+
+@pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("f,t,k", [(160, 5, 64), (352, 70, 128), (9, 2, 16), (1030, 200, 72)])
+def test_gemm_swiglu(dtype, _, rel, kind, f, t, k):
+    ops = _ops()
+    if kind == 1 and t > 8:
+        pytest.skip("the streaming kernel takes at most 8 rows")
+    g = torch.Generator().manual_seed(f + t)
+    gate = torch.randn(f, k, generator=g).to(dtype)
+    up = torch.randn(f, k, generator=g).to(dtype)
+    x = (torch.randn(t, k, generator=g) * 0.5).to(dtype).to(DEV)
+    w = torch.stack([gate, up], dim=1).reshape(2 * f, k).contiguous().to(DEV)
+    out = torch.empty(t, f, dtype=dtype, device=DEV)
+    ops.gemm(w, x, out, ops.EPI_SWIGLU, kind)
+    gd, ud = x.double().cpu() @ gate.double().T, x.double().cpu() @ up.double().T
+    want = gd / (1 + torch.exp(-gd)) * ud
+    close(out, want, rel, f"swiglu kind={kind}")
+
+
+def test_gemm_reference_vectors():
+    """blas/blas_test.go:21-64: identity, [[1,2],[3,4]]·[1,1] = [3,7], batch layout out[p*rows + r]."""
+    ops = _ops()
+    w = torch.zeros(4, 4, device=DEV)
+    w[:2, :2] = torch.tensor([[1., 2.], [3., 4.]])
+    x = torch.zeros(2, 4, device=DEV)
+    x[0, :2] = 1.0
+    x[1, 0] = 2.0
+    out = torch.empty(2, 4, device=DEV)
+    for kind in (1, 4):
+        ops.gemm(w, x, out, ops.EPI_STORE, kind)
+        assert out.cpu()[:, :2].tolist() == [[3.0, 7.0], [2.0, 6.0]]
+
+
+def test_gemm_refuses_what_it_cannot_do():
+    ops = _ops()
+    w = torch.zeros(8, 6, device=DEV)
+    x = torch.zeros(2, 6, device=DEV)
+    with pytest.raises(ops.KernelError, match="multiple of 4"):
+        ops.gemm(w, x, torch.empty(2, 8, device=DEV))
+    with pytest.raises(ops.KernelError):
+        ops.gemm(torch.zeros(8, 8, device=DEV), torch.zeros(2, 8, device=DEV), torch.empty(2, 9, device=DEV))
+
+
+# ---------------------------------------------------------------------------
+# rotation + cache write, attention over the paged cache
+# ---------------------------------------------------------------------------
+def _paged_setup(dtype, n_seq_lens, kv_heads, hd, n_units=2, unit=1, seed=0, shuffle=True):
+    """A page pool with pages handed out in a scrambled order, poisoned with NaN where nothing was written."""
+    from dlgo_amd.cache import PAGE
+    g = torch.Generator().manual_seed(seed)
+    pages_per = [(n + PAGE - 1) // PAGE for n in n_seq_lens]
+    n_pages = sum(pages_per) + 3
+    order = torch.randperm(n_pages, generator=g).tolist() if shuffle else list(range(n_pages))
+    max_pages = max(pages_per) + 1
+    table = torch.full((len(n_seq_lens) + 2, max_pages), -1, dtype=torch.int32)
+    it = iter(order)
+    slots = list(range(len(n_seq_lens), 0, -1))      # not the identity
+    for slot, npg in zip(slots, pages_per):
+        for j in range(npg):
+            table[slot, j] = next(it)
+    unit_elems = 2 * kv_heads * PAGE * hd
+    page_stride = unit_elems * n_units
+    storage = torch.full((n_pages * page_stride,), float("nan"), dtype=dtype)
+    return table, slots, storage, page_stride, unit * unit_elems, kv_heads * PAGE * hd
+
+
+def _rope_ref(v, pos, freqs, interleaved):
+    half = len(freqs)
+    ang = pos * freqs
+    c, s = np.cos(ang), np.sin(ang)
+    out = v.copy()
+    if interleaved:
+        x0, x1 = v[..., 0:2 * half:2], v[..., 1:2 * half:2]
+        out[..., 0:2 * half:2] = x0 * c - x1 * s
+        out[..., 1:2 * half:2] = x0 * s + x1 * c
+    else:
+        x0, x1 = v[..., :half], v[..., half:2 * half]
+        out[..., :half] = x0 * c - x1 * s
+        out[..., half:2 * half] = x0 * s + x1 * c
+    return out
+
+
+@pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("H,KV,hd,rot,inter", [(4, 2, 16, 16, False), (6, 3, 48, 48, True), (8, 1, 128, 64, False),
+                                               (2, 2, 32, 32, True)])
+def test_rope_kv_write(dtype, _, rel, H, KV, hd, rot, inter):
+    ops = _ops()
+    from dlgo_amd.cache import PAGE
+    from dlgo_amd.parts import rotary_frequencies
+    lens = [70, 3, 129]
+    starts = [5, 0, 64]                      # the rows continue sequences that already hold tokens
+    q_lens = [l - s for l, s in zip(lens, starts)]
+    table, slots, storage, page_stride, unit_off, v_off = _paged_setup(dtype, lens, KV, hd)
+    T = sum(q_lens)
+    g = torch.Generator().manual_seed(3)
+    qkv = torch.randn(T, (H + 2 * KV) * hd, generator=g).to(dtype)
+    positions = torch.tensor([p for s, n in zip(starts, q_lens) for p in range(s, s + n)], dtype=torch.int32)
+    tok_seq = torch.tensor([i for i, n in enumerate(q_lens) for _ in range(n)], dtype=torch.int32)
+    freqs = rotary_frequencies(rot, 10000.0)
+    ang = np.arange(200)[:, None] * freqs[None]
+    cos, sin = torch.from_numpy(np.cos(ang).astype(np.float32)), torch.from_numpy(np.sin(ang).astype(np.float32))
+    dq = qkv.clone().to(DEV)
+    store = storage.clone().to(DEV)
+    ops.rope_kv(dq, H, KV, hd, rot, inter, cos.to(DEV), sin.to(DEV), positions.to(DEV), tok_seq.to(DEV),
+                torch.tensor(slots, dtype=torch.int32, device=DEV), table.to(DEV), store[unit_off:], page_stride, v_off)
+    dq, store = dq.cpu(), store.cpu()
+    src = qkv.double().numpy().reshape(T, H + 2 * KV, hd)
+    for t in range(T):
+        pos = int(positions[t])
+        want_q = _rope_ref(src[t, :H], pos, freqs, inter)
+        close(dq[t, :H * hd].reshape(H, hd), torch.from_numpy(want_q), rel, "rotated q")
+        page = int(table[slots[int(tok_seq[t])], pos // PAGE])
+        base = page * page_stride + unit_off
+        kpage = store[base: base + KV * PAGE * hd].reshape(KV, PAGE, hd)
+        vpage = store[base + v_off: base + v_off + KV * hd * PAGE].reshape(KV, hd, PAGE)
+        close(kpage[:, pos % PAGE], torch.from_numpy(_rope_ref(src[t, H:H + KV], pos, freqs, inter)), rel, "stored k")
+        assert torch.equal(vpage[:, :, pos % PAGE], qkv[t].reshape(H + 2 * KV, hd)[H + KV:]), "stored v"
+    # nothing else was written: the other unit of each page and unused rows are still NaN
+    written = (~torch.isnan(store.float())).sum().item()
+    assert written == T * 2 * KV * hd
+
+
+def _attention_ref(q, k, v, H, KV, hd, pos_of_q, lo_of_q):
+    """q [n, H*hd]; k, v [len, KV*hd] for one sequence; row i attends keys lo..pos."""
+    g = H // KV
+    out = np.zeros_like(q)
+    for i in range(q.shape[0]):
+        for h in range(H):
+            kvh = h // g
+            ks = k[lo_of_q[i]:pos_of_q[i] + 1, kvh * hd:(kvh + 1) * hd]
+            vs = v[lo_of_q[i]:pos_of_q[i] + 1, kvh * hd:(kvh + 1) * hd]
+            s = ks @ q[i, h * hd:(h + 1) * hd] / math.sqrt(hd)
+            p = np.exp(s - s.max())
+            p /= p.sum()
+            out[i, h * hd:(h + 1) * hd] = p @ vs
+    return out
+
+
+def _fill_cache(storage, table, slot, k, v, KV, hd, page_stride, unit_off, v_off):
+    from dlgo_amd.cache import PAGE
+    for pos in range(k.shape[0]):
+        page = int(table[slot, pos // PAGE])
+        base = page * page_stride + unit_off
+        for kvh in range(KV):
+            o = base + (kvh * PAGE + pos % PAGE) * hd
+            storage[o:o + hd] = k[pos, kvh * hd:(kvh + 1) * hd]
+            ov = base + v_off + kvh * hd * PAGE + pos % PAGE
+            storage[ov: ov + hd * PAGE: PAGE] = v[pos, kvh * hd:(kvh + 1) * hd]
+
+
+ATT_CASES = [  # H, KV, hd, window, [(cached length, rows of this step)]
+    (4, 2, 16, 0, [(70, 70), (3, 1), (129, 5)]),
+    (6, 3, 48, 0, [(200, 200), (65, 1)]),
+    (4, 1, 32, 0, [(1, 1), (64, 64), (300, 1), (130, 66)]),
+    (8, 8, 64, 0, [(150, 150)]),
+    (4, 2, 16, 20, [(100, 100), (90, 1)]),
+    (2, 1, 128, 70, [(260, 3), (260, 260)]),
+]
+
+
+@pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("H,KV,hd,window,seqs", ATT_CASES)
+@pytest.mark.parametrize("kernel", ["rows", "auto"])
+def test_attention_over_pages(dtype, _, rel, H, KV, hd, window, seqs, kernel):
+    ops = _ops()
+    lens = [l for l, _ in seqs]
+    table, slots, storage, page_stride, unit_off, v_off = _paged_setup(dtype, lens, KV, hd, seed=hd)
+    g = torch.Generator().manual_seed(H * 100 + hd)
+    qs, pos, tok_seq, want = [], [], [], []
+    for i, (length, rows) in enumerate(seqs):
+        k = (torch.randn(length, KV * hd, generator=g) * 1.5).to(dtype)
+        v = torch.randn(length, KV * hd, generator=g).to(dtype)
+        q = (torch.randn(rows, H * hd, generator=g) * 1.5).to(dtype)
+        _fill_cache(storage, table, slots[i], k, v, KV, hd, page_stride, unit_off, v_off)
+        p = list(range(length - rows, length))
+        lo = [max(0, x - window + 1) if window else 0 for x in p]
+        want.append(_attention_ref(q.double().numpy(), k.double().numpy(), v.double().numpy(), H, KV, hd, p, lo))
+        qs.append(q)
+        pos += p
+        tok_seq += [i] * rows
+    q = torch.cat(qs).to(DEV)
+    out = torch.full((q.shape[0], H * hd), float("nan"), dtype=dtype, device=DEV)
+    args = (q, out, H, KV, hd, torch.tensor(pos, dtype=torch.int32, device=DEV),
+            torch.tensor(tok_seq, dtype=torch.int32, device=DEV), torch.tensor(slots, dtype=torch.int32, device=DEV),
+            table.to(DEV), storage.to(DEV)[unit_off:], page_stride, v_off)
+    if kernel == "rows":
+        ops.attention_rows(*args, window=window)
+    else:
+        q_lens = [r for _, r in seqs]
+        starts = [l - r for l, r in seqs]
+        ops.attention(*args, q_lens=q_lens, start_pos=starts, window=window)
+    close(out, torch.from_numpy(np.concatenate(want)), rel if dtype == torch.float32 else 2e-2, "attention")
+
+
+def test_attention_reference_vectors():
+    """layers/gqa_test.go: one cached position gives V for every head of the group (:8-43);
+    equal keys give the plain mean, with a window of 2 at position 3 of v = 0,1,2,3 that is 2.5 (:110-136)."""
+    ops = _ops()
+    H, KV, hd = 4, 2, 16
+    table, slots, storage, page_stride, unit_off, v_off = _paged_setup(torch.float32, [1, 4], KV, hd)
+    v0 = torch.arange(KV * hd, dtype=torch.float32)[None]
+    _fill_cache(storage, table, slots[0], torch.randn(1, KV * hd), v0, KV, hd, page_stride, unit_off, v_off)
+    kk = torch.ones(4, KV * hd)
+    vv = torch.arange(4, dtype=torch.float32)[:, None].repeat(1, KV * hd)
+    _fill_cache(storage, table, slots[1], kk, vv, KV, hd, page_stride, unit_off, v_off)
+    q = torch.randn(2, H * hd).to(DEV)
+    out = torch.empty(2, H * hd, device=DEV)
+    ops.attention_rows(q, out, H, KV, hd, torch.tensor([0, 3], dtype=torch.int32, device=DEV),
+                       torch.tensor([0, 1], dtype=torch.int32, device=DEV), torch.tensor(slots, dtype=torch.int32, device=DEV),
+                       table.to(DEV), storage.to(DEV)[unit_off:], page_stride, v_off, window=2)
+    got = out.cpu()
+    assert torch.equal(got[0].reshape(H, hd), v0.reshape(KV, hd).repeat_interleave(2, 0))
+    assert torch.allclose(got[1], torch.full((H * hd,), 2.5), atol=1e-6)
+
+
+# ---------------------------------------------------------------------------
+# sampling
+# ---------------------------------------------------------------------------
+def test_argmax_first_maximum():
+    ops = _ops()
+    x = torch.zeros(3, 70001, device=DEV)
+    x[0, 5] = 2.0
+    x[0, 69000] = 2.0
+    x[1, 70000] = 1.0
+    x[2, :] = -1.0
+    out = torch.empty(3, dtype=torch.int32, device=DEV)
+    ops.argmax(x, out)
+    assert out.tolist() == [5, 70000, 0]
+    v = torch.tensor([[1., 5., 2., 3.]], device=DEV)            # ops/sampling_test.go:9-16
+    ops.argmax(v, out[:1])
+    assert out[:1].tolist() == [1]
+
+
+def _sample(logits, temp, top_k=0, top_p=1.0, min_p=0.0, pen=1.0, recent=None, u=0.5):
+    ops = _ops()
+    n, v = logits.shape
+    lg = logits.float().to(DEV)
+    f = lambda val: torch.full((n,), val, dtype=torch.float32, device=DEV)
+    rec = None
+    if recent is not None:
+        rec = torch.tensor(recent, dtype=torch.int32, device=DEV)
+    uu = torch.tensor(u if isinstance(u, list) else [u] * n, dtype=torch.float32, device=DEV)
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    ops.sample(lg, torch.empty(n, v, device=DEV), torch.empty(n, v, device=DEV), f(temp),
+               torch.full((n,), top_k, dtype=torch.int32, device=DEV), f(top_p), f(min_p), f(pen), rec, uu, out)
+    return out.tolist()
+
+
+@pytest.mark.parametrize("v", [11, 384, 5000, 128256])
+def test_sample_matches_plain(v):
+    import plain_llama as plain
+    g = torch.Generator().manual_seed(v)
+    logits = torch.randn(6, v, generator=g) * 2.0
+    us = [0.03, 0.37, 0.5, 0.81, 0.999, 0.61]
+    cases = [dict(temp=0.8), dict(temp=1.0, top_k=5), dict(temp=0.7, top_p=0.6), dict(temp=1.3, min_p=0.2),
+             dict(temp=0.9, top_k=40, top_p=0.9, pen=1.1), dict(temp=0.0)]
+    recent = [[int(logits[i].argmax()), 3, 3, -1] for i in range(6)]
+    for c in cases:
+        got = _sample(logits, c.get("temp"), c.get("top_k", 0), c.get("top_p", 1.0), c.get("min_p", 0.0), c.get("pen", 1.0),
+                      recent, us)
+        for i in range(6):
+            want = plain.sample_token(logits[i].double().numpy(), us[i], c["temp"], c.get("top_k", 0), c.get("top_p", 1.0),
+                                      c.get("min_p", 0.0), c.get("pen", 1.0), [t for t in recent[i] if t >= 0])
+            assert got[i] == want, (c, i)
+
+
+def test_sample_reference_behaviour():
+    """ops/sampling_test.go: a dominant logit is always drawn (:18-30); temperature 2 halves the logits (:48-57)."""
+    logits = torch.zeros(1, 50)
+    logits[0, 17] = 100.0
+    for u in (1e-6, 0.3, 0.999):
+        assert _sample(logits, 1.0, u=u) == [17]
+    lg = torch.tensor([[2., 4., 6.]])          # temperature 2 -> [1,2,3]: p = softmax([1,2,3])
+    p = torch.softmax(torch.tensor([1., 2., 3.]), 0).cumsum(0)
+    assert _sample(lg, 2.0, u=float(p[0]) - 1e-3) == [0]
+    assert _sample(lg, 2.0, u=float(p[0]) + 1e-3) == [1]
+    assert _sample(lg, 2.0, u=float(p[1]) + 1e-3) == [2]
+    # top-k 2 on [1,4,2,5,3] keeps ids 1 and 3 (:59-70)
+    lg = torch.tensor([[1., 4., 2., 5., 3.]])
+    seen = {_sample(lg, 1.0, top_k=2, u=u / 20)[0] for u in range(20)}
+    assert seen == {1, 3}
+    # penalty 2 on [2,-1,3,0] for ids {0,1} -> [1,-2,3,0] (:32-46): id 0 drops below id 2 by more
+    lg = torch.tensor([[2., -1., 3., 0.]])
+    p = torch.softmax(torch.tensor([1., -2., 3., 0.]), 0)
+    assert _sample(lg, 1.0, pen=2.0, recent=[[0, 1]], u=float(p[0]) - 1e-3) == [0]
+    assert _sample(lg, 1.0, pen=2.0, recent=[[0, 1]], u=float(p[0] + p[1]) + 1e-3) == [2]
