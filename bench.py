@@ -1,0 +1,170 @@
+#!/usr/bin/env python3
+"""Decode and prefill throughput of the Llama 3.2 1B shape on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--dtype bf16|fp32]
+
+A step is one decode step of the whole batch: the step function on one token per
+sequence, greedy choice of the next tokens on the device, and their return to the
+host (what the generation loop does per step).  Random weights, seeded
+uniform-random token ids, no stop tokens.  Prints ONE JSON line.
+
+Peaks used for the fractions (MI355X, published): HBM 8 TB/s; dense MFMA bf16
+2.5 PFLOP/s, fp32 157.3 TFLOP/s.
+"""
+import argparse
+import json
+import statistics
+import sys
+import time
+
+# The benchmark's model: Llama 3.2 1B as config.json states it.
+LLAMA_1B = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "vocab_size": 128256, "hidden_size": 2048, "num_hidden_layers": 16, "intermediate_size": 8192,
+    "num_attention_heads": 32, "num_key_value_heads": 8, "head_dim": 64,
+    "rms_norm_eps": 1e-5, "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                     "original_max_position_embeddings": 8192},
+    "max_position_embeddings": 131072, "tie_word_embeddings": True, "initializer_range": 0.02,
+    "hidden_act": "silu", "torch_dtype": "bfloat16", "bos_token_id": 128000, "eos_token_id": 128001,
+}
+CONTEXT = 4096
+PROMPT = 2048
+HBM_PEAK = 8.0e12
+FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def weight_bytes(cfg, elem):
+    """Bytes a decode step must read of the weights: every matrix once (the tied table serves as the head)."""
+    d, f = cfg.hidden_size, cfg.intermediate_size
+    per_layer = (cfg.q_dim + 2 * cfg.kv_dim) * d + d * cfg.q_dim + 3 * d * f
+    head = cfg.vocab_size * d
+    norms = (2 * cfg.num_hidden_layers + 1) * d * 4
+    return (cfg.num_hidden_layers * per_layer + head) * elem + norms
+
+
+def kv_bytes_per_token(cfg, elem):
+    return cfg.num_hidden_layers * 2 * cfg.kv_dim * elem
+
+
+def prefill_flops(cfg, t):
+    d, f = cfg.hidden_size, cfg.intermediate_size
+    per_layer = (cfg.q_dim + 2 * cfg.kv_dim) * d + d * cfg.q_dim + 3 * d * f
+    linear = 2.0 * t * per_layer * cfg.num_hidden_layers
+    attn = cfg.num_hidden_layers * cfg.num_attention_heads * 2.0 * 2.0 * cfg.head_dim * t * (t + 1) / 2.0   # QK^T and PV, causal
+    head = 2.0 * cfg.vocab_size * d
+    return linear + attn + head
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the model has (0 = all)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--points", default="1,64", help="other batch sizes to report, comma separated ('' = none)")
+    ap.add_argument("--point-steps", type=int, default=64)
+    ap.add_argument("--no-prefill", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import numpy as np
+    import torch
+
+    from dlgo_amd import models  # noqa: F401
+    from dlgo_amd.config import config_from_dict
+    from dlgo_amd.engine import Engine, Entry
+    from dlgo_amd.sampling import Sampler, SamplerConfig
+
+    raw = dict(LLAMA_1B)
+    full_layers = raw["num_hidden_layers"]
+    if args.layers:
+        raw["num_hidden_layers"] = args.layers
+    cfg = config_from_dict(raw)
+    elem = 2 if args.dtype == "bf16" else 4
+    batches = [args.batch] + [int(b) for b in args.points.split(",") if b.strip()]
+    most = max(batches)
+    per_seq = PROMPT + args.warmup + max(args.steps, args.point_steps) + 64
+    assert per_seq <= CONTEXT
+    eng = Engine.from_random(cfg, seed=0, dtype=args.dtype, max_tokens=most * ((per_seq + 63) // 64 * 64), max_ctx=CONTEXT,
+                             max_step_tokens=8192, graph_max_batch=max(most, 8))
+    sampler = Sampler(eng.vocab, eng.device, max_rows=most)
+    rng = np.random.default_rng(0)
+    greedy = SamplerConfig(temperature=0.0)
+
+    def decode(batch, steps, warmup):
+        prompts = [rng.integers(0, cfg.vocab_size, size=PROMPT).tolist() for _ in range(batch)]
+        slots = eng.open(batch)
+        logits = eng.step([Entry(s, p, [PROMPT - 1]) for s, p in zip(slots, prompts)])
+        toks = sampler.choose(logits, [greedy] * batch, [0.0] * batch)
+
+        def one():
+            nonlocal toks
+            lg = eng.step([Entry(s, [t], [0]) for s, t in zip(slots, toks)])
+            toks = sampler.choose(lg, [greedy] * batch, [0.0] * batch)
+        for _ in range(warmup):
+            one()
+        torch.cuda.synchronize()
+        c0 = eng.length(slots[0])
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            one()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        eng.close(slots)
+        mean_ctx = c0 + (steps + 1) / 2.0       # keys a step reads per sequence, averaged over the timed steps
+        return dt, mean_ctx
+
+    dt, mean_ctx = decode(args.batch, args.steps, args.warmup)
+    ms_step = dt / args.steps * 1000.0
+    value = args.batch * args.steps / dt
+    step_bytes = weight_bytes(cfg, elem) + args.batch * mean_ctx * kv_bytes_per_token(cfg, elem)
+    achieved = step_bytes / (dt / args.steps)
+    points = {}
+    for b in batches[1:]:
+        pdt, _ = decode(b, args.point_steps, min(args.warmup, 8))
+        points[f"decode_b{b}"] = round(b * args.point_steps / pdt, 1)
+
+    prefill = None
+    if not args.no_prefill:
+        times = []
+        for i in range(6):
+            prompt = rng.integers(0, cfg.vocab_size, size=PROMPT).tolist()
+            (slot,) = eng.open(1)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            eng.step([Entry(slot, prompt, [PROMPT - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            eng.close([slot])
+        pt = statistics.median(times[1:])
+        prefill = {"value": round(PROMPT / pt, 1), "tokens": PROMPT, "ms": round(pt * 1000.0, 3),
+                   "frac": round(prefill_flops(cfg, PROMPT) / pt / FLOP_PEAK[args.dtype], 4)}
+
+    line = {
+        "metric": f"decode tok/s @ batch {args.batch} (Llama 3.2 1B shape, {PROMPT}-token prompts, context {CONTEXT})",
+        "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
+        "config": {"model": "llama-3.2-1b-shape", "layers": cfg.num_hidden_layers, "layers_of_model": full_layers,
+                   "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+                   "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+                   "tied_embeddings": cfg.tie_word_embeddings, "global_batch": args.batch, "seq_len": CONTEXT,
+                   "prompt_len": PROMPT, "parallelism": "single-gpu", "kv_cache_dtype": args.dtype,
+                   "sampling": "greedy on device, tokens returned to the host each step"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4)},
+        "points": points,
+    }
+    if prefill is not None:
+        line["prefill"] = prefill
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -276,7 +276,7 @@ class Engine:
     def _static_arrays(self) -> Dict[str, torch.Tensor]:
         if self._static is None:
             b = self.graph_max_batch
-            meta = torch.zeros(4 * b + 8, dtype=torch.int32, device=self.device)
+            meta = torch.zeros(8 * b + 64, dtype=torch.int32, device=self.device)
             self._static = {"meta": meta}
             self._static_logits = torch.empty((b, self.vocab), dtype=torch.float32, device=self.device)
         return self._static

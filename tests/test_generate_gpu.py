@@ -1,0 +1,181 @@
+"""Generation through the entry point, the command line and the replay program, on the GPU."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import plain_llama as plain
+from conftest import ROOT, TINY_A, TINY_B, make_folder
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def folder_a(tmp_path_factory):
+    return make_folder(TINY_A, 21, tmp_path_factory.mktemp("gen_a"), dtype="float32", std=0.1)
+
+
+@pytest.fixture(scope="module")
+def folder_b(tmp_path_factory):
+    return make_folder(TINY_B, 22, tmp_path_factory.mktemp("gen_b"), dtype="float32", std=0.08, norm_jitter=0.1)
+
+
+def _prompts(raw, lens, seed):
+    rng = np.random.default_rng(seed)
+    return [rng.integers(0, raw["vocab_size"], size=n).tolist() for n in lens]
+
+
+def test_greedy_matches_plain_in_unequal_batches(folder_a):
+    """Tiny A's workload: prompts of 5, 9 and 1 tokens, 8 tokens each, then more requests than fit at once."""
+    import dlgo_amd
+    cfg, w = plain.read_model(folder_a)
+    llm = dlgo_amd.load_llm(folder_a, dtype="float32", max_tokens=512, max_batch=3)
+    prompts = _prompts(TINY_A, [5, 9, 1, 12, 3, 30, 2], seed=1)
+    streamed = []
+    results = llm.generate(prompts, dlgo_amd.with_greedy(), dlgo_amd.with_max_tokens(8), dlgo_amd.with_ignore_eos())
+    for p, r in zip(prompts, results):
+        assert r.tokens == plain.greedy_generate(cfg, w, p, 8)
+        assert r.finish_reason == "length"
+    llm.engine.cache.check_consistent()
+    assert llm.engine.free_slots() == llm.engine.cache.max_slots
+    r = llm.generate_stream(prompts[0], streamed.append, dlgo_amd.with_greedy(), dlgo_amd.with_max_tokens(8),
+                            dlgo_amd.with_ignore_eos())
+    assert streamed == r.tokens == results[0].tokens          # one call per token, same tokens alone as in a batch
+
+
+def test_stop_tokens_end_sequences_early(folder_a):
+    import dlgo_amd
+    cfg, w = plain.read_model(folder_a)
+    llm = dlgo_amd.load_llm(folder_a, dtype="float32", max_tokens=512)
+    prompts = _prompts(TINY_A, [4, 7, 2], seed=2)
+    free = [plain.greedy_generate(cfg, w, p, 10) for p in prompts]
+    stop = free[1][3]
+    results = llm.generate(prompts, dlgo_amd.with_greedy(), dlgo_amd.with_max_tokens(10), dlgo_amd.with_stop_tokens([stop]))
+    for p, r in zip(prompts, results):
+        want = plain.greedy_generate(cfg, w, p, 10, stop_tokens=(stop,))
+        assert r.tokens == want
+        assert r.finish_reason == ("stop" if len(want) < 10 else "length")
+    assert results[1].finish_reason == "stop" and stop not in results[1].tokens
+
+
+def test_temperature_sampling_is_reproducible_and_matches_plain(folder_b):
+    """Tiny B's workload: prompts 17, 3, 40, 1; 12 tokens at temperature 0.8 with a fixed seed, beside a greedy run."""
+    import dlgo_amd
+    from dlgo_amd.sampling import uniform
+    cfg, w = plain.read_model(folder_b)
+    llm = dlgo_amd.load_llm(folder_b, dtype="float32", max_tokens=1024)
+    prompts = _prompts(TINY_B, [17, 3, 40, 1], seed=3)
+    opts = [dlgo_amd.with_temperature(0.8), dlgo_amd.with_top_k(0), dlgo_amd.with_top_p(1.0), dlgo_amd.with_repetition_penalty(1.0),
+            dlgo_amd.with_seed(1234), dlgo_amd.with_max_tokens(12), dlgo_amd.with_ignore_eos()]
+    a = llm.generate(prompts, *opts)
+    b = llm.generate(prompts, *opts)
+    assert [r.tokens for r in a] == [r.tokens for r in b]
+    alone = llm.generate([prompts[2]], *opts)
+    # a request's draws are keyed by its index in the call, so alone (index 0) it draws differently from index 2
+    assert len(alone[0].tokens) == 12
+    for i, (p, r) in enumerate(zip(prompts, a)):
+        seq, want = list(p), []
+        for step in range(12):
+            tok = plain.sample_token(plain.forward(cfg, w, seq)[-1], uniform(1234, i, step), 0.8)
+            want.append(tok)
+            seq.append(tok)
+        assert r.tokens == want, i
+    g = llm.generate(prompts, dlgo_amd.with_greedy(), dlgo_amd.with_max_tokens(12), dlgo_amd.with_ignore_eos())
+    for p, r in zip(prompts, g):
+        assert r.tokens == plain.greedy_generate(cfg, w, p, 12)
+    # dlgo's default sampler (temperature 0.7, top-k 40, top-p 0.9, penalty 1.1) runs and respects the seed
+    d1 = llm.generate(prompts, dlgo_amd.with_seed(5), dlgo_amd.with_max_tokens(12))
+    d2 = llm.generate(prompts, dlgo_amd.with_seed(5), dlgo_amd.with_max_tokens(12))
+    assert [r.tokens for r in d1] == [r.tokens for r in d2]
+
+
+def test_long_decoding_and_context_end(folder_a):
+    """Decoding up to the end of the context: the last tokens still match, and the run ends with "context"."""
+    import dlgo_amd
+    cfg, w = plain.read_model(folder_a)
+    llm = dlgo_amd.load_llm(folder_a, dtype="float32", max_tokens=512)
+    prompt = _prompts(TINY_A, [3], seed=4)[0]
+    r = llm.generate(prompt, dlgo_amd.with_greedy(), dlgo_amd.with_max_tokens(500), dlgo_amd.with_ignore_eos())
+    assert r.finish_reason == "context"
+    assert len(prompt) + len(r.tokens) == TINY_A["max_position_embeddings"] - 1
+    assert r.tokens == plain.greedy_generate(cfg, w, prompt, len(r.tokens))
+    with pytest.raises(ValueError, match="prompt too long"):
+        llm.generate([1] * 128, dlgo_amd.with_greedy())
+
+
+def test_command_line(folder_a):
+    out = subprocess.run([sys.executable, "-m", "dlgo_amd", "--greedy", "--max-tokens", "4", "--dtype", "float32", "--ignore-eos",
+                          "--prompt-ids", "5,6,7", "--prompt-ids", "9", folder_a], cwd=ROOT, capture_output=True, text=True,
+                         timeout=300)
+    assert out.returncode == 0, out.stderr
+    cfg, w = plain.read_model(folder_a)
+    lines = [json.loads(l) for l in out.stdout.splitlines() if l.startswith("{")]
+    assert lines[0]["tokens"] == plain.greedy_generate(cfg, w, [5, 6, 7], 4)
+    assert lines[1]["tokens"] == plain.greedy_generate(cfg, w, [9], 4)
+    bad = subprocess.run([sys.executable, "-m", "dlgo_amd", "--temp", "-1", folder_a], cwd=ROOT, capture_output=True, text=True)
+    assert bad.returncode == 1 and "--temp must be >= 0" in bad.stderr
+
+
+def _replay(folder, dtype, steps, out_dir, max_tokens):
+    text = "".join(json.dumps(s) + "\n" for s in steps)
+    p = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", str(out_dir),
+                        "--max-tokens", str(max_tokens)], input=text, capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr
+    assert [l for l in p.stdout.splitlines() if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_replay(folder_b, tmp_path, dtype):
+    cfg, w = plain.read_model(folder_b)
+    V = TINY_B["vocab_size"]
+    seqs = dict(zip("abcd", _prompts(TINY_B, [70, 40, 9, 100], seed=6)))
+    want = {k: plain.forward(cfg, w, v) for k, v in seqs.items()}
+    tol = 2e-5 if dtype == "float32" else 3e-2
+    # whole
+    steps = [{"step": i, "entries": [{"id": k, "tokens": v, "want": list(range(len(v)))}], "end": [k]}
+             for i, (k, v) in enumerate(seqs.items())]
+    _replay(folder_b, dtype, steps, tmp_path / "whole", 128)
+    for i, k in enumerate(seqs):
+        got = np.fromfile(tmp_path / "whole" / f"{i}.f32", dtype="<f4").reshape(-1, V)
+        assert np.abs(got - want[k]).max() <= tol * np.abs(want[k]).max()
+    # the last 32 one by one
+    v = seqs["d"]
+    head = len(v) - 32
+    steps = [{"step": 0, "entries": [{"id": "d", "tokens": v[:head], "want": [0, head - 1]}], "end": []}]
+    steps += [{"step": 1 + i, "entries": [{"id": "d", "tokens": [t], "want": [0]}], "end": ["d"] if i == 31 else []}
+              for i, t in enumerate(v[head:])]
+    _replay(folder_b, dtype, steps, tmp_path / "tail", 128)
+    got = np.fromfile(tmp_path / "tail" / "0.f32", dtype="<f4").reshape(-1, V)
+    assert np.abs(got - want["d"][[0, head - 1]]).max() <= tol * np.abs(want["d"]).max()
+    for i in range(32):
+        got = np.fromfile(tmp_path / "tail" / f"{1 + i}.f32", dtype="<f4").reshape(-1, V)
+        assert np.abs(got[0] - want["d"][head + i]).max() <= tol * np.abs(want["d"]).max()
+    # a batch of unequal lengths whose shorter requests end earlier, then another in the same room
+    first = {"a": 60, "b": 35, "c": 1}
+    steps = [{"step": 0, "entries": [{"id": k, "tokens": seqs[k][:p], "want": [p - 1]} for k, p in first.items()], "end": []}]
+    n = 1
+    pos = dict(first)
+    while any(pos[k] < len(seqs[k]) for k in first):
+        live = [k for k in first if pos[k] < len(seqs[k])]
+        ends = [k for k in live if pos[k] + 1 == len(seqs[k])]
+        steps.append({"step": n, "entries": [{"id": k, "tokens": [seqs[k][pos[k]]], "want": [0]} for k in live], "end": ends})
+        for k in live:
+            pos[k] += 1
+        n += 1
+    steps.append({"step": n, "entries": [{"id": "d", "tokens": seqs["d"], "want": [99]}], "end": ["d"]})
+    _replay(folder_b, dtype, steps, tmp_path / "batch", 256)
+    got0 = np.fromfile(tmp_path / "batch" / "0.f32", dtype="<f4").reshape(-1, V)
+    for r, (k, p) in enumerate(first.items()):
+        assert np.abs(got0[r] - want[k][p - 1]).max() <= tol * np.abs(want[k]).max()
+    pos = dict(first)
+    for s in steps[1:-1]:
+        got = np.fromfile(tmp_path / "batch" / f"{s['step']}.f32", dtype="<f4").reshape(-1, V)
+        for r, e in enumerate(s["entries"]):
+            k = e["id"]
+            assert np.abs(got[r] - want[k][pos[k]]).max() <= tol * np.abs(want[k]).max(), (s["step"], k)
+            pos[k] += 1
+    got = np.fromfile(tmp_path / "batch" / f"{n}.f32", dtype="<f4").reshape(-1, V)
+    assert np.abs(got[0] - want["d"][99]).max() <= tol * np.abs(want["d"]).max()
