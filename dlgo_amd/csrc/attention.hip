@@ -16,8 +16,19 @@
 // HEAD_DIM is fixed at compile time (one library per head size).
 //
 // Kernels:
-//   attn_rows_kernel   any dtype; one wave per (token, query head), online
-//                      softmax page by page in float32.  The float32 path.
+//   attn_rows_kernel     any dtype; one wave per (token, query head), online
+//                        softmax page by page in float32.  The float32 path.
+//   attn_prefill_kernel  bfloat16; flash-style: a block takes 128 query rows
+//                        (tokens x the heads of one group) that share one KV head,
+//                        walks the pages of keys through LDS, and keeps scores
+//                        transposed (keys x rows) so that each lane owns one query
+//                        row: softmax statistics stay in the lane and the
+//                        probabilities feed the second MFMA without a shuffle.
+//   attn_decode_kernel   bfloat16; one token per sequence: a wave takes a few
+//                        pages of one (sequence, KV head), all heads of the group
+//                        at once as the MFMA's 16 columns, and writes a partial
+//                        (max, sum, weighted values); attn_combine_kernel merges
+//                        the partials in page order.
 #include "common.h"
 
 #ifndef HEAD_DIM
@@ -123,6 +134,364 @@ __global__ __launch_bounds__(WAVE) void attn_rows_kernel(const T* __restrict__ q
   }
 }
 
+
+// ----------------------------------------------------------------------------
+// bfloat16 MFMA kernels
+// ----------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+
+__device__ __forceinline__ bf16x8_t as_bf16x8(const uint4& u) {
+  union { uint4 u; bf16x8_t v; } x;
+  x.u = u;
+  return x.v;
+}
+__device__ __forceinline__ bf16x8_t join_bf16x8(const uint2& lo, const uint2& hi) {
+  union { uint2 u[2]; bf16x8_t v; } x;
+  x.u[0] = lo;
+  x.u[1] = hi;
+  return x.v;
+}
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+#define PF_THREADS 256
+#define PF_ROWS 128   // query rows (token x head of the group) per block
+
+// Prefill.  grid (q tiles, sequences, kv heads).  bq = tokens per block (bq * group <= 128).
+__global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
+    const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, const int32_t* __restrict__ cu_q,
+    const int32_t* __restrict__ start_pos, const int32_t* __restrict__ slots, const int32_t* __restrict__ page_table,
+    int max_pages, const bf16_t* __restrict__ cache, long long page_stride, long long v_off, int group, int bq, int window,
+    float scale_log2e) {
+  constexpr int HD = HEAD_DIM;
+  constexpr int KS = HD / 16;               // k steps of K Q^T (32x32x16)
+  constexpr int DT = (HD + 31) / 32;        // 32-row tiles of the output's head dimension
+  constexpr int KROW = HD * 2 + 16;         // bytes of a key row in LDS (padded)
+  constexpr int VROW = PAGE * 2 + 16;       // bytes of a row of transposed values in LDS
+  constexpr int KCH = PAGE * HD / 8;        // 16-byte chunks of a key tile
+  constexpr int VCH = HD * PAGE / 8;
+  constexpr int NKC = (KCH + PF_THREADS - 1) / PF_THREADS;
+  constexpr int NVC = (VCH + PF_THREADS - 1) / PF_THREADS;
+  __shared__ __attribute__((aligned(16))) char ldsK[PAGE * KROW];
+  __shared__ __attribute__((aligned(16))) char ldsV[DT * 32 * VROW];
+
+  const int seq = blockIdx.y, kvh = blockIdx.z;
+  const int q0 = cu_q[seq], qn = cu_q[seq + 1] - q0;
+  const int t0 = blockIdx.x * bq;
+  if (t0 >= qn) return;
+  const int t1 = t0 + bq < qn ? t0 + bq : qn;           // tokens [t0, t1) of the sequence's rows
+  const int start = start_pos[seq];
+  const int slot = slots[seq];
+  const int kv_len = start + qn;                          // keys the cache holds for this sequence now
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5;
+
+  // this lane's query row
+  const int r = wave * 32 + (lane & 31);
+  const int tok = t0 + r / group, hig = r % group;
+  const bool row_ok = tok < t1;
+  const int pos = row_ok ? start + tok : -1;
+  const int lo = (row_ok && window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  // the wave's rows span tokens [wt0, wt1]
+  const int wt0 = t0 + (wave * 32) / group;
+  int wt1 = t0 + (wave * 32 + 31) / group;
+  wt1 = wt1 < t1 - 1 ? wt1 : t1 - 1;
+  const bool wave_ok = wt0 < t1;
+  const int w_pos_min = start + wt0, w_pos_max = start + wt1;
+  const int w_lo_max = window > 0 && w_pos_max - window + 1 > 0 ? w_pos_max - window + 1 : 0;
+  const int w_lo_min = window > 0 && w_pos_min - window + 1 > 0 ? w_pos_min - window + 1 : 0;
+
+  uint4 qf[KS];
+  {
+    const bf16_t* qrow = q + (size_t)(q0 + (row_ok ? tok : t0)) * ldq + (size_t)(kvh * group + hig) * HD;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = row_ok ? *(const uint4*)(qrow + ks * 16 + half * 8) : make_uint4(0, 0, 0, 0);
+  }
+  f32x16_t o[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o[d][v] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  const int b_lo = window > 0 && start + t0 - window + 1 > 0 ? start + t0 - window + 1 : 0;
+  const int pg_lo = b_lo / PAGE, pg_hi = (start + t1 - 1) / PAGE;
+
+  uint4 rk[NKC], rv[NVC];
+  auto fetch = [&](int pg) {
+    const int page = page_table[(size_t)slot * max_pages + pg];
+    const bf16_t* kpage = cache + (size_t)(page < 0 ? 0 : page) * page_stride + (size_t)kvh * PAGE * HD;
+    const bf16_t* vpage = cache + v_off + (size_t)(page < 0 ? 0 : page) * page_stride + (size_t)kvh * HD * PAGE;
+#pragma unroll
+    for (int i = 0; i < NKC; ++i) {
+      const int c = tid + i * PF_THREADS;
+      rk[i] = c < KCH ? *(const uint4*)(kpage + (size_t)c * 8) : make_uint4(0, 0, 0, 0);
+    }
+    const bool tail = pg * PAGE + PAGE > kv_len;      // keys beyond the sequence: their values must not reach the product
+#pragma unroll
+    for (int i = 0; i < NVC; ++i) {
+      const int c = tid + i * PF_THREADS;
+      uint4 u = c < VCH ? *(const uint4*)(vpage + (size_t)c * 8) : make_uint4(0, 0, 0, 0);
+      if (tail) {
+        const int k0 = pg * PAGE + (c & 7) * 8;
+        uint32_t* w = (uint32_t*)&u;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (k0 + 2 * e >= kv_len) w[e] = 0;
+          else if (k0 + 2 * e + 1 >= kv_len) w[e] &= 0xffffu;
+        }
+      }
+      rv[i] = u;
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < NKC; ++i) {
+      const int c = tid + i * PF_THREADS;
+      if (c < KCH) *(uint4*)(ldsK + (c / (HD / 8)) * KROW + (c % (HD / 8)) * 16) = rk[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NVC; ++i) {
+      const int c = tid + i * PF_THREADS;
+      if (c < VCH) *(uint4*)(ldsV + (c >> 3) * VROW + (c & 7) * 16) = rv[i];
+    }
+  };
+
+  fetch(pg_lo);
+  for (int pg = pg_lo; pg <= pg_hi; ++pg) {
+    stash();
+    __syncthreads();
+    if (pg < pg_hi) fetch(pg + 1);
+    const int key0 = pg * PAGE;
+    if (wave_ok && key0 <= w_pos_max && key0 + PAGE - 1 >= w_lo_min) {
+      f32x16_t s[2];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[kt][v] = 0.f;
+        const char* pk = ldsK + (kt * 32 + (lane & 31)) * KROW + half * 16;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(*(const uint4*)(pk + ks * 32)), as_bf16x8(qf[ks]), s[kt], 0, 0, 0);
+      }
+      // lane: row = lane%32; element v of tile kt is key  key0 + 32 kt + 8 (v/4) + 4 half + v%4
+      const bool need_mask = key0 + PAGE - 1 > w_pos_min || key0 < w_lo_max;
+      float mx = -INFINITY;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          float sv = s[kt][v] * scale_log2e;
+          if (need_mask) {
+            const int key = key0 + kt * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+            sv = (key <= pos && key >= lo) ? sv : -INFINITY;
+          }
+          s[kt][v] = sv;
+          mx = fmaxf(mx, sv);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+      const float m_new = fmaxf(m, mx);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = fast_exp2(m - m_use);
+      float rs = 0.f;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const float p = fast_exp2(s[kt][v] - m_use);
+          s[kt][v] = p;
+          rs += p;
+        }
+      rs += __shfl_xor(rs, 32, WAVE);
+      l = l * alpha + rs;
+      m = m_new;
+#pragma unroll
+      for (int d = 0; d < DT; ++d)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[d][v] *= alpha;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          bf16x8_t pb;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) pb[e] = (__bf16)s[kt][8 * u + e];
+          // element e of this operand is key 32 kt + 16 u + 8 (e/4) + 4 half + e%4: the values follow the same order
+          const char* pv = ldsV + (lane & 31) * VROW + (kt * 32 + 16 * u + 4 * half) * 2;
+#pragma unroll
+          for (int d = 0; d < DT; ++d) {
+            const uint2 lo8 = *(const uint2*)(pv + d * 32 * VROW);
+            const uint2 hi8 = *(const uint2*)(pv + d * 32 * VROW + 16);
+            o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(join_bf16x8(lo8, hi8), pb, o[d], 0, 0, 0);
+          }
+        }
+    }
+    __syncthreads();
+  }
+  if (!row_ok) return;
+  const float inv = 1.0f / l;
+  bf16_t* orow = out + (size_t)(q0 + tok) * ldo + (size_t)(kvh * group + hig) * HD;
+#pragma unroll
+  for (int d = 0; d < DT; ++d)
+#pragma unroll
+    for (int qd = 0; qd < 4; ++qd) {
+      const int dd = d * 32 + 8 * qd + 4 * half;
+      if (dd < HD) {
+        uint2 pk;
+        pk.x = (uint32_t)f32_to_bf16(o[d][4 * qd] * inv) | ((uint32_t)f32_to_bf16(o[d][4 * qd + 1] * inv) << 16);
+        pk.y = (uint32_t)f32_to_bf16(o[d][4 * qd + 2] * inv) | ((uint32_t)f32_to_bf16(o[d][4 * qd + 3] * inv) << 16);
+        *(uint2*)(orow + dd) = pk;
+      }
+    }
+}
+
+// Decode: one token per sequence.  grid (splits, kv heads x head blocks of 16, sequences), one wave per block.
+// A wave takes pages [split * ppw, (split+1) * ppw) of its sequence and writes one partial per head:
+// part[((seq * H + head) * n_splits + split) * (HD + 4)] = weighted values [HD], max, sum (base-2 exponents), 2 unused.
+__global__ __launch_bounds__(WAVE) void attn_decode_kernel(
+    const bf16_t* __restrict__ q, int ldq, float* __restrict__ part, const int32_t* __restrict__ positions,
+    const int32_t* __restrict__ slots, const int32_t* __restrict__ page_table, int max_pages,
+    const bf16_t* __restrict__ cache, long long page_stride, long long v_off, int n_heads, int group, int head_blocks, int ppw,
+    int n_splits, int window, float scale_log2e) {
+  constexpr int HD = HEAD_DIM;
+  constexpr int KS = (HD + 31) / 32;   // k steps of K Q^T (16x16x32)
+  constexpr int DT = HD / 16;          // 16-row tiles of the output's head dimension
+  const int split = blockIdx.x, seq = blockIdx.z;
+  const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
+  const int pos = positions[seq];
+  const int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+  int pg0 = split * ppw, pg1 = pg0 + ppw - 1;
+  if (pg0 < lo / PAGE) pg0 = lo / PAGE;
+  if (pg1 > pos / PAGE) pg1 = pos / PAGE;
+  if (pg0 > pg1) return;
+  const int slot = slots[seq];
+  const int lane = threadIdx.x, j = lane & 15, G = lane >> 4;
+  const int hig = hb * 16 + j;                    // head within the group
+  const bool head_ok = hig < group;
+  const int head = kvh * group + hig;
+
+  uint4 qf[KS];
+  {
+    const bf16_t* qrow = q + (size_t)seq * ldq + (size_t)(head_ok ? head : kvh * group) * HD;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      qf[ks] = (head_ok && ks * 32 + G * 8 < HD) ? *(const uint4*)(qrow + ks * 32 + G * 8) : make_uint4(0, 0, 0, 0);
+  }
+  f32x4_t o[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d) o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  for (int pg = pg0; pg <= pg1; ++pg) {
+    const int page = page_table[(size_t)slot * max_pages + pg];
+    if (page < 0) continue;
+    const bf16_t* kpage = cache + (size_t)page * page_stride + (size_t)kvh * PAGE * HD;
+    const bf16_t* vpage = cache + v_off + (size_t)page * page_stride + (size_t)kvh * HD * PAGE;
+    const int key0 = pg * PAGE;
+    f32x4_t s[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      s[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      const bf16_t* krow = kpage + (size_t)(t * 16 + j) * HD + G * 8;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const uint4 a = (ks * 32 + G * 8 < HD) ? *(const uint4*)(krow + ks * 32) : make_uint4(0, 0, 0, 0);
+        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(qf[ks]), s[t], 0, 0, 0);
+      }
+    }
+    // lane: head = lane%16; element v of tile t is key  key0 + 16 t + 4 G + v
+    const bool need_mask = key0 + PAGE - 1 > pos || key0 < lo;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        float sv = s[t][v] * scale_log2e;
+        if (need_mask) {
+          const int key = key0 + 16 * t + 4 * G + v;
+          sv = (key <= pos && key >= lo) ? sv : -INFINITY;
+        }
+        s[t][v] = sv;
+        mx = fmaxf(mx, sv);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = fmaxf(m, mx);      // finite: every page of the range holds a valid key
+    const float alpha = fast_exp2(m - m_new);
+    float rs = 0.f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const float p = fast_exp2(s[t][v] - m_new);
+        s[t][v] = p;
+        rs += p;
+      }
+    rs += __shfl_xor(rs, 16, WAVE);
+    rs += __shfl_xor(rs, 32, WAVE);
+    l = l * alpha + rs;
+    m = m_new;
+#pragma unroll
+    for (int d = 0; d < DT; ++d) o[d] *= alpha;
+    const bool tail = key0 + PAGE - 1 > pos;   // keys beyond the sequence: their values must not reach the product
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {              // 32 keys each: tiles 2u and 2u+1
+      bf16x8_t pb;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        pb[e] = (__bf16)s[2 * u][e];
+        pb[4 + e] = (__bf16)s[2 * u + 1][e];
+      }
+      const int ka = 32 * u + 4 * G, kb = ka + 16;      // first keys (within the page) of the two 4-key pieces
+#pragma unroll
+      for (int d = 0; d < DT; ++d) {
+        const bf16_t* vrow = vpage + (size_t)(d * 16 + j) * PAGE;
+        uint2 a0 = *(const uint2*)(vrow + ka), a1 = *(const uint2*)(vrow + kb);
+        if (tail) {
+          uint32_t* w0 = (uint32_t*)&a0;
+          uint32_t* w1 = (uint32_t*)&a1;
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            if (key0 + ka + 2 * e > pos) w0[e] = 0;
+            else if (key0 + ka + 2 * e + 1 > pos) w0[e] &= 0xffffu;
+            if (key0 + kb + 2 * e > pos) w1[e] = 0;
+            else if (key0 + kb + 2 * e + 1 > pos) w1[e] &= 0xffffu;
+          }
+        }
+        o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(join_bf16x8(a0, a1), pb, o[d], 0, 0, 0);
+      }
+    }
+  }
+  if (!head_ok) return;
+  float* dst = part + ((size_t)(seq * n_heads + head) * n_splits + split) * (HD + 4);
+#pragma unroll
+  for (int d = 0; d < DT; ++d) *(float4*)(dst + d * 16 + 4 * G) = make_float4(o[d][0], o[d][1], o[d][2], o[d][3]);
+  if (G == 0) {
+    dst[HD] = m;
+    dst[HD + 1] = l;
+  }
+}
+
+// grid (sequences, heads); merges the partials of the splits that hold keys of the token, in page order.
+__global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, int ldo,
+                                                            const int32_t* __restrict__ positions, int n_heads, int ppw,
+                                                            int n_splits, int window) {
+  constexpr int HD = HEAD_DIM;
+  const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int pos = positions[seq];
+  const int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+  const int s0 = (lo / PAGE) / ppw, s1 = (pos / PAGE) / ppw;
+  const float* base = part + (size_t)(seq * n_heads + head) * n_splits * (HD + 4);
+  float M = -INFINITY;
+  for (int s = s0; s <= s1; ++s) M = fmaxf(M, base[(size_t)s * (HD + 4) + HD]);
+  float L = 0.f;
+  for (int s = s0; s <= s1; ++s) L += fast_exp2(base[(size_t)s * (HD + 4) + HD] - M) * base[(size_t)s * (HD + 4) + HD + 1];
+  const float inv = 1.0f / L;
+  for (int d = lane; d < HD; d += WAVE) {
+    float acc = 0.f;
+    for (int s = s0; s <= s1; ++s) acc += fast_exp2(base[(size_t)s * (HD + 4) + HD] - M) * base[(size_t)s * (HD + 4) + d];
+    out[(size_t)seq * ldo + (size_t)head * HD + d] = f32_to_bf16(acc * inv);
+  }
+}
+
 extern "C" int dlgo_attention_head_dim() { return HEAD_DIM; }
 
 // q: rows of the step [T, >= H*hd] (rotated); out [T, >= H*hd]; positions, tok_seq per token; slots per sequence.
@@ -149,5 +518,61 @@ extern "C" const char* dlgo_attention_rows(const void* q, int ldq, void* out, in
   else
     DLGO_FAIL("attention: unknown dtype code %d", dtype);
   DLGO_LAUNCH_CHECK("attention_rows");
+  return nullptr;
+}
+
+#define LOG2E 1.4426950408889634f
+
+// bfloat16, every sequence's rows of this step: cu_q [n_seq+1], start_pos [n_seq] (length before the step), slots [n_seq].
+extern "C" const char* dlgo_attention_prefill(const void* q, int ldq, void* out, int ldo, int n_seq, int max_q_len, int n_heads,
+                                              int n_kv, int head_dim, const int32_t* cu_q, const int32_t* start_pos,
+                                              const int32_t* slots, const int32_t* page_table, int max_pages, const void* cache,
+                                              long long page_stride, long long v_off, int window, float scale,
+                                              hipStream_t stream) {
+  DLGO_REQUIRE(head_dim == HEAD_DIM, "attention: this library is built for head size %d, got %d", HEAD_DIM, head_dim);
+  DLGO_REQUIRE(HEAD_DIM <= 256, "attention: the tiled kernel takes head sizes up to 256");
+  DLGO_REQUIRE(n_seq >= 0 && max_q_len >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention: bad sizes");
+  const int group = n_heads / n_kv;
+  DLGO_REQUIRE(group <= PF_ROWS, "attention: the tiled kernel takes up to %d query heads per kv head, got %d", PF_ROWS, group);
+  DLGO_REQUIRE(ldq >= n_heads * head_dim && ldo >= n_heads * head_dim && ldq % 8 == 0 && ldo % 4 == 0, "attention: row strides");
+  DLGO_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)out & 7) == 0 && ((uintptr_t)cache & 15) == 0 && page_stride % 8 == 0 && v_off % 8 == 0,
+               "attention: operands must be 16-byte aligned");
+  DLGO_REQUIRE(window >= 0 && max_pages > 0, "attention: bad window or page table width");
+  if (n_seq == 0 || max_q_len == 0) return nullptr;
+  const int bq = PF_ROWS / group;
+  dim3 grid((max_q_len + bq - 1) / bq, n_seq, n_kv);
+  hipLaunchKernelGGL(attn_prefill_kernel, grid, dim3(PF_THREADS), 0, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo, cu_q,
+                     start_pos, slots, page_table, max_pages, (const bf16_t*)cache, page_stride, v_off, group, bq, window,
+                     scale * LOG2E);
+  DLGO_LAUNCH_CHECK("attention_prefill");
+  return nullptr;
+}
+
+// bfloat16, one row per sequence.  part: float32 scratch of n_seq * n_heads * n_splits * (hd + 4), n_splits =
+// ceil(max_pages_used / pages_per_wave), where max_pages_used bounds the pages of any sequence of the step.
+extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, int ldo, float* part, long long part_elems,
+                                             int n_seq, int n_heads, int n_kv, int head_dim, const int32_t* positions,
+                                             const int32_t* slots, const int32_t* page_table, int max_pages,
+                                             int max_pages_used, int pages_per_wave, const void* cache, long long page_stride,
+                                             long long v_off, int window, float scale, hipStream_t stream) {
+  DLGO_REQUIRE(head_dim == HEAD_DIM, "attention: this library is built for head size %d, got %d", HEAD_DIM, head_dim);
+  DLGO_REQUIRE(n_seq >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention: bad sizes");
+  DLGO_REQUIRE(pages_per_wave >= 1 && max_pages_used >= 1 && max_pages_used <= max_pages, "attention: bad split of the pages");
+  DLGO_REQUIRE(ldq >= n_heads * head_dim && ldo >= n_heads * head_dim && ldq % 8 == 0, "attention: row strides");
+  DLGO_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)part & 15) == 0 && ((uintptr_t)cache & 15) == 0 && page_stride % 8 == 0 && v_off % 8 == 0,
+               "attention: operands must be 16-byte aligned");
+  const int group = n_heads / n_kv;
+  const int head_blocks = (group + 15) / 16;
+  const int n_splits = (max_pages_used + pages_per_wave - 1) / pages_per_wave;
+  DLGO_REQUIRE(part_elems >= (long long)n_seq * n_heads * n_splits * (HEAD_DIM + 4), "attention: scratch for partial results too small");
+  DLGO_REQUIRE((long long)n_kv * head_blocks <= 65535 && n_seq <= 65535 && n_heads <= 65535, "attention: grid too large");
+  if (n_seq == 0) return nullptr;
+  hipLaunchKernelGGL(attn_decode_kernel, dim3(n_splits, n_kv * head_blocks, n_seq), dim3(WAVE), 0, stream, (const bf16_t*)q, ldq, part,
+                     positions, slots, page_table, max_pages, (const bf16_t*)cache, page_stride, v_off, n_heads, group, head_blocks,
+                     pages_per_wave, n_splits, window, scale * LOG2E);
+  DLGO_LAUNCH_CHECK("attention_decode");
+  hipLaunchKernelGGL(attn_combine_kernel, dim3(n_seq, n_heads), dim3(WAVE), 0, stream, part, (bf16_t*)out, ldo, positions, n_heads,
+                     pages_per_wave, n_splits, window);
+  DLGO_LAUNCH_CHECK("attention_combine");
   return nullptr;
 }

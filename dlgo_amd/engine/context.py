@@ -17,6 +17,7 @@ class Workspace:
         self.device = device
         self.max_rows = max_rows
         self._bufs: Dict[Tuple[str, int, torch.dtype], torch.Tensor] = {}
+        self._retired: List[torch.Tensor] = []
 
     def get(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
         rows, cols = int(shape[0]), int(np.prod(shape[1:], dtype=np.int64)) if len(shape) > 1 else 1
@@ -28,6 +29,18 @@ class Workspace:
             buf = torch.empty((self.max_rows, cols), dtype=dtype, device=self.device)
             self._bufs[key] = buf
         return buf[:rows].view(rows, *shape[1:]) if len(shape) > 1 else buf[:rows, 0]
+
+    def flat(self, name: str, n: int, dtype: torch.dtype) -> torch.Tensor:
+        """A flat scratch buffer of at least n elements.  When a larger one is needed the old one is kept
+        alive, because a captured step may still point at it."""
+        key = ("flat:" + name, 0, dtype)
+        buf = self._bufs.get(key)
+        if buf is None or buf.numel() < n:
+            if buf is not None:
+                self._retired.append(buf)
+            buf = torch.empty(n, dtype=dtype, device=self.device)
+            self._bufs[key] = buf
+        return buf
 
     def bytes(self) -> int:
         return sum(b.numel() * b.element_size() for b in self._bufs.values())
@@ -61,5 +74,11 @@ class StepContext:
         self.is_decode = bool(n_seq) and self.max_q_len == 1
         self.max_kv_len = int((host["start_pos"] + q_lens).max()) if n_seq else 0
 
+        #: pages any sequence of this step may hold (a captured step must allow for the whole context)
+        self.max_pages_used: Optional[int] = None
+
     def buffer(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
         return self.engine.workspace.get(name, shape, dtype)
+
+    def scratch(self, name: str, n: int, dtype: torch.dtype) -> torch.Tensor:
+        return self.engine.workspace.flat(name, n, dtype)

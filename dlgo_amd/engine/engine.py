@@ -16,6 +16,7 @@ tokens is captured once per batch size as a HIP graph and replayed.
 """
 from __future__ import annotations
 
+import gc
 from dataclasses import dataclass, field
 from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
@@ -313,6 +314,7 @@ class Engine:
                     "slots": np.asarray(slots, dtype=np.int64)}
             ctx = StepContext(self, b, b, arrays, host)
             ctx.is_decode = True
+            ctx.max_pages_used = self.cache.max_pages_per_seq     # the recorded launch must cover any later length
             x = self.model.hidden(ctx, ctx.token_ids)
             self.model.logits(ctx, x, None, logits)
             # the second time a batch size is seen it is worth capturing
@@ -329,7 +331,16 @@ class Engine:
         each replay."""
         graph = torch.cuda.CUDAGraph()
         torch.cuda.synchronize()
-        with torch.cuda.graph(graph):
-            x = self.model.hidden(ctx, ctx.token_ids)
-            self.model.logits(ctx, x, None, logits)
+        # No garbage collection while recording: a collected tensor or event would make calls into the
+        # runtime that a recording stream forbids, and the error is raised inside a destructor.
+        gc.collect()
+        was_enabled = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(graph):
+                x = self.model.hidden(ctx, ctx.token_ids)
+                self.model.logits(ctx, x, None, logits)
+        finally:
+            if was_enabled:
+                gc.enable()
         self._graphs[b] = _Graph(graph, b, ctx)

@@ -146,6 +146,14 @@ def ensure_built(variants: Iterable[Variant], force: bool = False, quiet: bool =
                     os.remove(tmp)
             else:
                 os.replace(tmp, final)
+                stem = os.path.basename(final).rsplit("-", 1)[0] + "-"
+                for other in os.listdir(out_dir):     # builds of older sources of the same variant
+                    if other.startswith(stem) and other.endswith(".so") and other != os.path.basename(final) \
+                            and len(other) == len(os.path.basename(final)):
+                        try:
+                            os.remove(os.path.join(out_dir, other))
+                        except OSError:
+                            pass
                 if not quiet:
                     _say(f"built {os.path.basename(final)} ({time.time() - t0:.0f}s)")
                 last_note = time.time()
@@ -187,7 +195,7 @@ def loaded_libraries() -> Sequence[str]:
 
 
 #: head sizes compiled ahead by build_all(): those of the test configurations and of the benchmark shapes
-DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 128)
+DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128)
 
 
 def all_variants(head_dims: Sequence[int] = DEFAULT_HEAD_DIMS) -> list[Variant]:

@@ -196,11 +196,80 @@ def attention_rows(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, 
 def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, positions: torch.Tensor,
               tok_seq: torch.Tensor, slots: torch.Tensor, page_table: torch.Tensor, cache: torch.Tensor, page_stride: int,
               v_off: int, q_lens: Sequence[int], start_pos: Sequence[int], window: int = 0,
-              scale: Optional[float] = None) -> torch.Tensor:
-    """Attention of a step's query rows over the cache, with the kernel chosen by the step's shape
-    (q_lens, start_pos: per sequence, on the host).  All kernels compute the same thing."""
-    return attention_rows(q, out, n_heads, n_kv, head_dim, positions, tok_seq, slots, page_table, cache, page_stride,
-                          v_off, window, scale)
+              scale: Optional[float] = None, cu_q: Optional[torch.Tensor] = None,
+              start_pos_dev: Optional[torch.Tensor] = None, scratch=None, max_pages_used: Optional[int] = None,
+              kernel: str = "auto") -> torch.Tensor:
+    """Attention of a step's query rows over the cache, with the kernel chosen by the step's shape and dtype.
+
+    q_lens, start_pos: per sequence, on the host (rows of the step, and the length before it).  cu_q and
+    start_pos_dev are the same numbers on the device (built here if not given).  scratch(n) returns a
+    float32 buffer of at least n elements (decode partials).  max_pages_used bounds the pages any sequence
+    of the step holds (default: from q_lens and start_pos; a captured step passes the context's bound).
+    kernel: "auto", "rows", "tiled" (prefill) or "split" (decode).  All kernels compute the same thing.
+    """
+    n_seq = len(q_lens)
+    max_q = int(max(q_lens)) if n_seq else 0
+    group = n_heads // n_kv
+    fast_ok = q.dtype == torch.bfloat16 and head_dim <= 256 and group <= 128
+    if kernel == "auto":
+        kernel = "rows" if not fast_ok else ("split" if max_q == 1 else "tiled")
+    if kernel == "rows" or n_seq == 0:
+        return attention_rows(q, out, n_heads, n_kv, head_dim, positions, tok_seq, slots, page_table, cache, page_stride,
+                              v_off, window, scale)
+    if not fast_ok:
+        raise KernelError("attention: the tiled and split kernels take bfloat16, head sizes up to 256 and up to 128 heads per kv head")
+    _need(q, "query rows", torch.bfloat16, 2)
+    _need(out, "attention output", torch.bfloat16, 2)
+    _need(slots, "slots", torch.int32, 1)
+    _need(page_table, "page table", torch.int32, 2)
+    _need(cache, "cache", torch.bfloat16)
+    if slots.shape[0] != n_seq or out.shape[0] != q.shape[0] or q.shape[0] != int(sum(q_lens)) or not page_table.is_contiguous():
+        raise KernelError("attention: rows, sequences and slots do not match")
+    if scale is None:
+        scale = 1.0 / math.sqrt(head_dim)
+    lib = _lib("attention", (("HEAD_DIM", head_dim),))
+    if kernel == "split":
+        if max_q != 1:
+            raise KernelError("attention: the split kernel takes one row per sequence")
+        _need(positions, "positions", torch.int32, 1)
+        if positions.shape[0] != n_seq:
+            raise KernelError("attention: one position per sequence")
+        max_pages = page_table.shape[1]
+        if max_pages_used is None:
+            max_pages_used = (int(max(start_pos)) + 1 + PAGE - 1) // PAGE
+        max_pages_used = max(1, min(max_pages_used, max_pages))
+        ppw = decode_pages_per_wave(n_seq * n_kv * ((group + 15) // 16), max_pages_used)
+        n_splits = (max_pages_used + ppw - 1) // ppw
+        need = n_seq * n_heads * n_splits * (head_dim + 4)
+        part = scratch(need) if scratch is not None else torch.empty(need, dtype=torch.float32, device=q.device)
+        _need(part, "attention scratch", torch.float32, 1)
+        _check(lib.dlgo_attention_decode(_ptr(q), _rows(q, "query rows"), _ptr(out), _rows(out, "attention output"), _ptr(part),
+                                         ctypes.c_longlong(part.numel()), n_seq, n_heads, n_kv, head_dim, _ptr(positions),
+                                         _ptr(slots), _ptr(page_table), max_pages, max_pages_used, ppw, _ptr(cache),
+                                         ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(window),
+                                         ctypes.c_float(scale), _stream()))
+        return out
+    if kernel != "tiled":
+        raise KernelError(f"attention: unknown kernel {kernel!r}")
+    if cu_q is None:
+        import numpy as np
+        cu = np.concatenate([[0], np.cumsum(np.asarray(q_lens, dtype=np.int64))]).astype(np.int32)
+        cu_q = torch.from_numpy(cu).to(q.device)
+        start_pos_dev = torch.as_tensor(list(start_pos), dtype=torch.int32).to(q.device)
+    _need(cu_q, "row offsets", torch.int32, 1)
+    _need(start_pos_dev, "start positions", torch.int32, 1)
+    if cu_q.shape[0] != n_seq + 1 or start_pos_dev.shape[0] != n_seq:
+        raise KernelError("attention: row offsets and start positions do not match the sequences")
+    _check(lib.dlgo_attention_prefill(_ptr(q), _rows(q, "query rows"), _ptr(out), _rows(out, "attention output"), n_seq, max_q,
+                                      n_heads, n_kv, head_dim, _ptr(cu_q), _ptr(start_pos_dev), _ptr(slots), _ptr(page_table),
+                                      page_table.shape[1], _ptr(cache), ctypes.c_longlong(page_stride),
+                                      ctypes.c_longlong(v_off), int(window), ctypes.c_float(scale), _stream()))
+    return out
+
+
+def decode_pages_per_wave(n_pairs: int, max_pages: int) -> int:
+    """Pages of keys one wave of the split kernel takes: enough waves to fill the chip, few enough partials."""
+    return max(1, min(8, (n_pairs * max_pages) // 2048))
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

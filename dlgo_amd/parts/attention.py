@@ -104,4 +104,6 @@ class Attention(Mixer):
         step's shape and the run dtype, the arithmetic is the same."""
         ops.attention(q, out, self.n_heads, self.n_kv_heads, self.head_dim, ctx.positions, ctx.tok_seq, ctx.slots,
                       kv.page_table, kv.cache, kv.page_stride, kv.v_off, ctx.host["q_lens"], ctx.host["start_pos"],
-                      window=self.window or 0, scale=self.scale)
+                      window=self.window or 0, scale=self.scale, cu_q=ctx.cu_q, start_pos_dev=ctx.start_pos,
+                      scratch=lambda n: ctx.scratch("attention.partials", n, torch.float32),
+                      max_pages_used=ctx.max_pages_used)

@@ -255,6 +255,16 @@ ATT_CASES = [  # H, KV, hd, window, [(cached length, rows of this step)]
     (8, 8, 64, 0, [(150, 150)]),
     (4, 2, 16, 20, [(100, 100), (90, 1)]),
     (2, 1, 128, 70, [(260, 3), (260, 260)]),
+    # one row per sequence (the split kernel in bfloat16)
+    (4, 2, 16, 0, [(70, 1), (3, 1), (129, 1), (64, 1), (65, 1)]),
+    (32, 8, 64, 0, [(700, 1), (1, 1), (333, 1)]),
+    (40, 2, 32, 0, [(200, 1), (77, 1)]),
+    (6, 2, 48, 50, [(300, 1), (20, 1), (128, 1)]),
+    (8, 8, 128, 0, [(150, 1)]),
+    # groups that do not divide a tile
+    (6, 2, 48, 0, [(100, 100), (31, 7)]),
+    (40, 2, 32, 0, [(90, 90)]),
+    (4, 4, 80, 0, [(130, 130), (5, 5)]),
 ]
 
 
