@@ -49,6 +49,11 @@ def run_dtype(name) -> torch.dtype:
         raise EngineError(f"unknown dtype {name!r}: bfloat16 or float32") from None
 
 
+def _require_gpu() -> None:
+    if not torch.cuda.is_available():
+        raise EngineError("no HIP device: dlgo_amd runs on an AMD GPU only and has no CPU path")
+
+
 @dataclass
 class Entry:
     """One sequence's part of a step: its slot, its next tokens, and the places among
@@ -70,8 +75,7 @@ class Engine:
                  max_slots: Optional[int] = None, max_step_tokens: int = 8192, logits_rows: int = 1024,
                  use_graphs: bool = True, graph_max_batch: int = 128):
         """`model` holds its weights already (see from_folder / from_random)."""
-        if not torch.cuda.is_available():
-            raise EngineError("no HIP device: dlgo_amd runs on an AMD GPU only and has no CPU path")
+        _require_gpu()
         self.model = model
         self.dtype = run_dtype(dtype)
         self.device = torch.device(device)
@@ -102,6 +106,7 @@ class Engine:
     # -- construction ------------------------------------------------------------
     @classmethod
     def from_folder(cls, folder: str, dtype="bfloat16", device="cuda:0", **kw) -> "Engine":
+        _require_gpu()
         config = load_config(folder)
         model = build_model(config)
         load_weights(model, folder, device, run_dtype(dtype))
@@ -111,6 +116,7 @@ class Engine:
     def from_random(cls, config: ModelConfig, seed: int, dtype="bfloat16", device="cuda:0", std: Optional[float] = None,
                     norm_jitter: float = 0.0, **kw) -> "Engine":
         """Random weights drawn on the device and never written (benchmarks)."""
+        _require_gpu()
         model = build_model(config)
         rd = run_dtype(dtype)
         tensors = random_tensors(config, seed, rd, std, norm_jitter, device=device)

@@ -29,13 +29,14 @@ class LayerRun:
 class DecoderModel:
     def __init__(self, config, embedding: Tuple[str, Embedding], layers: Sequence[Tuple[str, Block]],
                  final_norm: Tuple[str, Part], head: Tuple[str, OutputHead], order: Optional[Sequence[LayerRun]] = None,
-                 position: Optional[PositionEncoding] = None, ignorable_tensors: Sequence[str] = ()):
+                 position: Optional[Tuple[str, PositionEncoding]] = None, ignorable_tensors: Sequence[str] = ()):
         self.config = config
         self.embedding_name, self.embedding = embedding
         self.layers = list(layers)
         self.final_norm_name, self.final_norm = final_norm
         self.head_name, self.head = head
-        self.position = position            # asked for its on_embedding hook; may be None
+        # a position encoding that acts on the embedded rows (its on_embedding hook), mounted under its own name
+        self.position_name, self.position = position if position is not None else (None, None)
         self.order: List[LayerRun] = list(order) if order is not None else [LayerRun(i) for i in range(len(self.layers))]
         self.ignorable_tensors = set(ignorable_tensors)
         self.vocab = self.embedding.vocab
@@ -61,6 +62,8 @@ class DecoderModel:
     # -- tensors ---------------------------------------------------------------
     def named_parts(self) -> Iterator[Tuple[str, Part]]:
         yield self.embedding_name, self.embedding
+        if self.position is not None:
+            yield self.position_name, self.position
         for prefix, block in self.layers:
             for name, part in block.parts():
                 yield f"{prefix}.{name}", part

@@ -1,0 +1,316 @@
+"""The cache's bookkeeping (no slot or page lost, held twice or freed twice) and the generation
+loop's decisions, with stand-ins for the engine and the sampler; no GPU."""
+import random
+
+import numpy as np
+import pytest
+import torch
+
+from dlgo_amd.cache import PAGE, Cache, CacheError, OutOfPages, PagePool
+from dlgo_amd.engine.generate import GenerationError, generate, plan_batch
+from dlgo_amd.parts import CacheNeed
+from dlgo_amd.sampling import GenerateConfig, SamplerConfig, apply_options, uniform, with_greedy, with_max_tokens, \
+    with_seed, with_temperature, with_top_k, with_top_p
+
+KV = [CacheNeed(kind="kv", kv_heads=2, head_dim=16)]
+
+
+def make_cache(n_units=2, max_tokens=8 * PAGE, max_ctx=4 * PAGE, needs=None, **kw):
+    return Cache([needs or KV for _ in range(n_units)], max_tokens, max_ctx, torch.float32, "cpu", **kw)
+
+
+def test_page_pool():
+    pool = PagePool(4)
+    a = pool.take(3)
+    assert sorted(a) == [0, 1, 2] and pool.n_free == 1
+    with pytest.raises(OutOfPages):
+        pool.take(2)
+    pool.give(a[:1])
+    with pytest.raises(CacheError):
+        pool.give(a[:1])              # freed twice
+    with pytest.raises(CacheError):
+        pool.give([7])                # not a page of this pool
+    assert pool.n_free == 2
+
+
+def test_slots_and_pages_round_trip():
+    c = make_cache()
+    assert c.n_pages == 8 and c.max_pages_per_seq == 4 and len(c.groups) == 1      # both units share one group
+    g = c.groups[0]
+    assert g.page_stride == 2 * g.unit_elems and g.storage.numel() == 8 * g.page_stride
+    a, b = c.alloc_slot(), c.alloc_slot()
+    c.reserve([(a, 70), (b, 1)])
+    assert len(c.held_pages(a)) == 2 and len(c.held_pages(b)) == 1 and g.pool.n_free == 5
+    c.advance(a, 70)
+    c.advance(b, 1)
+    assert c.length(a) == 70
+    c.reserve([(a, 71), (b, 2)])                          # nothing new needed
+    assert g.pool.n_free == 5
+    c.reserve([(a, 129)])
+    assert len(c.held_pages(a)) == 3
+    assert (g.table_host[a, :3] >= 0).all() and g.table_host[a, 3] == -1
+    c.check_consistent()
+    c.free_slot(a)
+    assert g.pool.n_free == 7 and (g.table_host[a] == -1).all()
+    with pytest.raises(CacheError):
+        c.free_slot(a)                                    # freed twice
+    with pytest.raises(CacheError):
+        c.length(a)
+    c.sync_tables()
+    assert torch.equal(g.table, torch.from_numpy(g.table_host))
+    a2 = c.alloc_slot()
+    assert a2 == a and c.length(a2) == 0                  # the slot is used again, empty
+    c.check_consistent()
+
+
+def test_limits_are_errors_before_anything_changes():
+    c = make_cache(max_tokens=3 * PAGE, max_ctx=2 * PAGE)
+    s = [c.alloc_slot() for _ in range(3)]
+    with pytest.raises(CacheError, match="no free slot"):
+        c.alloc_slot()
+    assert "context" in c.can_reserve([(s[0], 2 * PAGE + 1)])
+    c.reserve([(s[0], 2 * PAGE)])
+    before = c.groups[0].pool.n_free
+    with pytest.raises(OutOfPages):
+        c.reserve([(s[1], 1), (s[2], 65)])
+    assert c.groups[0].pool.n_free == before and not c.held_pages(s[1])
+    c.check_consistent()
+
+
+def test_groups_by_need_and_window_release():
+    needs = [[CacheNeed("kv", 2, 16)], [CacheNeed("kv", 2, 16, window=100)], [CacheNeed("kv", 1, 32)],
+             [CacheNeed("kv", 2, 16), CacheNeed("state", state_shape=(3, 4))], [CacheNeed("none")]]
+    c = Cache(needs, 64 * PAGE, 32 * PAGE, torch.float32, "cpu", max_slots=4, max_step_tokens=128)
+    assert len(c.groups) == 3
+    assert [c.unit_group.get(u) for u in range(5)] == [(0, 0), (1, 0), (2, 0), (0, 1), None]
+    windowed = c.groups[1]
+    assert windowed.pool.n_pages == 4 * ((100 + 128 + 63) // 64 + 1) < c.groups[0].pool.n_pages      # storage of its own, smaller
+    assert c.state_of(3).shape == (4, 3, 4)
+    s = c.alloc_slot()
+    total = 0
+    for step in [128, 128, 100, 1, 1, 64, 128]:
+        c.reserve([(s, total + step)])
+        c.advance(s, step)
+        total += step
+        held = c.held_pages(s, 1)
+        first_needed = max(0, total - 100 + 1) // PAGE
+        assert min(held) == first_needed and max(held) == (total - 1) // PAGE       # a window of pages, no more
+        assert len(c.held_pages(s, 0)) == (total + PAGE - 1) // PAGE                # the full group keeps everything
+        c.check_consistent()
+    kv = c.kv_view(1)
+    assert kv.window == 100 and kv.page_table is windowed.table
+    c.free_slot(s)
+    assert all(g.pool.n_free == g.pool.n_pages for g in c.groups)
+
+
+def test_state_is_zeroed_when_a_slot_is_handed_out():
+    c = Cache([[CacheNeed("state", state_shape=(5,), state_dtype=torch.float32)]], PAGE, PAGE, torch.float32, "cpu", max_slots=2)
+    s = c.alloc_slot()
+    c.state_of(0)[s] = 7.0
+    c.free_slot(s)
+    t = c.alloc_slot()
+    assert t == s and torch.equal(c.state_of(0)[t], torch.zeros(5))
+
+
+def test_random_traffic_keeps_the_books():
+    rng = random.Random(0)
+    c = make_cache(n_units=3, max_tokens=40 * PAGE, max_ctx=10 * PAGE, max_slots=6,
+                   needs=[CacheNeed("kv", 2, 16), ])
+    live = {}
+    for _ in range(600):
+        r = rng.random()
+        if r < 0.25 and c.n_free_slots:
+            live[c.alloc_slot()] = 0
+        elif r < 0.4 and live:
+            s = rng.choice(list(live))
+            c.free_slot(s)
+            del live[s]
+        elif live:
+            s = rng.choice(list(live))
+            n = rng.choice([1, 1, 1, 5, 64, 130])
+            if live[s] + n <= c.max_ctx and c.can_reserve([(s, live[s] + n)]) is None:
+                c.reserve([(s, live[s] + n)])
+                c.advance(s, n)
+                live[s] += n
+        c.check_consistent()
+        assert sorted(live) == c.live_slots()
+        assert all(c.length(s) == n for s, n in live.items())
+        held = sum((n + PAGE - 1) // PAGE for n in live.values())
+        assert c.groups[0].pool.n_free == 40 - held
+
+
+# -- the generation loop -------------------------------------------------------------
+class FakeEngine:
+    """Slots and pages like the real one; 'logits' are the (request, position) pairs the sampler decides on."""
+
+    def __init__(self, max_ctx=64, slots=3, pages=6):
+        self.max_ctx, self._slots, self._pages = max_ctx, slots, pages
+        self.free = list(range(slots))
+        self.held = {}
+        self.steps = []
+        self.closed = []
+
+    def free_slots(self):
+        return len(self.free)
+
+    def free_pages(self):
+        return self._pages - sum((n + PAGE - 1) // PAGE for n in self.held.values())
+
+    def open(self, n):
+        out = [self.free.pop(0) for _ in range(n)]
+        for s in out:
+            self.held[s] = 0
+        return out
+
+    def close(self, slots):
+        for s in slots:
+            assert s in self.held, "slot closed twice"
+            del self.held[s]
+            self.free.append(s)
+            self.closed.append(s)
+
+    def step(self, entries):
+        assert len({e.slot for e in entries}) == len(entries)
+        for e in entries:
+            assert e.slot in self.held
+            self.held[e.slot] += len(e.tokens)
+            assert self.held[e.slot] <= self.max_ctx
+        assert self.free_pages() >= 0
+        self.steps.append([(e.slot, list(e.tokens), list(e.want)) for e in entries])
+        return [(e.slot, self.held[e.slot]) for e in entries]
+
+
+class ScriptSampler:
+    """Token = 100 + length of the sequence so far, or a scripted stop."""
+
+    def __init__(self, stop_at=None):
+        self.stop_at = stop_at or {}
+        self.calls = []
+
+    def choose(self, logits, configs, uniforms, recent):
+        self.calls.append((list(logits), list(uniforms), [list(r) for r in recent]))
+        return [self.stop_at.get((slot, n), 100 + n) for slot, n in logits]
+
+
+def test_plan_batch():
+    assert plan_batch([5, 9, 1], [8, 8, 8], free_slots=3, free_pages=6, max_batch=64, max_ctx=4096) == 3
+    assert plan_batch([5, 9, 1], [8, 8, 8], free_slots=2, free_pages=6, max_batch=64, max_ctx=4096) == 2
+    assert plan_batch([60, 60, 60], [8, 8, 8], free_slots=3, free_pages=5, max_batch=64, max_ctx=4096) == 2
+    assert plan_batch([60, 60], [1000, 8], free_slots=3, free_pages=2, max_batch=64, max_ctx=64) == 2      # capped by the context
+    assert plan_batch([200], [8], free_slots=3, free_pages=2, max_batch=64, max_ctx=4096) == 0
+    assert plan_batch([1] * 9, [1] * 9, free_slots=9, free_pages=9, max_batch=4, max_ctx=64) == 4
+
+
+def test_loop_unequal_batch_early_finishers_and_slot_reuse():
+    eng, samp = FakeEngine(), ScriptSampler()
+    cfgs = [GenerateConfig(max_tokens=n, sampler=SamplerConfig(temperature=0)) for n in (3, 1, 5, 2, 4)]
+    prompts = [[1] * 5, [2] * 9, [3], [4] * 2, [5] * 7]
+    seen = []
+    results, stats = generate(eng, samp, prompts, cfgs, on_token=lambda i, t: seen.append((i, t)))
+    assert [len(r.tokens) for r in results] == [3, 1, 5, 2, 4]
+    assert all(r.finish_reason == "length" for r in results)
+    assert results[0].tokens == [105, 106, 107] and results[2].tokens == [101, 102, 103, 104, 105]
+    assert stats.batches == 2 and stats.output_tokens == 15 and len(seen) == 15        # one call per token
+    assert [t for i, t in seen if i == 4] == results[4].tokens
+    # first batch: three prompts in one step with the last place wanted, then one token each for the living
+    assert eng.steps[0] == [(0, [1] * 5, [4]), (1, [2] * 9, [8]), (2, [3], [0])]
+    assert eng.steps[1] == [(0, [105], [0]), (2, [101], [0])]                          # request 1 ended after one token
+    assert eng.steps[3] == [(2, [103], [0])]
+    # no step feeds a sequence's last token back; the second batch runs in slots the first gave back
+    assert sum(len(s) for s in eng.steps) == 3 + 2 + 2 + 1 + 1 + 2 + 2 + 1 + 1
+    assert sorted(eng.closed) == [0, 0, 1, 1, 2] and not eng.held and eng.free_slots() == 3
+
+
+def test_loop_stop_tokens_are_not_emitted_nor_fed_back():
+    eng = FakeEngine()
+    samp = ScriptSampler(stop_at={(0, 7): 2, (1, 3): 9})      # request 0 stops at its third choice, request 1 at once
+    cfg = GenerateConfig(max_tokens=6, sampler=SamplerConfig(temperature=0))
+    results, _ = generate(eng, samp, [[1] * 5, [1] * 3, [1] * 2], [cfg] * 3, default_stop=(2, 9))
+    assert results[0].tokens == [105, 106] and results[0].finish_reason == "stop"
+    assert results[1].tokens == [] and results[1].finish_reason == "stop"             # immediate stop: nothing
+    assert len(results[2].tokens) == 6 and results[2].finish_reason == "length"
+    fed = [t for s in eng.steps[1:] for _, toks, _ in s for t in toks]
+    assert 2 not in fed and 9 not in fed
+    # the same script with ignore_eos runs to the length
+    cfg2 = GenerateConfig(max_tokens=6, sampler=SamplerConfig(temperature=0), ignore_eos=True)
+    r2, _ = generate(FakeEngine(), ScriptSampler(stop_at={(0, 7): 2}), [[1] * 5], [cfg2], default_stop=(2,))
+    assert len(r2[0].tokens) == 6 and 2 in r2[0].tokens
+    # a request's own stop set replaces the model's
+    cfg3 = GenerateConfig(max_tokens=6, sampler=SamplerConfig(temperature=0), stop_tokens=(106,))
+    r3, _ = generate(FakeEngine(), ScriptSampler(), [[1] * 5], [cfg3], default_stop=(105,))
+    assert r3[0].tokens == [105] and r3[0].finish_reason == "stop"
+
+
+def test_loop_context_end_and_errors():
+    eng = FakeEngine(max_ctx=16, pages=4)
+    cfg = GenerateConfig(max_tokens=100, sampler=SamplerConfig(temperature=0))
+    results, _ = generate(eng, ScriptSampler(), [[1] * 10], [cfg])
+    assert results[0].finish_reason == "context" and len(results[0].tokens) == 5      # stops when 15 tokens are cached
+    with pytest.raises(GenerationError, match="prompt too long: 16 tokens"):
+        generate(eng, ScriptSampler(), [[1] * 16], [cfg])
+    with pytest.raises(GenerationError, match="empty prompt"):
+        generate(eng, ScriptSampler(), [[]], [cfg])
+    with pytest.raises(GenerationError, match="do not fit"):
+        generate(FakeEngine(max_ctx=4096, pages=1), ScriptSampler(), [[1] * 70], [cfg])
+    zero, _ = generate(eng, ScriptSampler(), [[1] * 3], [GenerateConfig(max_tokens=0)])
+    assert zero[0].tokens == [] and zero[0].finish_reason == "length" and not eng.held
+
+
+def test_loop_gives_slots_back_when_a_step_fails():
+    class Failing(FakeEngine):
+        def step(self, entries):
+            if len(self.steps) == 2:
+                raise RuntimeError("boom")
+            return super().step(entries)
+    eng = Failing()
+    cfg = GenerateConfig(max_tokens=5, sampler=SamplerConfig(temperature=0))
+    with pytest.raises(RuntimeError, match="boom"):
+        generate(eng, ScriptSampler(), [[1] * 5, [1] * 2], [cfg, cfg])
+    assert not eng.held and eng.free_slots() == 3
+
+
+def test_draws_are_per_request_and_seeded():
+    samp = ScriptSampler()
+    cfg = GenerateConfig(max_tokens=3, seed=77)
+    generate(FakeEngine(), samp, [[1] * 4, [1] * 2], [cfg, cfg])
+    u0 = [c[1] for c in samp.calls]
+    assert u0[0] == [uniform(77, 0, 0), uniform(77, 1, 0)] and u0[2] == [uniform(77, 0, 2), uniform(77, 1, 2)]
+    assert all(0.0 <= x < 1.0 for call in u0 for x in call)
+    assert np.float32(u0[1][0]) == u0[1][0]                      # representable in float32
+    assert samp.calls[2][2] == [[104, 105], [102, 103]]          # the tokens so far, for the repetition penalty
+    vals = [uniform(1, 0, s) for s in range(4000)]
+    assert abs(np.mean(vals) - 0.5) < 0.02 and len(set(vals)) > 3990
+
+
+def test_options_have_the_reference_defaults_and_meanings():
+    """ops/sampling.go:19-27, models/llm/generate.go:25-31, dlgo.go:213-248."""
+    d = apply_options([])
+    assert (d.max_tokens, d.seed) == (256, -1)
+    s = d.sampler
+    assert (s.temperature, s.top_k, s.top_p, s.min_p, s.repetition_penalty) == (0.7, 40, 0.9, 0.0, 1.1)
+    c = apply_options([with_max_tokens(5), with_temperature(0.3), with_top_k(7), with_top_p(0.5), with_seed(9)])
+    assert (c.max_tokens, c.sampler.temperature, c.sampler.top_k, c.sampler.top_p, c.seed) == (5, 0.3, 7, 0.5, 9)
+    assert apply_options([with_greedy()]).sampler.greedy and apply_options([with_temperature(0)]).sampler.greedy
+    assert apply_options([]).sampler is not apply_options([]).sampler
+    with pytest.raises(ValueError):
+        apply_options([with_temperature(-1)])
+    import dlgo_amd
+    assert dlgo_amd.WithMaxTokens is dlgo_amd.with_max_tokens and dlgo_amd.LoadLLM is dlgo_amd.load_llm
+
+
+def test_command_line_checks_like_the_reference(capsys):
+    """examples/simple_chat/main.go:28-39."""
+    from dlgo_amd.cli import main
+    assert main(["--ctx", "0", "x"]) == 1 and "--ctx must be > 0" in capsys.readouterr().err
+    assert main(["--max-tokens", "0", "x"]) == 1 and "--max-tokens must be > 0" in capsys.readouterr().err
+    assert main(["--temp", "-0.1", "x"]) == 1 and "--temp must be >= 0" in capsys.readouterr().err
+
+
+def test_engine_refuses_to_run_without_a_gpu(tmp_path):
+    if torch.cuda.is_available():
+        pytest.skip("a GPU is present")
+    from conftest import TINY_A, make_folder
+    from dlgo_amd.engine import Engine, EngineError
+    folder = make_folder(TINY_A, 1, tmp_path)
+    with pytest.raises(EngineError, match="no HIP device"):
+        Engine.from_folder(folder, "float32")

@@ -1,0 +1,206 @@
+"""Configuration, registry and weight loading: the errors a user can cause, without a GPU."""
+import copy
+import json
+import os
+
+import pytest
+import torch
+
+from conftest import TINY_A, TINY_B, TINY_C, make_folder
+from dlgo_amd import models  # noqa: F401
+from dlgo_amd.config import (ConfigError, LlamaConfig, build_model, config_from_dict, known_architectures, load_config,
+                             register_architecture)
+from dlgo_amd.weights import (SafetensorsFile, WeightsError, load_state, load_weights, random_tensors, write_random_model,
+                              write_safetensors)
+
+
+def test_config_reads_every_key(tiny_b):
+    c = config_from_dict(tiny_b)
+    assert isinstance(c, LlamaConfig)
+    assert (c.vocab_size, c.hidden_size, c.num_hidden_layers, c.intermediate_size) == (384, 128, 3, 352)
+    assert (c.num_attention_heads, c.num_key_value_heads, c.head_dim) == (4, 1, 32)
+    assert (c.q_dim, c.kv_dim, c.group) == (128, 32, 4)
+    assert c.rms_norm_eps == 1e-6 and c.rope_theta == 500000.0 and c.max_position_embeddings == 512
+    assert c.rope_scaling.factor == 4.0 and c.rope_scaling.original_max_position_embeddings == 64
+    assert c.tie_word_embeddings is False and c.eos_token_ids == (3, 5) and c.bos_token_id == 0
+    # round trip
+    assert config_from_dict(c.to_dict()) == c
+
+
+def test_config_defaults_are_derived_not_invented(tiny_a):
+    raw = dict(tiny_a)
+    del raw["num_key_value_heads"], raw["head_dim"]
+    c = config_from_dict(raw)
+    assert c.num_key_value_heads == 4 and c.head_dim == 16
+    for key in ("vocab_size", "hidden_size", "num_hidden_layers", "intermediate_size", "num_attention_heads",
+                "rms_norm_eps", "rope_theta", "max_position_embeddings"):
+        bad = dict(tiny_a)
+        del bad[key]
+        with pytest.raises(ConfigError, match=key):
+            config_from_dict(bad)
+
+
+@pytest.mark.parametrize("change,needle", [
+    ({"num_key_value_heads": 3}, "multiple of num_key_value_heads"),
+    ({"head_dim": 15}, "even"),
+    ({"hidden_act": "gelu"}, "hidden_act"),
+    ({"attention_bias": True}, "attention_bias"),
+    ({"mlp_bias": True}, "mlp_bias"),
+    ({"rope_scaling": {"rope_type": "yarn", "factor": 2.0}}, "rope_type"),
+    ({"rope_scaling": {"rope_type": "llama3", "factor": 2.0}}, "low_freq_factor"),
+    ({"vocab_size": "many"}, "vocab_size"),
+    ({"rms_norm_eps": 0}, "rms_norm_eps"),
+    ({"eos_token_id": 999}, "outside the vocabulary"),
+    ({"architectures": ["MambaForCausalLM"]}, "unknown architecture"),
+    ({"architectures": None}, "architectures"),
+])
+def test_config_errors_name_the_key(tiny_a, change, needle):
+    raw = dict(tiny_a)
+    raw.update(change)
+    with pytest.raises(ConfigError, match=needle):
+        config_from_dict(raw)
+
+
+def test_config_collects_all_problems(tiny_a):
+    raw = dict(tiny_a, vocab_size=-1, rope_theta="x", hidden_act="relu")
+    with pytest.raises(ConfigError) as e:
+        config_from_dict(raw)
+    assert all(k in str(e.value) for k in ("vocab_size", "rope_theta", "hidden_act"))
+
+
+def test_registry(tmp_path, tiny_a):
+    assert "LlamaForCausalLM" in known_architectures()
+    (tmp_path / "config.json").write_text(json.dumps(tiny_a))
+    assert load_config(str(tmp_path)) == config_from_dict(tiny_a)
+    with pytest.raises(ConfigError, match="no such file"):
+        load_config(str(tmp_path / "nowhere"))
+    (tmp_path / "config.json").write_text("{ not json")
+    with pytest.raises(ConfigError, match="not JSON"):
+        load_config(str(tmp_path))
+
+
+def test_model_is_made_of_parts_chosen_by_name(tiny_b):
+    m = build_model(config_from_dict(tiny_b))
+    names = m.expected_tensors()
+    assert names["model.layers.2.self_attn.k_proj.weight"].shape == (32, 128)
+    assert names["model.layers.0.mlp.down_proj.weight"].shape == (128, 352)
+    assert names["lm_head.weight"].shape == (384, 128) and names["model.norm.weight"].kind == "vector"
+    assert len(names) == 3 * 9 + 3
+    tied = build_model(config_from_dict(TINY_A))
+    assert "lm_head.weight" not in tied.expected_tensors()
+    assert [r.layer for r in m.order] == [0, 1, 2] and m.run_unit == [0, 1, 2]
+    need = m.unit_needs[0][0]
+    assert (need.kind, need.kv_heads, need.head_dim, need.window) == ("kv", 1, 32, None)
+
+
+# -- weights --------------------------------------------------------------------
+def test_random_folder_round_trip(tmp_path, tiny_c):
+    folder = make_folder(tiny_c, 5, tmp_path, norm_jitter=0.1)
+    cfg = load_config(folder)
+    sf = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+    assert set(sf.infos) == set(build_model(cfg).expected_tensors())
+    assert all(i.dtype == "BF16" for i in sf.infos.values())               # the configuration says bfloat16
+    t = sf.tensor("model.layers.1.mlp.gate_proj.weight")
+    assert t.shape == (136, 96) and abs(t.float().std().item() - 0.05) < 0.005
+    n = sf.tensor("model.norm.weight").float()
+    assert 0.05 < n.std().item() < 0.2 and abs(n.mean().item() - 1) < 0.1
+    # a seed gives the same tensors again, another seed others; a tensor does not depend on its neighbours
+    again = random_tensors(cfg, 5, norm_jitter=0.1)
+    assert torch.equal(again["model.layers.1.mlp.gate_proj.weight"], t)
+    assert not torch.equal(random_tensors(cfg, 6)["model.layers.1.mlp.gate_proj.weight"], t)
+    model = build_model(cfg)
+    load_weights(model, folder, "cpu", torch.float32)
+    w = model.layers[0][1].mixer.w_qkv
+    assert w.shape == (6 * 48 + 2 * 3 * 48, 96) and w.dtype == torch.float32
+    assert model.final_norm.weight.dtype == torch.float32
+    gu = model.layers[1][1].ffn.w_gate_up
+    assert torch.equal(gu[0::2], t.float()) and gu.shape == (272, 96)       # gate rows interleaved with up rows
+    assert model.head.weight is model.embedding.weight                      # tied
+
+
+def test_storage_rule(tmp_path, tiny_a):
+    """Matrices in the run dtype; norm weights in float32 whatever the file holds."""
+    folder = make_folder(tiny_a, 1, tmp_path, dtype="float32")
+    m = build_model(load_config(folder))
+    load_weights(m, folder, "cpu", torch.bfloat16)
+    assert m.embedding.weight.dtype == torch.bfloat16
+    assert m.layers[0][1].mixer_norm.weight.dtype == torch.float32
+
+
+def _rewrite(folder, edit):
+    path = os.path.join(folder, "model.safetensors")
+    sf = SafetensorsFile(path)
+    tensors = {n: sf.tensor(n).clone() for n in sf.infos}
+    edit(tensors)
+    write_safetensors(path, tensors)
+
+
+def test_one_error_lists_everything_wrong(tmp_path, tiny_b):
+    folder = make_folder(tiny_b, 2, tmp_path)
+
+    def edit(t):
+        del t["model.layers.1.self_attn.v_proj.weight"]
+        del t["lm_head.weight"]
+        t["model.layers.0.mlp.up_proj.weight"] = torch.zeros(352, 127)
+        t["model.layers.9.self_attn.q_proj.weight"] = torch.zeros(2, 2)
+        t["model.norm.weight"] = torch.zeros(128, dtype=torch.int32)
+    _rewrite(folder, edit)
+    m = build_model(load_config(folder))
+    with pytest.raises(WeightsError) as e:
+        load_weights(m, folder, "cpu", torch.float32)
+    err = e.value
+    assert sorted(err.missing) == ["lm_head.weight", "model.layers.1.self_attn.v_proj.weight"]
+    assert err.unexpected == ["model.layers.9.self_attn.q_proj.weight"]
+    assert err.wrong_shape == [("model.layers.0.mlp.up_proj.weight", (352, 128), (352, 127))]
+    assert err.wrong_type == [("model.norm.weight", "I32")]
+    text = str(err)
+    for needle in ("missing (2)", "unexpected (1)", "expected [352, 128], found [352, 127]", "model.norm.weight is I32"):
+        assert needle in text
+
+
+def test_tied_model_may_carry_the_head(tmp_path, tiny_a):
+    folder = make_folder(tiny_a, 3, tmp_path)
+    _rewrite(folder, lambda t: t.__setitem__("lm_head.weight", t["model.embed_tokens.weight"].clone()))
+    load_weights(build_model(load_config(folder)), folder, "cpu", torch.float32)
+
+
+def test_missing_and_truncated_files(tmp_path, tiny_a):
+    folder = make_folder(tiny_a, 4, tmp_path)
+    m = build_model(load_config(folder))
+    path = os.path.join(folder, "model.safetensors")
+    data = open(path, "rb").read()
+    open(path, "wb").write(data[:len(data) // 2])
+    with pytest.raises(WeightsError, match="truncated"):
+        load_weights(m, folder, "cpu", torch.float32)
+    os.remove(path)
+    with pytest.raises(WeightsError, match="model.safetensors"):
+        load_weights(m, folder, "cpu", torch.float32)
+
+
+def test_sharded_folder(tmp_path, tiny_a):
+    folder = make_folder(tiny_a, 5, tmp_path)
+    path = os.path.join(folder, "model.safetensors")
+    sf = SafetensorsFile(path)
+    names = sorted(sf.infos)
+    half = len(names) // 2
+    shards = {"a.safetensors": names[:half], "b.safetensors": names[half:]}
+    for fname, ns in shards.items():
+        write_safetensors(os.path.join(folder, fname), {n: sf.tensor(n).clone() for n in ns})
+    os.remove(path)
+    json.dump({"weight_map": {n: f for f, ns in shards.items() for n in ns}},
+              open(os.path.join(folder, "model.safetensors.index.json"), "w"))
+    m = build_model(load_config(folder))
+    load_weights(m, folder, "cpu", torch.float32)
+    assert m.embedding.weight.shape == (256, 64)
+
+
+def test_load_state_checks_too(tiny_a):
+    cfg = config_from_dict(tiny_a)
+    tensors = random_tensors(cfg, 0)
+    tensors.pop("model.norm.weight")
+    with pytest.raises(WeightsError, match="model.norm.weight"):
+        load_state(build_model(cfg), tensors, "cpu", torch.float32)
+    with pytest.raises(ValueError, match="initializer_range"):
+        raw = dict(tiny_a)
+        del raw["initializer_range"]
+        random_tensors(config_from_dict(raw), 0)
