@@ -386,16 +386,29 @@ __global__ __launch_bounds__(WAVE) void attn_decode_kernel(
     const bf16_t* kpage = cache + (size_t)page * page_stride + (size_t)kvh * PAGE * HD;
     const bf16_t* vpage = cache + v_off + (size_t)page * page_stride + (size_t)kvh * HD * PAGE;
     const int key0 = pg * PAGE;
+    // every load of the page is issued before the first product
+    uint4 kf[4][KS];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const bf16_t* krow = kpage + (size_t)(t * 16 + j) * HD + G * 8;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) kf[t][ks] = (ks * 32 + G * 8 < HD) ? *(const uint4*)(krow + ks * 32) : make_uint4(0, 0, 0, 0);
+    }
+    uint2 vf[2][DT][2];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int d = 0; d < DT; ++d) {
+        const bf16_t* vrow = vpage + (size_t)(d * 16 + j) * PAGE + 32 * u + 4 * G;
+        vf[u][d][0] = *(const uint2*)(vrow);
+        vf[u][d][1] = *(const uint2*)(vrow + 16);
+      }
     f32x4_t s[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       s[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-      const bf16_t* krow = kpage + (size_t)(t * 16 + j) * HD + G * 8;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const uint4 a = (ks * 32 + G * 8 < HD) ? *(const uint4*)(krow + ks * 32) : make_uint4(0, 0, 0, 0);
-        s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), as_bf16x8(qf[ks]), s[t], 0, 0, 0);
-      }
+      for (int ks = 0; ks < KS; ++ks) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[t][ks]), as_bf16x8(qf[ks]), s[t], 0, 0, 0);
     }
     // lane: head = lane%16; element v of tile t is key  key0 + 16 t + 4 G + v
     const bool need_mask = key0 + PAGE - 1 > pos || key0 < lo;
@@ -443,8 +456,7 @@ __global__ __launch_bounds__(WAVE) void attn_decode_kernel(
       const int ka = 32 * u + 4 * G, kb = ka + 16;      // first keys (within the page) of the two 4-key pieces
 #pragma unroll
       for (int d = 0; d < DT; ++d) {
-        const bf16_t* vrow = vpage + (size_t)(d * 16 + j) * PAGE;
-        uint2 a0 = *(const uint2*)(vrow + ka), a1 = *(const uint2*)(vrow + kb);
+        uint2 a0 = vf[u][d][0], a1 = vf[u][d][1];
         if (tail) {
           uint32_t* w0 = (uint32_t*)&a0;
           uint32_t* w1 = (uint32_t*)&a1;
@@ -475,19 +487,22 @@ __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restr
                                                             const int32_t* __restrict__ positions, int n_heads, int ppw,
                                                             int n_splits, int window) {
   constexpr int HD = HEAD_DIM;
+  constexpr int PS = HD + 4;
   const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int pos = positions[seq];
   const int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
   const int s0 = (lo / PAGE) / ppw, s1 = (pos / PAGE) / ppw;
-  const float* base = part + (size_t)(seq * n_heads + head) * n_splits * (HD + 4);
+  const float* base = part + (size_t)(seq * n_heads + head) * n_splits * PS;
   float M = -INFINITY;
-  for (int s = s0; s <= s1; ++s) M = fmaxf(M, base[(size_t)s * (HD + 4) + HD]);
+  for (int s = s0 + lane; s <= s1; s += WAVE) M = fmaxf(M, base[(size_t)s * PS + HD]);
+  M = wave_max(M);
   float L = 0.f;
-  for (int s = s0; s <= s1; ++s) L += fast_exp2(base[(size_t)s * (HD + 4) + HD] - M) * base[(size_t)s * (HD + 4) + HD + 1];
+  for (int s = s0 + lane; s <= s1; s += WAVE) L += fast_exp2(base[(size_t)s * PS + HD] - M) * base[(size_t)s * PS + HD + 1];
+  L = wave_sum(L);
   const float inv = 1.0f / L;
   for (int d = lane; d < HD; d += WAVE) {
     float acc = 0.f;
-    for (int s = s0; s <= s1; ++s) acc += fast_exp2(base[(size_t)s * (HD + 4) + HD] - M) * base[(size_t)s * (HD + 4) + d];
+    for (int s = s0; s <= s1; ++s) acc = fmaf(fast_exp2(base[(size_t)s * PS + HD] - M), base[(size_t)s * PS + d], acc);
     out[(size_t)seq * ldo + (size_t)head * HD + d] = f32_to_bf16(acc * inv);
   }
 }

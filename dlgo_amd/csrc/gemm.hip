@@ -277,6 +277,153 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE) void gemv_kernel(const T* __restr
 }
 
 // ----------------------------------------------------------------------------
+// MFMA kernel for a few rows of X (decode): 16 rows of W per block, k split over the waves
+// ----------------------------------------------------------------------------
+// A block owns 16 consecutive rows of W and every token of the step (up to 16 * TB).  Its NW waves take
+// the 128-byte pieces of those rows in turn (wave w: pieces w, w + NW, ...), so together they stream the
+// rows front to back; each piece is two 16x16 MFMA steps with W as the row operand and X as the column
+// operand.  The waves' partial tiles are summed through LDS in wave order, then wave 0 runs the epilogue:
+// a lane holds four consecutive n of one token, as in the tiled kernel.
+//
+// NORM: X is the float32 residual stream and the product is taken with rmsnorm(X) * norm_w without
+// writing the normed rows: the column operand is X[t,k] * norm_w[k], the sum of squares of each token is
+// gathered on the way, and 1/sqrt(mean + eps) multiplies the finished sums (it is a scalar per token).
+template <typename T> struct Mma16;
+template <> struct Mma16<bf16_t> {
+  static __device__ __forceinline__ void run(const uint4& a, const uint4& b, f32x4_t& c) {
+    union { uint4 u; bf16x8_t v; } ua, ub;
+    ua.u = a;
+    ub.u = b;
+    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ua.v, ub.v, c, 0, 0, 0);
+  }
+  // 8 floats -> one 16-byte operand
+  static __device__ __forceinline__ uint4 pack(const float* f) {
+    union { uint4 u; bf16x8_t v; } x;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x.v[e] = (__bf16)f[e];
+    return x.u;
+  }
+};
+template <> struct Mma16<float> {
+  static __device__ __forceinline__ void run(const uint4& a, const uint4& b, f32x4_t& c) {
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint4 pack(const float* f) {
+    return make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3]));
+  }
+};
+
+#define SKINNY_WAVES 8
+
+template <typename T, int TB, int EPI, bool NORM>
+__global__ __launch_bounds__(SKINNY_WAVES* WAVE) void skinny_kernel(const T* __restrict__ W, const void* __restrict__ Xv,
+                                                                     const float* __restrict__ norm_w, float eps,
+                                                                     void* __restrict__ Y, int N, int Tn, int K, int ldw,
+                                                                     int ldx, int ldy) {
+  constexpr int NW = SKINNY_WAVES;
+  constexpr int EPC = 16 / sizeof(T);          // elements of a 16-byte operand
+  constexpr int PIECE = 8 * EPC;               // elements of a 128-byte piece of a row
+  __shared__ float red[NW][TB][16][17];
+  __shared__ float ssq[NW][TB][16];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int j = lane & 15, G = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const T* wrow = W + (size_t)(n0 + j < N ? n0 + j : N - 1) * ldw;
+
+  f32x4_t acc[TB];
+  float ss[TB];
+#pragma unroll
+  for (int c = 0; c < TB; ++c) {
+    acc[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    ss[c] = 0.f;
+  }
+  const int pieces = (K + PIECE - 1) / PIECE;
+#pragma unroll 2
+  for (int p = wave; p < pieces; p += NW) {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {            // the two 64-byte halves of the piece
+      const int k = p * PIECE + h * 4 * EPC + G * EPC;
+      const bool in = k < K;
+      const uint4 a = in ? *(const uint4*)(wrow + k) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int c = 0; c < TB; ++c) {
+        const int t = c * 16 + j;
+        uint4 b = make_uint4(0, 0, 0, 0);
+        if (in && t < Tn) {
+          if (NORM) {
+            const float* xr = (const float*)Xv + (size_t)t * ldx + k;
+            float f[EPC];
+#pragma unroll
+            for (int e = 0; e < EPC; e += 4) {
+              const float4 x4 = *(const float4*)(xr + e);
+              const float4 w4 = *(const float4*)(norm_w + k + e);
+              ss[c] = fmaf(x4.x, x4.x, ss[c]);
+              ss[c] = fmaf(x4.y, x4.y, ss[c]);
+              ss[c] = fmaf(x4.z, x4.z, ss[c]);
+              ss[c] = fmaf(x4.w, x4.w, ss[c]);
+              f[e] = x4.x * w4.x;
+              f[e + 1] = x4.y * w4.y;
+              f[e + 2] = x4.z * w4.z;
+              f[e + 3] = x4.w * w4.w;
+            }
+            b = Mma16<T>::pack(f);
+          } else {
+            b = *(const uint4*)((const T*)Xv + (size_t)t * ldx + k);
+          }
+        }
+        Mma16<T>::run(a, b, acc[c]);
+      }
+    }
+  }
+  // lane: token = 16 c + j, rows 4 G + v.  Partial tiles go to LDS; wave 0 adds them in wave order.
+#pragma unroll
+  for (int c = 0; c < TB; ++c) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[wave][c][4 * G + v][j] = acc[c][v];
+    if (NORM) {
+      float s = ss[c];
+      s += __shfl_xor(s, 16, WAVE);
+      s += __shfl_xor(s, 32, WAVE);
+      if (G == 0) ssq[wave][c][j] = s;
+    }
+  }
+  __syncthreads();
+  if (wave != 0) return;
+#pragma unroll
+  for (int c = 0; c < TB; ++c) {
+    const int t = c * 16 + j;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int w = 0; w < NW; ++w)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[r] += red[w][c][4 * G + r][j];
+    if (NORM) {
+      float s = 0.f;
+      for (int w = 0; w < NW; ++w) s += ssq[w][c][j];
+      const float scale = 1.0f / sqrtf(s / (float)K + eps);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[r] *= scale;
+    }
+    if (t < Tn) epilogue4<T, EPI>(Y, ldy, N, t, n0 + 4 * G, v[0], v[1], v[2], v[3]);
+  }
+}
+
+template <typename T, int EPI, bool NORM>
+static void launch_skinny(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K, int ldw,
+                          int ldx, int ldy, hipStream_t stream) {
+  dim3 g((N + 15) / 16), b(SKINNY_WAVES * WAVE);
+  const int tb = (Tn + 15) / 16;
+#define SKINNY_GO(TB_) hipLaunchKernelGGL((skinny_kernel<T, TB_, EPI, NORM>), g, b, 0, stream, (const T*)W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy)
+  if (tb <= 1) SKINNY_GO(1);
+  else if (tb == 2) SKINNY_GO(2);
+  else if (tb == 3) SKINNY_GO(3);
+  else SKINNY_GO(4);
+#undef SKINNY_GO
+}
+
+// ----------------------------------------------------------------------------
 // host side
 // ----------------------------------------------------------------------------
 template <typename T, int BN, int BT, int WN, int WT, int EPI>
@@ -301,10 +448,10 @@ static void launch_gemv(const void* W, const void* X, void* Y, int N, int Tn, in
 template <typename T, int EPI>
 static void dispatch(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy, int force,
                      hipStream_t stream) {
-  // force: 0 = choose, 1 = gemv, 2 = 128x128 tiles, 3 = 64x64, 4 = 32x32
+  // force: 0 = choose, 1 = gemv, 2 = 128x128 tiles, 3 = 64x64, 4 = 32x32, 5 = 16 rows of W per block
   int kind = force;
   if (kind == 0) {
-    if (Tn <= 8) kind = 1;
+    if (Tn <= 64) kind = 5;
     else {
       const long big = (long)((N + 127) / 128) * ((Tn + 127) / 128);
       const long mid = (long)((N + 63) / 64) * ((Tn + 63) / 64);
@@ -312,6 +459,7 @@ static void dispatch(const void* W, const void* X, void* Y, int N, int Tn, int K
     }
   }
   if (kind == 1) launch_gemv<T, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else if (kind == 5) launch_skinny<T, EPI, false>(W, X, nullptr, 0.f, Y, N, Tn, K, ldw, ldx, ldy, stream);
   else if (kind == 2) launch_tiled<T, 128, 128, 2, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   else if (kind == 3) launch_tiled<T, 64, 64, 2, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   else launch_tiled<T, 32, 32, 1, 1, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
@@ -341,12 +489,50 @@ extern "C" const char* dlgo_gemm(const void* W, const void* X, void* Y, int dtyp
   DLGO_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && ((uintptr_t)Y & 15) == 0, "gemm: operands must be 16-byte aligned");
   DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm: SwiGLU epilogue needs an even N and ldy >= N/2");
   DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm: ldy %d shorter than N %d", ldy, N);
-  DLGO_REQUIRE(force_kind >= 0 && force_kind <= 4, "gemm: unknown kernel choice %d", force_kind);
+  DLGO_REQUIRE(force_kind >= 0 && force_kind <= 5, "gemm: unknown kernel choice %d", force_kind);
   DLGO_REQUIRE(force_kind != 1 || Tn <= 8, "gemm: the streaming kernel takes at most 8 rows, got %d", Tn);
+  DLGO_REQUIRE(force_kind != 5 || Tn <= 64, "gemm: the 16-row kernel takes at most 64 rows of X, got %d", Tn);
   if (Tn == 0) return nullptr;
   const char* err = dtype == DLGO_DTYPE_F32 ? by_epilogue<float>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, force_kind, stream)
                                             : by_epilogue<bf16_t>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, force_kind, stream);
   if (err) return err;
   DLGO_LAUNCH_CHECK("gemm");
+  return nullptr;
+}
+
+// Y (epilogue)= (rmsnorm(X) * norm_w) W^T for up to 64 rows of the float32 residual stream X [T, K], without
+// writing the normed rows.  Epilogues as dlgo_gemm.
+extern "C" const char* dlgo_gemm_rmsnorm(const void* W, const float* X, const float* norm_w, float eps, void* Y, int dtype, int N,
+                                         int Tn, int K, int ldw, int ldx, int ldy, int epilogue, hipStream_t stream) {
+  DLGO_REQUIRE(N > 0 && Tn >= 0 && Tn <= 64 && K > 0, "gemm_rmsnorm: bad sizes N=%d T=%d K=%d (at most 64 rows)", N, Tn, K);
+  DLGO_REQUIRE(dtype == DLGO_DTYPE_F32 || dtype == DLGO_DTYPE_BF16, "gemm_rmsnorm: unknown dtype code %d", dtype);
+  const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
+  DLGO_REQUIRE(K % epc == 0 && ldw % epc == 0 && ldx % 4 == 0 && ldw >= K && ldx >= K, "gemm_rmsnorm: K and the row strides must be multiples of %d", epc);
+  DLGO_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && ((uintptr_t)Y & 15) == 0 && ((uintptr_t)norm_w & 15) == 0,
+               "gemm_rmsnorm: operands must be 16-byte aligned");
+  DLGO_REQUIRE(eps > 0.f, "gemm_rmsnorm: eps must be positive");
+  DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm_rmsnorm: SwiGLU epilogue needs an even N and ldy >= N/2");
+  DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm_rmsnorm: ldy %d shorter than N %d", ldy, N);
+  if (Tn == 0) return nullptr;
+#define NORM_GO(T_, E_) launch_skinny<T_, E_, true>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream)
+  if (dtype == DLGO_DTYPE_F32) {
+    switch (epilogue) {
+      case EPI_STORE: NORM_GO(float, EPI_STORE); break;
+      case EPI_ACCUM_F32: NORM_GO(float, EPI_ACCUM_F32); break;
+      case EPI_SWIGLU: NORM_GO(float, EPI_SWIGLU); break;
+      case EPI_STORE_F32: NORM_GO(float, EPI_STORE_F32); break;
+      default: DLGO_FAIL("gemm_rmsnorm: unknown epilogue %d", epilogue);
+    }
+  } else {
+    switch (epilogue) {
+      case EPI_STORE: NORM_GO(bf16_t, EPI_STORE); break;
+      case EPI_ACCUM_F32: NORM_GO(bf16_t, EPI_ACCUM_F32); break;
+      case EPI_SWIGLU: NORM_GO(bf16_t, EPI_SWIGLU); break;
+      case EPI_STORE_F32: NORM_GO(bf16_t, EPI_STORE_F32); break;
+      default: DLGO_FAIL("gemm_rmsnorm: unknown epilogue %d", epilogue);
+    }
+  }
+#undef NORM_GO
+  DLGO_LAUNCH_CHECK("gemm_rmsnorm");
   return nullptr;
 }

@@ -16,7 +16,7 @@ from . import build
 PAGE = 64   # tokens per cache page; the kernels are compiled with the same number
 
 EPI_STORE, EPI_ACCUM_F32, EPI_SWIGLU, EPI_STORE_F32 = 0, 1, 2, 3
-GEMM_AUTO, GEMM_STREAM, GEMM_TILE128, GEMM_TILE64, GEMM_TILE32 = 0, 1, 2, 3, 4
+GEMM_AUTO, GEMM_STREAM, GEMM_TILE128, GEMM_TILE64, GEMM_TILE32, GEMM_ROWS16 = 0, 1, 2, 3, 4, 5
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 
@@ -68,7 +68,7 @@ def _lib(module: str, defines=()):
     lib = build.load(module, defines)
     key = (module, tuple(defines))
     if key not in _protos_done:
-        for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_attention_rows",
+        for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_rmsnorm", "dlgo_attention_rows",
                      "dlgo_attention_prefill", "dlgo_attention_decode", "dlgo_argmax", "dlgo_sample"):
             if hasattr(lib, name):
                 getattr(lib, name).restype = ctypes.c_char_p
@@ -132,6 +132,31 @@ def gemm(weight: torch.Tensor, x: torch.Tensor, out: torch.Tensor, epilogue: int
     _check(_lib("gemm").dlgo_gemm(_ptr(weight), _ptr(x), _ptr(out), dtype_code(weight.dtype), n, t, k,
                                   _rows(weight, "gemm weight"), _rows(x, "gemm input"), _rows(out, "gemm output"),
                                   epilogue, kind, _stream()))
+    return out
+
+
+FUSED_NORM_ROWS = 64   # most rows of the residual stream that gemm_rmsnorm takes
+
+
+def gemm_rmsnorm(weight: torch.Tensor, x: torch.Tensor, norm_weight: torch.Tensor, eps: float, out: torch.Tensor,
+                 epilogue: int = EPI_STORE) -> torch.Tensor:
+    """out (epilogue)= (rmsnorm(x) * norm_weight) @ weight.T for up to 64 rows x of the float32 residual stream,
+    without writing the normed rows.  Epilogues as gemm()."""
+    _need(weight, "gemm weight", dims=2)
+    _need(x, "residual rows", torch.float32, 2)
+    _need(norm_weight, "norm weight", torch.float32, 1)
+    n, k = weight.shape
+    t = x.shape[0]
+    if x.shape[1] != k or norm_weight.shape[0] != k or t > FUSED_NORM_ROWS:
+        raise KernelError(f"gemm_rmsnorm: rows {tuple(x.shape)} and norm weight {tuple(norm_weight.shape)} do not fit weight {tuple(weight.shape)} (at most {FUSED_NORM_ROWS} rows)")
+    want_dtype = torch.float32 if epilogue in (EPI_ACCUM_F32, EPI_STORE_F32) else weight.dtype
+    _need(out, "gemm output", want_dtype, 2)
+    cols = n // 2 if epilogue == EPI_SWIGLU else n
+    if tuple(out.shape) != (t, cols):
+        raise KernelError(f"gemm_rmsnorm: output {tuple(out.shape)}, expected {(t, cols)}")
+    _check(_lib("gemm").dlgo_gemm_rmsnorm(_ptr(weight), _ptr(x), _ptr(norm_weight), ctypes.c_float(eps), _ptr(out),
+                                          dtype_code(weight.dtype), n, t, k, _rows(weight, "gemm weight"),
+                                          _rows(x, "residual rows"), _rows(out, "gemm output"), epilogue, _stream()))
     return out
 
 
@@ -269,7 +294,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
 
 def decode_pages_per_wave(n_pairs: int, max_pages: int) -> int:
     """Pages of keys one wave of the split kernel takes: enough waves to fill the chip, few enough partials."""
-    return max(1, min(8, (n_pairs * max_pages) // 2048))
+    return max(1, min(8, (n_pairs * max_pages) // 4096))
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:

@@ -21,6 +21,7 @@ import torch
 
 from ..kernels import ops
 from .base import CacheNeed, Part, TensorSpec, stored
+from .norm import RMSNorm
 from .position import PositionEncoding
 
 
@@ -40,7 +41,12 @@ class Mixer(Part):
     def prepare(self, max_positions: int, device: torch.device) -> None:
         pass
 
-    def forward(self, xn: torch.Tensor, ctx, unit: int, residual: torch.Tensor, owns_cache: bool = True) -> None:
+    def fuses_norm(self, norm, ctx) -> bool:
+        """True if, for this step, the mixer would rather be given the float32 residual rows and the norm
+        part (forward(x, ..., norm=norm)) than the normed rows."""
+        return False
+
+    def forward(self, xn: torch.Tensor, ctx, unit: int, residual: torch.Tensor, owns_cache: bool = True, norm=None) -> None:
         raise NotImplementedError
 
 
@@ -84,18 +90,24 @@ class Attention(Mixer):
         self.w_qkv = stored(fused, spec["q_proj.weight"], device, dtype)
         self.w_o = stored(tensors["o_proj.weight"], spec["o_proj.weight"], device, dtype)
 
-    def forward(self, xn, ctx, unit, residual, owns_cache=True) -> None:
+    def fuses_norm(self, norm, ctx) -> bool:
+        return isinstance(norm, RMSNorm) and ctx.n_tokens <= ops.FUSED_NORM_ROWS
+
+    def forward(self, xn, ctx, unit, residual, owns_cache=True, norm=None) -> None:
         t = xn.shape[0]
         n_kv = self.n_kv_heads if owns_cache else 0
         cols = self.q_dim + 2 * n_kv * self.head_dim
-        qkv = ctx.buffer("attention.qkv", (t, self.q_dim + 2 * self.kv_dim), xn.dtype)
-        ops.gemm(self.w_qkv[:cols], xn, qkv[:, :cols])
+        qkv = ctx.buffer("attention.qkv", (t, self.q_dim + 2 * self.kv_dim), ctx.dtype)
+        if norm is not None:      # xn are the float32 residual rows: the norm rides in the product
+            ops.gemm_rmsnorm(self.w_qkv[:cols], xn, norm.weight, norm.eps, qkv[:, :cols])
+        else:
+            ops.gemm(self.w_qkv[:cols], xn, qkv[:, :cols])
         kv = ctx.cache.kv_view(unit)
         rot = self.position.rotation()
         ops.rope_kv(qkv, self.n_heads, n_kv, self.head_dim, rot.width if rot else 0, rot.interleaved if rot else False,
                     rot.cos if rot else None, rot.sin if rot else None, ctx.positions,
                     ctx.tok_seq, ctx.slots, kv.page_table, kv.cache, kv.page_stride, kv.v_off, write_kv=owns_cache)
-        out = ctx.buffer("attention.out", (t, self.q_dim), xn.dtype)
+        out = ctx.buffer("attention.out", (t, self.q_dim), ctx.dtype)
         self.attend(qkv, out, ctx, kv)
         ops.gemm(self.w_o, out, residual, ops.EPI_ACCUM_F32)
 

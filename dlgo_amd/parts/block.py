@@ -42,10 +42,16 @@ class PreNormBlock(Block):
 
     def forward(self, x, ctx, unit, owns_cache=True) -> None:
         xn = ctx.buffer("block.normed", tuple(x.shape), ctx.dtype)
-        self.mixer_norm(x, xn)
-        self._mixer.forward(xn, ctx, unit, x, owns_cache)
-        self.ffn_norm(x, xn)
-        self.ffn.forward(xn, ctx, x)
+        if self._mixer.fuses_norm(self.mixer_norm, ctx):
+            self._mixer.forward(x, ctx, unit, x, owns_cache, norm=self.mixer_norm)
+        else:
+            self.mixer_norm(x, xn)
+            self._mixer.forward(xn, ctx, unit, x, owns_cache)
+        if self.ffn.fuses_norm(self.ffn_norm, ctx):
+            self.ffn.forward(x, ctx, x, norm=self.ffn_norm)
+        else:
+            self.ffn_norm(x, xn)
+            self.ffn.forward(xn, ctx, x)
 
 
 BLOCKS = {"pre_norm": PreNormBlock}

@@ -10,6 +10,7 @@ import torch
 
 from ..kernels import ops
 from .base import Part, TensorSpec, stored
+from .norm import RMSNorm
 
 
 class Embedding(Part):
@@ -48,6 +49,11 @@ class OutputHead(Part):
     def weight(self) -> torch.Tensor:
         return self.tied_to.weight if self.tied_to is not None else self._weight
 
-    def __call__(self, xn: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-        """xn: normed rows (run dtype); out: float32 [rows, vocab]."""
+    def fuses_norm(self, norm, ctx) -> bool:
+        return isinstance(norm, RMSNorm) and ctx.n_tokens <= ops.FUSED_NORM_ROWS
+
+    def __call__(self, xn: torch.Tensor, out: torch.Tensor, norm=None) -> torch.Tensor:
+        """xn: normed rows (run dtype), or with `norm` the float32 residual rows; out: float32 [rows, vocab]."""
+        if norm is not None:
+            return ops.gemm_rmsnorm(self.weight, xn, norm.weight, norm.eps, out, ops.EPI_STORE_F32)
         return ops.gemm(self.weight, xn, out, ops.EPI_STORE_F32)

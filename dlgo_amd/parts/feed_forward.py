@@ -11,12 +11,17 @@ import torch
 
 from ..kernels import ops
 from .base import Part, TensorSpec, stored
+from .norm import RMSNorm
 
 
 class FeedForward(Part):
     """Interface: forward(xn, ctx, residual) adds the result for the step's rows into `residual`."""
 
-    def forward(self, xn: torch.Tensor, ctx, residual: torch.Tensor) -> None:
+    def fuses_norm(self, norm, ctx) -> bool:
+        """True if, for this step, it would rather be given the float32 residual rows and the norm part."""
+        return False
+
+    def forward(self, xn: torch.Tensor, ctx, residual: torch.Tensor, norm=None) -> None:
         raise NotImplementedError
 
 
@@ -44,7 +49,13 @@ class GatedFeedForward(FeedForward):
         self.w_gate_up = stored(inter, spec["gate_proj.weight"], device, dtype)
         self.w_down = stored(tensors["down_proj.weight"], spec["down_proj.weight"], device, dtype)
 
-    def forward(self, xn, ctx, residual) -> None:
-        hid = ctx.buffer("feed_forward.hidden", (xn.shape[0], self.inner), xn.dtype)
-        ops.gemm(self.w_gate_up, xn, hid, ops.EPI_SWIGLU)
+    def fuses_norm(self, norm, ctx) -> bool:
+        return isinstance(norm, RMSNorm) and ctx.n_tokens <= ops.FUSED_NORM_ROWS
+
+    def forward(self, xn, ctx, residual, norm=None) -> None:
+        hid = ctx.buffer("feed_forward.hidden", (xn.shape[0], self.inner), ctx.dtype)
+        if norm is not None:      # xn are the float32 residual rows: the norm rides in the product
+            ops.gemm_rmsnorm(self.w_gate_up, xn, norm.weight, norm.eps, hid, ops.EPI_SWIGLU)
+        else:
+            ops.gemm(self.w_gate_up, xn, hid, ops.EPI_SWIGLU)
         ops.gemm(self.w_down, hid, residual, ops.EPI_ACCUM_F32)

@@ -105,6 +105,8 @@ class DecoderModel:
 
     def logits(self, ctx, x: torch.Tensor, rows: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
         """Final norm and output head on the wanted rows of x (all rows if `rows` is None)."""
+        if rows is None and self.head.fuses_norm(self.final_norm, ctx):
+            return self.head(x, out, norm=self.final_norm)
         xn = ctx.buffer("model.head_in", (out.shape[0], self.width), ctx.dtype)
         self.final_norm(x, xn, rows)
         return self.head(xn, out)

@@ -74,12 +74,12 @@ GEMM_SHAPES = [(200, 37, 96), (130, 5, 40), (64, 1, 64), (388, 130, 352), (34, 8
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
-@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("n,t,k", GEMM_SHAPES)
 def test_gemm_store_and_accumulate(dtype, _, rel, kind, n, t, k):
     ops = _ops()
-    if kind == 1 and t > 8:
-        pytest.skip("the streaming kernel takes at most 8 rows")
+    if (kind == 1 and t > 8) or (kind == 5 and t > 64):
+        pytest.skip("the streaming kernels take a few rows only")
     if dtype == torch.bfloat16 and k % 8:
         pytest.skip("bfloat16 rows come in 16-byte pieces")
     g = torch.Generator().manual_seed(n * 1000 + t)
@@ -99,12 +99,12 @@ def test_gemm_store_and_accumulate(dtype, _, rel, kind, n, t, k):
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
-@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4])
-@pytest.mark.parametrize("f,t,k", [(160, 5, 64), (352, 70, 128), (9, 2, 16), (1030, 200, 72)])
+@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("f,t,k", [(160, 5, 64), (352, 70, 128), (9, 2, 16), (1030, 200, 72), (40, 33, 2056), (8200, 64, 256)])
 def test_gemm_swiglu(dtype, _, rel, kind, f, t, k):
     ops = _ops()
-    if kind == 1 and t > 8:
-        pytest.skip("the streaming kernel takes at most 8 rows")
+    if (kind == 1 and t > 8) or (kind == 5 and t > 64):
+        pytest.skip("the streaming kernels take a few rows only")
     g = torch.Generator().manual_seed(f + t)
     gate = torch.randn(f, k, generator=g).to(dtype)
     up = torch.randn(f, k, generator=g).to(dtype)
@@ -115,6 +115,36 @@ def test_gemm_swiglu(dtype, _, rel, kind, f, t, k):
     gd, ud = x.double().cpu() @ gate.double().T, x.double().cpu() @ up.double().T
     want = gd / (1 + torch.exp(-gd)) * ud
     close(out, want, rel, f"swiglu kind={kind}")
+
+
+@pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("n,t,k", [(200, 8, 96), (130, 1, 40), (96, 17, 2048), (388, 64, 352), (34, 48, 160)])
+def test_gemm_with_fused_rmsnorm(dtype, _, rel, n, t, k):
+    """The product with the normed rows that are never written, in every epilogue."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(n + t)
+    w = (0.5 * torch.randn(n, k, generator=g)).to(dtype).to(DEV)
+    x = (2 * torch.randn(t, k, generator=g)).to(DEV)
+    nw = (1 + 0.3 * torch.randn(k, generator=g)).to(DEV)
+    eps = 1e-2
+    xd = x.double()
+    xn = xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + eps) * nw.double()
+    want = xn @ w.double().T
+    tol = 1e-5 if dtype == torch.float32 else 1.5e-2
+    out = torch.empty(t, n, dtype=dtype, device=DEV)
+    ops.gemm_rmsnorm(w, x, nw, eps, out)
+    close(out, want, tol, "store")
+    out32 = torch.empty(t, n, device=DEV)
+    ops.gemm_rmsnorm(w, x, nw, eps, out32, ops.EPI_STORE_F32)
+    close(out32, want, tol, "store f32")
+    res = torch.randn(t, n, generator=g).to(DEV)
+    res0 = res.clone()
+    ops.gemm_rmsnorm(w, x, nw, eps, res, ops.EPI_ACCUM_F32)
+    close(res, res0.double() + want, tol, "accumulate")
+    hid = torch.empty(t, n // 2, dtype=dtype, device=DEV)
+    ops.gemm_rmsnorm(w, x, nw, eps, hid, ops.EPI_SWIGLU)
+    gd, ud = want[:, 0::2], want[:, 1::2]
+    close(hid, gd / (1 + torch.exp(-gd)) * ud, tol * 2, "swiglu")
 
 
 def test_gemm_reference_vectors():
