@@ -24,11 +24,12 @@
 //                        transposed (keys x rows) so that each lane owns one query
 //                        row: softmax statistics stay in the lane and the
 //                        probabilities feed the second MFMA without a shuffle.
-//   attn_decode_kernel   bfloat16; one token per sequence: a wave takes a few
+//   attn_decode_kernel   bfloat16; one token per sequence: the waves of a block take the
 //                        pages of one (sequence, KV head), all heads of the group
-//                        at once as the MFMA's 16 columns, and writes a partial
-//                        (max, sum, weighted values); attn_combine_kernel merges
-//                        the partials in page order.
+//                        at once as the MFMA's 16 columns,
+//                        in turn; the waves of a block are merged through LDS, and
+//                        blocks, when a long sequence is split over several, by
+//                        attn_combine_kernel, always in page order.
 #include "common.h"
 
 #ifndef HEAD_DIM
@@ -343,29 +344,38 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
     }
 }
 
-// Decode: one token per sequence.  grid (splits, kv heads x head blocks of 16, sequences), one wave per block.
-// A wave takes pages [split * ppw, (split+1) * ppw) of its sequence and writes one partial per head:
-// part[((seq * H + head) * n_splits + split) * (HD + 4)] = weighted values [HD], max, sum (base-2 exponents), 2 unused.
-__global__ __launch_bounds__(WAVE) void attn_decode_kernel(
-    const bf16_t* __restrict__ q, int ldq, float* __restrict__ part, const int32_t* __restrict__ positions,
-    const int32_t* __restrict__ slots, const int32_t* __restrict__ page_table, int max_pages,
-    const bf16_t* __restrict__ cache, long long page_stride, long long v_off, int n_heads, int group, int head_blocks, int ppw,
-    int n_splits, int window, float scale_log2e) {
+// Decode: one token per sequence.  grid (splits, kv heads x head blocks of 16, sequences), NWV waves per block.
+// The pages that hold keys of a sequence's token are dealt evenly to the splits; a block's waves take its pages
+// in turn (wave w: the first page + w, + NWV, ...), all heads of the group at once as the MFMA's 16 columns, and are merged
+// through LDS in wave order.  With one split the block writes the finished rows; else it writes a partial per
+// head, part[((seq * H + head) * n_splits + split) * (HD + 4)] = weighted values [HD], max, sum (base-2
+// exponents), 2 unused, and attn_combine_kernel merges the partials in page order.
+template <int NWV>
+__global__ __launch_bounds__(NWV* WAVE) void attn_decode_kernel(
+    const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, float* __restrict__ part,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, const int32_t* __restrict__ page_table,
+    int max_pages, const bf16_t* __restrict__ cache, long long page_stride, long long v_off, int n_heads, int group,
+    int head_blocks, int n_splits, int window, float scale_log2e) {
   constexpr int HD = HEAD_DIM;
   constexpr int KS = (HD + 31) / 32;   // k steps of K Q^T (16x16x32)
   constexpr int DT = HD / 16;          // 16-row tiles of the output's head dimension
+  constexpr int LS = HD + 2;           // floats a wave leaves in LDS per head: values, max, sum
+  extern __shared__ float lds[];
   const int split = blockIdx.x, seq = blockIdx.z;
   const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
   const int pos = positions[seq];
   const int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
-  int pg0 = split * ppw, pg1 = pg0 + ppw - 1;
-  if (pg0 < lo / PAGE) pg0 = lo / PAGE;
-  if (pg1 > pos / PAGE) pg1 = pos / PAGE;
-  if (pg0 > pg1) return;
+  // the pages that hold keys of this token are dealt evenly to the splits
+  const int first_pg = lo / PAGE, last_pg = pos / PAGE;
+  const int span = (last_pg - first_pg + n_splits) / n_splits;
+  const int pg0 = first_pg + split * span;
+  const int pg1 = pg0 + span - 1 < last_pg ? pg0 + span - 1 : last_pg;
+  if (pg0 > pg1) return;               // the whole block: fewer pages than splits
   const int slot = slots[seq];
-  const int lane = threadIdx.x, j = lane & 15, G = lane >> 4;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, j = lane & 15, G = lane >> 4;
   const int hig = hb * 16 + j;                    // head within the group
-  const bool head_ok = hig < group;
+  const int heads_here = group - hb * 16 < 16 ? group - hb * 16 : 16;
+  const bool head_ok = j < heads_here;
   const int head = kvh * group + hig;
 
   uint4 qf[KS];
@@ -380,7 +390,7 @@ __global__ __launch_bounds__(WAVE) void attn_decode_kernel(
   for (int d = 0; d < DT; ++d) o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
 
-  for (int pg = pg0; pg <= pg1; ++pg) {
+  for (int pg = pg0 + wave; pg <= pg1; pg += NWV) {
     const int page = page_table[(size_t)slot * max_pages + pg];
     if (page < 0) continue;
     const bf16_t* kpage = cache + (size_t)page * page_stride + (size_t)kvh * PAGE * HD;
@@ -472,38 +482,79 @@ __global__ __launch_bounds__(WAVE) void attn_decode_kernel(
       }
     }
   }
-  if (!head_ok) return;
-  float* dst = part + ((size_t)(seq * n_heads + head) * n_splits + split) * (HD + 4);
+  // each wave leaves (values, max, sum) per head in LDS; a wave that saw no page leaves (0, -inf, 0)
+  if (head_ok) {
+    float* dst = lds + (size_t)(wave * heads_here + j) * LS;
 #pragma unroll
-  for (int d = 0; d < DT; ++d) *(float4*)(dst + d * 16 + 4 * G) = make_float4(o[d][0], o[d][1], o[d][2], o[d][3]);
-  if (G == 0) {
-    dst[HD] = m;
-    dst[HD + 1] = l;
+    for (int d = 0; d < DT; ++d)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) dst[d * 16 + 4 * G + v] = o[d][v];
+    if (G == 0) {
+      dst[HD] = m;
+      dst[HD + 1] = l;
+    }
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < heads_here * HD; idx += NWV * WAVE) {
+    const int hh = idx / HD, d = idx - hh * HD;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NWV; ++w) M = fmaxf(M, lds[(size_t)(w * heads_here + hh) * LS + HD]);
+    float L = 0.f, acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < NWV; ++w) {
+      const float* src = lds + (size_t)(w * heads_here + hh) * LS;
+      const float wt = fast_exp2(src[HD] - M);
+      L = fmaf(wt, src[HD + 1], L);
+      acc = fmaf(wt, src[d], acc);
+    }
+    const int hd_ = kvh * group + hb * 16 + hh;
+    if (n_splits == 1) {
+      out[(size_t)seq * ldo + (size_t)hd_ * HD + d] = f32_to_bf16(acc / L);
+    } else {
+      float* dst = part + ((size_t)(seq * n_heads + hd_) * n_splits + split) * (HD + 4);
+      dst[d] = acc;
+      if (d == 0) {
+        dst[HD] = M;
+        dst[HD + 1] = L;
+      }
+    }
   }
 }
 
 // grid (sequences, heads); merges the partials of the splits that hold keys of the token, in page order.
 __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, int ldo,
-                                                            const int32_t* __restrict__ positions, int n_heads, int ppw,
+                                                            const int32_t* __restrict__ positions, int n_heads,
                                                             int n_splits, int window) {
   constexpr int HD = HEAD_DIM;
   constexpr int PS = HD + 4;
   const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
   const int pos = positions[seq];
   const int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
-  const int s0 = (lo / PAGE) / ppw, s1 = (pos / PAGE) / ppw;
+  const int n_pages = pos / PAGE - lo / PAGE + 1;
+  const int span = (n_pages - 1 + n_splits) / n_splits;
+  const int s0 = 0, s1 = (n_pages - 1) / span;         // the splits that were given pages
   const float* base = part + (size_t)(seq * n_heads + head) * n_splits * PS;
-  float M = -INFINITY;
-  for (int s = s0 + lane; s <= s1; s += WAVE) M = fmaxf(M, base[(size_t)s * PS + HD]);
-  M = wave_max(M);
-  float L = 0.f;
-  for (int s = s0 + lane; s <= s1; s += WAVE) L += fast_exp2(base[(size_t)s * PS + HD] - M) * base[(size_t)s * PS + HD + 1];
-  L = wave_sum(L);
+  float M = -INFINITY, L = 0.f;
+  for (int c0 = s0; c0 <= s1; c0 += WAVE) {            // weights of up to 64 splits at a time, one per lane
+    const int sl = c0 + lane;
+    const float ms = sl <= s1 ? base[(size_t)sl * PS + HD] : -INFINITY;
+    const float ls = sl <= s1 ? base[(size_t)sl * PS + HD + 1] : 0.f;
+    const float M_new = fmaxf(M, wave_max(ms));
+    L = L * fast_exp2(M - M_new) + wave_sum(fast_exp2(ms - M_new) * ls);
+    M = M_new;
+  }
   const float inv = 1.0f / L;
-  for (int d = lane; d < HD; d += WAVE) {
+  for (int d0 = 0; d0 < HD; d0 += WAVE) {              // every lane stays in the loop: the shuffles need them all
+    const int d = d0 + lane < HD ? d0 + lane : HD - 1;
     float acc = 0.f;
-    for (int s = s0; s <= s1; ++s) acc = fmaf(fast_exp2(base[(size_t)s * PS + HD] - M), base[(size_t)s * PS + d], acc);
-    out[(size_t)seq * ldo + (size_t)head * HD + d] = f32_to_bf16(acc * inv);
+    for (int c0 = s0; c0 <= s1; c0 += WAVE) {
+      const int sl = c0 + lane;
+      const float w = sl <= s1 ? fast_exp2(base[(size_t)sl * PS + HD] - M) : 0.f;
+      const int n = s1 - c0 + 1 < WAVE ? s1 - c0 + 1 : WAVE;
+      for (int i = 0; i < n; ++i) acc = fmaf(__shfl(w, i, WAVE), base[(size_t)(c0 + i) * PS + d], acc);
+    }
+    if (d0 + lane < HD) out[(size_t)seq * ldo + (size_t)head * HD + d] = f32_to_bf16(acc * inv);
   }
 }
 
@@ -563,31 +614,68 @@ extern "C" const char* dlgo_attention_prefill(const void* q, int ldq, void* out,
   return nullptr;
 }
 
-// bfloat16, one row per sequence.  part: float32 scratch of n_seq * n_heads * n_splits * (hd + 4), n_splits =
-// ceil(max_pages_used / pages_per_wave), where max_pages_used bounds the pages of any sequence of the step.
+// bfloat16, one row per sequence.  max_pages_used bounds the pages of any sequence of the step (a recorded
+// launch passes the context's bound).  part: float32 scratch, used when the pages are split over several
+// blocks: n_seq * n_heads * n_splits * (hd + 4) with n_splits = dlgo_attention_decode_splits(...).
+static void decode_plan(int n_pairs, int group, int max_pages_used, int* nwv, int* n_splits) {
+  const int heads_here = group < 16 ? group : 16;
+  const int per_wave = heads_here * (HEAD_DIM + 2) * 4;      // bytes of LDS a wave needs for the merge
+  int w = 16;
+  while (w > 1 && w * per_wave > 60 * 1024) w >>= 1;
+  // enough blocks to fill the chip: with few (sequence, kv head) pairs each pair's pages go to several blocks
+  int splits = n_pairs >= 256 ? 1 : (256 + n_pairs - 1) / n_pairs;
+  if (splits > max_pages_used) splits = max_pages_used;
+  if (max_pages_used > w * 8 && splits < (max_pages_used + w * 8 - 1) / (w * 8)) splits = (max_pages_used + w * 8 - 1) / (w * 8);
+  if (splits > 1 && w > 8) w = 8;
+  *nwv = w;
+  *n_splits = splits;
+}
+
+extern "C" int dlgo_attention_decode_splits(int n_seq, int n_heads, int n_kv, int max_pages_used) {
+  int nwv, n_splits;
+  const int group = n_heads / n_kv;
+  decode_plan(n_seq * n_kv * ((group + 15) / 16), group, max_pages_used, &nwv, &n_splits);
+  return n_splits;
+}
+
 extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, int ldo, float* part, long long part_elems,
                                              int n_seq, int n_heads, int n_kv, int head_dim, const int32_t* positions,
                                              const int32_t* slots, const int32_t* page_table, int max_pages,
-                                             int max_pages_used, int pages_per_wave, const void* cache, long long page_stride,
-                                             long long v_off, int window, float scale, hipStream_t stream) {
+                                             int max_pages_used, const void* cache, long long page_stride, long long v_off,
+                                             int window, float scale, hipStream_t stream) {
   DLGO_REQUIRE(head_dim == HEAD_DIM, "attention: this library is built for head size %d, got %d", HEAD_DIM, head_dim);
+  DLGO_REQUIRE(HEAD_DIM <= 256, "attention: the split kernel takes head sizes up to 256");
   DLGO_REQUIRE(n_seq >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention: bad sizes");
-  DLGO_REQUIRE(pages_per_wave >= 1 && max_pages_used >= 1 && max_pages_used <= max_pages, "attention: bad split of the pages");
+  DLGO_REQUIRE(max_pages_used >= 1 && max_pages_used <= max_pages, "attention: bad bound on the pages of a sequence");
   DLGO_REQUIRE(ldq >= n_heads * head_dim && ldo >= n_heads * head_dim && ldq % 8 == 0, "attention: row strides");
-  DLGO_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)part & 15) == 0 && ((uintptr_t)cache & 15) == 0 && page_stride % 8 == 0 && v_off % 8 == 0,
+  DLGO_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)cache & 15) == 0 && page_stride % 8 == 0 && v_off % 8 == 0,
                "attention: operands must be 16-byte aligned");
   const int group = n_heads / n_kv;
   const int head_blocks = (group + 15) / 16;
-  const int n_splits = (max_pages_used + pages_per_wave - 1) / pages_per_wave;
-  DLGO_REQUIRE(part_elems >= (long long)n_seq * n_heads * n_splits * (HEAD_DIM + 4), "attention: scratch for partial results too small");
+  int nwv, n_splits;
+  decode_plan(n_seq * n_kv * head_blocks, group, max_pages_used, &nwv, &n_splits);
+  DLGO_REQUIRE(n_splits == 1 || (part && part_elems >= (long long)n_seq * n_heads * n_splits * (HEAD_DIM + 4)),
+               "attention: scratch for partial results too small");
   DLGO_REQUIRE((long long)n_kv * head_blocks <= 65535 && n_seq <= 65535 && n_heads <= 65535, "attention: grid too large");
   if (n_seq == 0) return nullptr;
-  hipLaunchKernelGGL(attn_decode_kernel, dim3(n_splits, n_kv * head_blocks, n_seq), dim3(WAVE), 0, stream, (const bf16_t*)q, ldq, part,
-                     positions, slots, page_table, max_pages, (const bf16_t*)cache, page_stride, v_off, n_heads, group, head_blocks,
-                     pages_per_wave, n_splits, window, scale * LOG2E);
+  const int heads_here = group < 16 ? group : 16;
+  const size_t smem = (size_t)nwv * heads_here * (HEAD_DIM + 2) * 4;
+  dim3 grid(n_splits, n_kv * head_blocks, n_seq);
+#define DECODE_GO(W_)                                                                                                          \
+  hipLaunchKernelGGL(attn_decode_kernel<W_>, grid, dim3(W_ * WAVE), smem, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo, part, \
+                     positions, slots, page_table, max_pages, (const bf16_t*)cache, page_stride, v_off, n_heads, group,      \
+                     head_blocks, n_splits, window, scale * LOG2E)
+  if (nwv == 16) DECODE_GO(16);
+  else if (nwv == 8) DECODE_GO(8);
+  else if (nwv == 4) DECODE_GO(4);
+  else if (nwv == 2) DECODE_GO(2);
+  else DECODE_GO(1);
+#undef DECODE_GO
   DLGO_LAUNCH_CHECK("attention_decode");
-  hipLaunchKernelGGL(attn_combine_kernel, dim3(n_seq, n_heads), dim3(WAVE), 0, stream, part, (bf16_t*)out, ldo, positions, n_heads,
-                     pages_per_wave, n_splits, window);
-  DLGO_LAUNCH_CHECK("attention_combine");
+  if (n_splits > 1) {
+    hipLaunchKernelGGL(attn_combine_kernel, dim3(n_seq, n_heads), dim3(WAVE), 0, stream, part, (bf16_t*)out, ldo, positions, n_heads,
+                       n_splits, window);
+    DLGO_LAUNCH_CHECK("attention_combine");
+  }
   return nullptr;
 }

@@ -316,14 +316,11 @@ template <> struct Mma16<float> {
   }
 };
 
-#define SKINNY_WAVES 8
-
-template <typename T, int TB, int EPI, bool NORM>
-__global__ __launch_bounds__(SKINNY_WAVES* WAVE) void skinny_kernel(const T* __restrict__ W, const void* __restrict__ Xv,
+template <typename T, int NW, int TB, int EPI, bool NORM>
+__global__ __launch_bounds__(NW* WAVE) void skinny_kernel(const T* __restrict__ W, const void* __restrict__ Xv,
                                                                      const float* __restrict__ norm_w, float eps,
                                                                      void* __restrict__ Y, int N, int Tn, int K, int ldw,
                                                                      int ldx, int ldy) {
-  constexpr int NW = SKINNY_WAVES;
   constexpr int EPC = 16 / sizeof(T);          // elements of a 16-byte operand
   constexpr int PIECE = 8 * EPC;               // elements of a 128-byte piece of a row
   __shared__ float red[NW][TB][16][17];
@@ -341,8 +338,11 @@ __global__ __launch_bounds__(SKINNY_WAVES* WAVE) void skinny_kernel(const T* __r
     ss[c] = 0.f;
   }
   const int pieces = (K + PIECE - 1) / PIECE;
-#pragma unroll 2
-  for (int p = wave; p < pieces; p += NW) {
+  // blocks start at different places of their rows, so that at any moment they ask different memory channels
+  const int rot = (int)((blockIdx.x * 7u) % (unsigned)pieces);
+#pragma unroll 4
+  for (int pi = wave; pi < pieces; pi += NW) {
+    const int p = pi + rot < pieces ? pi + rot : pi + rot - pieces;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {            // the two 64-byte halves of the piece
       const int k = p * PIECE + h * 4 * EPC + G * EPC;
@@ -410,17 +410,31 @@ __global__ __launch_bounds__(SKINNY_WAVES* WAVE) void skinny_kernel(const T* __r
   }
 }
 
-template <typename T, int EPI, bool NORM>
-static void launch_skinny(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K, int ldw,
-                          int ldx, int ldy, hipStream_t stream) {
-  dim3 g((N + 15) / 16), b(SKINNY_WAVES * WAVE);
+template <typename T, int NW, int EPI, bool NORM>
+static void launch_skinny_nw(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K, int ldw,
+                             int ldx, int ldy, hipStream_t stream) {
+  dim3 g((N + 15) / 16), b(NW * WAVE);
   const int tb = (Tn + 15) / 16;
-#define SKINNY_GO(TB_) hipLaunchKernelGGL((skinny_kernel<T, TB_, EPI, NORM>), g, b, 0, stream, (const T*)W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy)
+#define SKINNY_GO(TB_) hipLaunchKernelGGL((skinny_kernel<T, NW, TB_, EPI, NORM>), g, b, 0, stream, (const T*)W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy)
   if (tb <= 1) SKINNY_GO(1);
   else if (tb == 2) SKINNY_GO(2);
   else if (tb == 3) SKINNY_GO(3);
   else SKINNY_GO(4);
 #undef SKINNY_GO
+}
+
+// The number of waves that share a block's rows is a function of K alone, so the order of the sums does not
+// depend on the step.  force_nw (1, 2, 4, 8) is for tuning and tests.
+template <typename T, int EPI, bool NORM>
+static void launch_skinny(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K, int ldw,
+                          int ldx, int ldy, hipStream_t stream, int force_nw = 0) {
+  const int pieces = (K * (int)sizeof(T) + 127) / 128;
+  int nw = pieces >= 32 ? 8 : (pieces >= 16 ? 4 : (pieces >= 8 ? 2 : 1));
+  if (force_nw) nw = force_nw;
+  if (nw == 8) launch_skinny_nw<T, 8, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else if (nw == 4) launch_skinny_nw<T, 4, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else if (nw == 2) launch_skinny_nw<T, 2, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else launch_skinny_nw<T, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
 }
 
 // ----------------------------------------------------------------------------
@@ -448,7 +462,8 @@ static void launch_gemv(const void* W, const void* X, void* Y, int N, int Tn, in
 template <typename T, int EPI>
 static void dispatch(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy, int force,
                      hipStream_t stream) {
-  // force: 0 = choose, 1 = gemv, 2 = 128x128 tiles, 3 = 64x64, 4 = 32x32, 5 = 16 rows of W per block
+  // force: 0 = choose, 1 = gemv, 2 = 128x128 tiles, 3 = 64x64, 4 = 32x32, 5 = 16 rows of W per block,
+  // 6..9 = the same with 1, 2, 4, 8 waves per block
   int kind = force;
   if (kind == 0) {
     if (Tn <= 64) kind = 5;
@@ -459,7 +474,7 @@ static void dispatch(const void* W, const void* X, void* Y, int N, int Tn, int K
     }
   }
   if (kind == 1) launch_gemv<T, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
-  else if (kind == 5) launch_skinny<T, EPI, false>(W, X, nullptr, 0.f, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else if (kind >= 5) launch_skinny<T, EPI, false>(W, X, nullptr, 0.f, Y, N, Tn, K, ldw, ldx, ldy, stream, kind == 5 ? 0 : 1 << (kind - 6));
   else if (kind == 2) launch_tiled<T, 128, 128, 2, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   else if (kind == 3) launch_tiled<T, 64, 64, 2, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   else launch_tiled<T, 32, 32, 1, 1, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
@@ -489,9 +504,9 @@ extern "C" const char* dlgo_gemm(const void* W, const void* X, void* Y, int dtyp
   DLGO_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && ((uintptr_t)Y & 15) == 0, "gemm: operands must be 16-byte aligned");
   DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm: SwiGLU epilogue needs an even N and ldy >= N/2");
   DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm: ldy %d shorter than N %d", ldy, N);
-  DLGO_REQUIRE(force_kind >= 0 && force_kind <= 5, "gemm: unknown kernel choice %d", force_kind);
+  DLGO_REQUIRE(force_kind >= 0 && force_kind <= 9, "gemm: unknown kernel choice %d", force_kind);
   DLGO_REQUIRE(force_kind != 1 || Tn <= 8, "gemm: the streaming kernel takes at most 8 rows, got %d", Tn);
-  DLGO_REQUIRE(force_kind != 5 || Tn <= 64, "gemm: the 16-row kernel takes at most 64 rows of X, got %d", Tn);
+  DLGO_REQUIRE(force_kind < 5 || Tn <= 64, "gemm: the 16-row kernel takes at most 64 rows of X, got %d", Tn);
   if (Tn == 0) return nullptr;
   const char* err = dtype == DLGO_DTYPE_F32 ? by_epilogue<float>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, force_kind, stream)
                                             : by_epilogue<bf16_t>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, force_kind, stream);

@@ -63,11 +63,49 @@ __device__ float block_sum_f(float v, float* red) {
   return t;
 }
 
-__global__ __launch_bounds__(SAMP_THREADS) void argmax_kernel(const float* __restrict__ logits, int ld, int V,
-                                                              int32_t* __restrict__ out) {
-  __shared__ BestIdx red[SAMP_WAVES];
-  const BestIdx b = block_argmax(logits + (size_t)blockIdx.x * ld, V, red);
-  if (threadIdx.x == 0) out[blockIdx.x] = b.i < 0 ? 0 : b.i;
+// argmax in two stages, so that a few rows still fill the chip: ARGMAX_CHUNKS blocks per row each find the
+// best of their part of the row, then one wave per row picks among them (larger value, then smaller index).
+#define ARGMAX_CHUNKS 64
+#define ARGMAX_THREADS 256
+
+__global__ __launch_bounds__(ARGMAX_THREADS) void argmax_part_kernel(const float* __restrict__ logits, int ld, int V,
+                                                                     BestIdx* __restrict__ partial) {
+  __shared__ BestIdx red[ARGMAX_THREADS / WAVE];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const int per = (V + ARGMAX_CHUNKS - 1) / ARGMAX_CHUNKS;
+  const int b0 = chunk * per, b1 = b0 + per < V ? b0 + per : V;
+  const float* lg = logits + (size_t)row * ld;
+  BestIdx best = {-INFINITY, -1};
+  for (int i = b0 + threadIdx.x; i < b1; i += ARGMAX_THREADS) {
+    const float v = lg[i];
+    if (v == v) best = better(best, BestIdx{v, i});
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    BestIdx other;
+    other.v = __shfl_xor(best.v, o, WAVE);
+    other.i = __shfl_xor(best.i, o, WAVE);
+    best = better(best, other);
+  }
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = best;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    BestIdx r = red[0];
+    for (int w = 1; w < ARGMAX_THREADS / WAVE; ++w) r = better(r, red[w]);
+    partial[(size_t)row * ARGMAX_CHUNKS + chunk] = r;
+  }
+}
+
+__global__ __launch_bounds__(WAVE) void argmax_final_kernel(const BestIdx* __restrict__ partial, int32_t* __restrict__ out) {
+  BestIdx best = partial[(size_t)blockIdx.x * ARGMAX_CHUNKS + threadIdx.x];
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    BestIdx other;
+    other.v = __shfl_xor(best.v, o, WAVE);
+    other.i = __shfl_xor(best.i, o, WAVE);
+    best = better(best, other);
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = best.i < 0 ? 0 : best.i;
 }
 
 // Largest key tau with measure({i : key_i >= tau}) >= need, by bisection on the key's bits.
@@ -196,10 +234,17 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
   if (threadIdx.x == 0) out[row] = chosen >= 0 ? chosen : (top.i < 0 ? 0 : top.i);
 }
 
-extern "C" const char* dlgo_argmax(const float* logits, int ld, int n_rows, int V, int32_t* out, hipStream_t stream) {
+// partial: scratch of n_rows * 64 pairs (float, int32), 8 bytes each.
+extern "C" const char* dlgo_argmax(const float* logits, int ld, int n_rows, int V, void* partial, long long partial_bytes,
+                                   int32_t* out, hipStream_t stream) {
   DLGO_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "argmax: bad sizes rows=%d V=%d ld=%d", n_rows, V, ld);
+  DLGO_REQUIRE(n_rows <= 65535, "argmax: at most 65535 rows at a time");
+  DLGO_REQUIRE(partial && partial_bytes >= (long long)n_rows * ARGMAX_CHUNKS * (long long)sizeof(BestIdx), "argmax: scratch too small");
+  static_assert(ARGMAX_CHUNKS == WAVE, "the final stage reads one candidate per lane");
   if (n_rows == 0) return nullptr;
-  hipLaunchKernelGGL(argmax_kernel, dim3(n_rows), dim3(SAMP_THREADS), 0, stream, logits, ld, V, out);
+  hipLaunchKernelGGL(argmax_part_kernel, dim3(ARGMAX_CHUNKS, n_rows), dim3(ARGMAX_THREADS), 0, stream, logits, ld, V, (BestIdx*)partial);
+  DLGO_LAUNCH_CHECK("argmax");
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(n_rows), dim3(WAVE), 0, stream, (const BestIdx*)partial, out);
   DLGO_LAUNCH_CHECK("argmax");
   return nullptr;
 }

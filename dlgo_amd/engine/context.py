@@ -30,15 +30,15 @@ class Workspace:
             self._bufs[key] = buf
         return buf[:rows].view(rows, *shape[1:]) if len(shape) > 1 else buf[:rows, 0]
 
-    def flat(self, name: str, n: int, dtype: torch.dtype) -> torch.Tensor:
-        """A flat scratch buffer of at least n elements.  When a larger one is needed the old one is kept
-        alive, because a captured step may still point at it."""
+    def flat(self, name: str, n: int, dtype: torch.dtype, zero: bool = False) -> torch.Tensor:
+        """A flat scratch buffer of at least n elements (zero-filled when made, if asked).  When a larger one
+        is needed the old one is kept alive, because a captured step may still point at it."""
         key = ("flat:" + name, 0, dtype)
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < n:
             if buf is not None:
                 self._retired.append(buf)
-            buf = torch.empty(n, dtype=dtype, device=self.device)
+            buf = (torch.zeros if zero else torch.empty)(n, dtype=dtype, device=self.device)
             self._bufs[key] = buf
         return buf
 
@@ -80,5 +80,5 @@ class StepContext:
     def buffer(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
         return self.engine.workspace.get(name, shape, dtype)
 
-    def scratch(self, name: str, n: int, dtype: torch.dtype) -> torch.Tensor:
-        return self.engine.workspace.flat(name, n, dtype)
+    def scratch(self, name: str, n: int, dtype: torch.dtype, zero: bool = False) -> torch.Tensor:
+        return self.engine.workspace.flat(name, n, dtype, zero)

@@ -130,7 +130,10 @@ def ensure_built(variants: Iterable[Variant], force: bool = False, quiet: bool =
             final = os.path.join(out_dir, _file_name(module, defines))
             tmp = final + f".tmp{os.getpid()}"
             cmd = [hipcc, *FLAGS, *[f"-D{k}={v}" for k, v in defines], os.path.join(CSRC, module + ".hip"), "-o", tmp]
-            p = subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env, cwd=out_dir)
+            # the compiler's messages go to a file: a pipe that nobody reads while waiting would fill up and stall it
+            log_file = open(tmp + ".log", "w+b")
+            p = subprocess.Popen(cmd, stdout=log_file, stderr=subprocess.STDOUT, env=env, cwd=out_dir)
+            p.log_file = log_file
             running.append((p, module, defines, tmp, final))
         still = []
         for item in running:
@@ -138,7 +141,13 @@ def ensure_built(variants: Iterable[Variant], force: bool = False, quiet: bool =
             if p.poll() is None:
                 still.append(item)
                 continue
-            log = p.stdout.read().decode(errors="replace")
+            p.log_file.seek(0)
+            log = p.log_file.read().decode(errors="replace")
+            p.log_file.close()
+            try:
+                os.remove(tmp + ".log")
+            except OSError:
+                pass
             if p.returncode != 0 or not os.path.exists(tmp):
                 log = "\n".join(l for l in log.splitlines() if "not a recognized feature" not in l)
                 failures.append(f"{module} {dict(defines)}:\n{log}")

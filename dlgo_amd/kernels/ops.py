@@ -222,13 +222,13 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
               tok_seq: torch.Tensor, slots: torch.Tensor, page_table: torch.Tensor, cache: torch.Tensor, page_stride: int,
               v_off: int, q_lens: Sequence[int], start_pos: Sequence[int], window: int = 0,
               scale: Optional[float] = None, cu_q: Optional[torch.Tensor] = None,
-              start_pos_dev: Optional[torch.Tensor] = None, scratch=None, max_pages_used: Optional[int] = None,
-              kernel: str = "auto") -> torch.Tensor:
+              start_pos_dev: Optional[torch.Tensor] = None, scratch=None,
+              max_pages_used: Optional[int] = None, kernel: str = "auto") -> torch.Tensor:
     """Attention of a step's query rows over the cache, with the kernel chosen by the step's shape and dtype.
 
     q_lens, start_pos: per sequence, on the host (rows of the step, and the length before it).  cu_q and
     start_pos_dev are the same numbers on the device (built here if not given).  scratch(n) returns a
-    float32 buffer of at least n elements (decode partials).  max_pages_used bounds the pages any sequence
+    float32 buffer of at least n elements (partials of long sequences in decode).  max_pages_used bounds the pages any sequence
     of the step holds (default: from q_lens and start_pos; a captured step passes the context's bound).
     kernel: "auto", "rows", "tiled" (prefill) or "split" (decode).  All kernels compute the same thing.
     """
@@ -263,15 +263,17 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
         if max_pages_used is None:
             max_pages_used = (int(max(start_pos)) + 1 + PAGE - 1) // PAGE
         max_pages_used = max(1, min(max_pages_used, max_pages))
-        ppw = decode_pages_per_wave(n_seq * n_kv * ((group + 15) // 16), max_pages_used)
-        n_splits = (max_pages_used + ppw - 1) // ppw
-        need = n_seq * n_heads * n_splits * (head_dim + 4)
-        part = scratch(need) if scratch is not None else torch.empty(need, dtype=torch.float32, device=q.device)
-        _need(part, "attention scratch", torch.float32, 1)
+        lib.dlgo_attention_decode_splits.restype = ctypes.c_int
+        n_splits = lib.dlgo_attention_decode_splits(n_seq, n_heads, n_kv, max_pages_used)
+        part = None
+        if n_splits > 1:
+            need = n_seq * n_heads * n_splits * (head_dim + 4)
+            part = scratch(need) if scratch is not None else torch.empty(need, dtype=torch.float32, device=q.device)
+            _need(part, "attention scratch", torch.float32, 1)
         _check(lib.dlgo_attention_decode(_ptr(q), _rows(q, "query rows"), _ptr(out), _rows(out, "attention output"), _ptr(part),
-                                         ctypes.c_longlong(part.numel()), n_seq, n_heads, n_kv, head_dim, _ptr(positions),
-                                         _ptr(slots), _ptr(page_table), max_pages, max_pages_used, ppw, _ptr(cache),
-                                         ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(window),
+                                         ctypes.c_longlong(part.numel() if part is not None else 0), n_seq, n_heads, n_kv,
+                                         head_dim, _ptr(positions), _ptr(slots), _ptr(page_table), max_pages, max_pages_used,
+                                         _ptr(cache), ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(window),
                                          ctypes.c_float(scale), _stream()))
         return out
     if kernel != "tiled":
@@ -292,18 +294,23 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
     return out
 
 
-def decode_pages_per_wave(n_pairs: int, max_pages: int) -> int:
-    """Pages of keys one wave of the split kernel takes: enough waves to fill the chip, few enough partials."""
-    return max(1, min(8, (n_pairs * max_pages) // 4096))
+_argmax_scratch: dict = {}
 
 
-def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+def argmax(logits: torch.Tensor, out: torch.Tensor, scratch: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out[r] = index of the first maximum of row r.  scratch: 512 bytes per row (kept here per device if not given)."""
     _need(logits, "logits", torch.float32, 2)
     _need(out, "argmax output", torch.int32, 1)
-    if out.shape[0] != logits.shape[0]:
+    n = logits.shape[0]
+    if out.shape[0] != n:
         raise KernelError("argmax: one output per row")
-    _check(_lib("sampling").dlgo_argmax(_ptr(logits), _rows(logits, "logits"), logits.shape[0], logits.shape[1], _ptr(out),
-                                        _stream()))
+    if scratch is None:
+        scratch = _argmax_scratch.get(logits.device)
+        if scratch is None or scratch.numel() < n * 512:
+            scratch = torch.empty(max(n, 256) * 512, dtype=torch.uint8, device=logits.device)
+            _argmax_scratch[logits.device] = scratch
+    _check(_lib("sampling").dlgo_argmax(_ptr(logits), _rows(logits, "logits"), n, logits.shape[1], _ptr(scratch),
+                                        ctypes.c_longlong(scratch.numel() * scratch.element_size()), _ptr(out), _stream()))
     return out
 
 

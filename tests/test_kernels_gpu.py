@@ -74,11 +74,11 @@ GEMM_SHAPES = [(200, 37, 96), (130, 5, 40), (64, 1, 64), (388, 130, 352), (34, 8
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
-@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9])
 @pytest.mark.parametrize("n,t,k", GEMM_SHAPES)
 def test_gemm_store_and_accumulate(dtype, _, rel, kind, n, t, k):
     ops = _ops()
-    if (kind == 1 and t > 8) or (kind == 5 and t > 64):
+    if (kind == 1 and t > 8) or (kind >= 5 and t > 64):
         pytest.skip("the streaming kernels take a few rows only")
     if dtype == torch.bfloat16 and k % 8:
         pytest.skip("bfloat16 rows come in 16-byte pieces")
@@ -291,6 +291,10 @@ ATT_CASES = [  # H, KV, hd, window, [(cached length, rows of this step)]
     (40, 2, 32, 0, [(200, 1), (77, 1)]),
     (6, 2, 48, 50, [(300, 1), (20, 1), (128, 1)]),
     (8, 8, 128, 0, [(150, 1)]),
+    # long sequences: the pages of one sequence are split over several blocks and merged by a second kernel
+    (4, 2, 16, 0, [(9000, 1), (70, 1)]),
+    (32, 2, 128, 0, [(2700, 1), (100, 1), (2049, 1)]),
+    (8, 8, 64, 300, [(9000, 1), (8500, 1)]),
     # groups that do not divide a tile
     (6, 2, 48, 0, [(100, 100), (31, 7)]),
     (40, 2, 32, 0, [(90, 90)]),

@@ -51,8 +51,8 @@ class _Ctx:
     def buffer(self, name, shape, dtype):
         return self.workspace.get(name, shape, dtype)
 
-    def scratch(self, name, n, dtype):
-        return self.workspace.flat(name, n, dtype)
+    def scratch(self, name, n, dtype, zero=False):
+        return self.workspace.flat(name, n, dtype, zero)
 
 
 def _rel(got, want):
