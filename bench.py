@@ -3,9 +3,9 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--dtype bf16|fp32]
 
-A step is one decode step of the whole batch: the step function on one token per
-sequence, greedy choice of the next tokens on the device, and their return to the
-host (what the generation loop does per step).  Random weights, seeded
+A step is one decode step of the whole batch: greedy choice of the next tokens on
+the device, the step function on those tokens, and the ids' return to the host
+(what the generation loop does per step, in its order).  Random weights, seeded
 uniform-random token ids, no stop tokens.  Prints ONE JSON line.
 
 Peaks used for the fractions (MI355X, published): HBM 8 TB/s; dense MFMA bf16
@@ -100,12 +100,14 @@ def main() -> int:
         prompts = [rng.integers(0, cfg.vocab_size, size=PROMPT).tolist() for _ in range(batch)]
         slots = eng.open(batch)
         logits = eng.step([Entry(s, p, [PROMPT - 1]) for s, p in zip(slots, prompts)])
-        toks = sampler.choose(logits, [greedy] * batch, [0.0] * batch)
+        # the generation loop's own order (engine/generate.py, _decode_ahead): choose on the device, queue the next
+        # step with the ids still on the device, then bring the ids of the step before to the host
+        state = {"logits": logits}
 
         def one():
-            nonlocal toks
-            lg = eng.step([Entry(s, [t], [0]) for s, t in zip(slots, toks)])
-            toks = sampler.choose(lg, [greedy] * batch, [0.0] * batch)
+            tok_dev, wait = sampler.choose_async(state["logits"], [greedy] * batch, [0.0] * batch)
+            state["logits"] = eng.decode(slots, tok_dev)
+            state["tokens"] = wait()
         for _ in range(warmup):
             one()
         torch.cuda.synchronize()

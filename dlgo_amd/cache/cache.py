@@ -243,6 +243,18 @@ class Cache:
                 g.table_host[slot, gone] = -1
                 g.dirty.add(slot)
 
+    @property
+    def has_windows(self) -> bool:
+        return any(g.spec.window is not None for g in self.groups)
+
+    def advance_many(self, slots: np.ndarray, n_tokens: int) -> None:
+        """advance() for several live slots at once."""
+        if self.has_windows:
+            for s in slots:
+                self.advance(int(s), n_tokens)
+        else:
+            self.lengths[slots] += n_tokens
+
     def sync_tables(self) -> None:
         """Bring the device page tables up to date (rows of slots that changed)."""
         for g in self.groups:

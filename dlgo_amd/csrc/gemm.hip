@@ -316,25 +316,27 @@ template <> struct Mma16<float> {
   }
 };
 
-template <typename T, int NW, int TB, int EPI, bool NORM>
+template <typename T, int NW, int R, int TB, int EPI, bool NORM>
 __global__ __launch_bounds__(NW* WAVE) void skinny_kernel(const T* __restrict__ W, const void* __restrict__ Xv,
-                                                                     const float* __restrict__ norm_w, float eps,
-                                                                     void* __restrict__ Y, int N, int Tn, int K, int ldw,
-                                                                     int ldx, int ldy) {
+                                                           const float* __restrict__ norm_w, float eps, void* __restrict__ Y,
+                                                           int N, int Tn, int K, int ldw, int ldx, int ldy) {
   constexpr int EPC = 16 / sizeof(T);          // elements of a 16-byte operand
   constexpr int PIECE = 8 * EPC;               // elements of a 128-byte piece of a row
-  __shared__ float red[NW][TB][16][17];
+  __shared__ float red[NW][16][17];
   __shared__ float ssq[NW][TB][16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = lane & 15, G = lane >> 4;
-  const int n0 = blockIdx.x * 16;
-  const T* wrow = W + (size_t)(n0 + j < N ? n0 + j : N - 1) * ldw;
+  const int n0 = blockIdx.x * 16 * R;          // R groups of 16 rows share every load of X
+  const T* wrow[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) wrow[r] = W + (size_t)(n0 + r * 16 + j < N ? n0 + r * 16 + j : N - 1) * ldw;
 
-  f32x4_t acc[TB];
+  f32x4_t acc[R][TB];
   float ss[TB];
 #pragma unroll
   for (int c = 0; c < TB; ++c) {
-    acc[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     ss[c] = 0.f;
   }
   const int pieces = (K + PIECE - 1) / PIECE;
@@ -347,7 +349,9 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_kernel(const T* __restrict__ 
     for (int h = 0; h < 2; ++h) {            // the two 64-byte halves of the piece
       const int k = p * PIECE + h * 4 * EPC + G * EPC;
       const bool in = k < K;
-      const uint4 a = in ? *(const uint4*)(wrow + k) : make_uint4(0, 0, 0, 0);
+      uint4 a[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) a[r] = in ? *(const uint4*)(wrow[r] + k) : make_uint4(0, 0, 0, 0);
 #pragma unroll
       for (int c = 0; c < TB; ++c) {
         const int t = c * 16 + j;
@@ -374,48 +378,68 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_kernel(const T* __restrict__ 
             b = *(const uint4*)((const T*)Xv + (size_t)t * ldx + k);
           }
         }
-        Mma16<T>::run(a, b, acc[c]);
+#pragma unroll
+        for (int r = 0; r < R; ++r) Mma16<T>::run(a[r], b, acc[r][c]);
       }
     }
   }
-  // lane: token = 16 c + j, rows 4 G + v.  Partial tiles go to LDS; wave 0 adds them in wave order.
+  // lane: token = 16 c + j, rows 16 r + 4 G + v.  Tile by tile the partial sums go to LDS and wave 0 adds them in
+  // wave order and runs the epilogue.
+  float scale[TB];
+  if (NORM) {
 #pragma unroll
-  for (int c = 0; c < TB; ++c) {
-#pragma unroll
-    for (int v = 0; v < 4; ++v) red[wave][c][4 * G + v][j] = acc[c][v];
-    if (NORM) {
+    for (int c = 0; c < TB; ++c) {
       float s = ss[c];
       s += __shfl_xor(s, 16, WAVE);
       s += __shfl_xor(s, 32, WAVE);
       if (G == 0) ssq[wave][c][j] = s;
     }
-  }
-  __syncthreads();
-  if (wave != 0) return;
+    __syncthreads();
 #pragma unroll
-  for (int c = 0; c < TB; ++c) {
-    const int t = c * 16 + j;
-    float v[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int w = 0; w < NW; ++w)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) v[r] += red[w][c][4 * G + r][j];
-    if (NORM) {
+    for (int c = 0; c < TB; ++c) {
       float s = 0.f;
       for (int w = 0; w < NW; ++w) s += ssq[w][c][j];
-      const float scale = 1.0f / sqrtf(s / (float)K + eps);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) v[r] *= scale;
+      scale[c] = 1.0f / sqrtf(s / (float)K + eps);
     }
-    if (t < Tn) epilogue4<T, EPI>(Y, ldy, N, t, n0 + 4 * G, v[0], v[1], v[2], v[3]);
   }
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int c = 0; c < TB; ++c) {
+      if (NW > 1) {
+        if (r + c) __syncthreads();          // wave 0 has read the tile before
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave][4 * G + v][j] = acc[r][c][v];
+        __syncthreads();
+      }
+      if (wave == 0) {
+        float v[4];
+        if (NW > 1) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] = 0.f;
+          for (int w = 0; w < NW; ++w)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] += red[w][4 * G + q][j];
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] = acc[r][c][q];
+        }
+        if (NORM) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] *= scale[c];
+        }
+        const int t = c * 16 + j;
+        if (t < Tn) epilogue4<T, EPI>(Y, ldy, N, t, n0 + r * 16 + 4 * G, v[0], v[1], v[2], v[3]);
+      }
+    }
 }
 
-template <typename T, int NW, int EPI, bool NORM>
+template <typename T, int NW, int R, int EPI, bool NORM>
 static void launch_skinny_nw(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K, int ldw,
                              int ldx, int ldy, hipStream_t stream) {
-  dim3 g((N + 15) / 16), b(NW * WAVE);
+  dim3 g((N + 16 * R - 1) / (16 * R)), b(NW * WAVE);
   const int tb = (Tn + 15) / 16;
-#define SKINNY_GO(TB_) hipLaunchKernelGGL((skinny_kernel<T, NW, TB_, EPI, NORM>), g, b, 0, stream, (const T*)W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy)
+#define SKINNY_GO(TB_) hipLaunchKernelGGL((skinny_kernel<T, NW, R, TB_, EPI, NORM>), g, b, 0, stream, (const T*)W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy)
   if (tb <= 1) SKINNY_GO(1);
   else if (tb == 2) SKINNY_GO(2);
   else if (tb == 3) SKINNY_GO(3);
@@ -431,10 +455,14 @@ static void launch_skinny(const void* W, const void* X, const float* norm_w, flo
   const int pieces = (K * (int)sizeof(T) + 127) / 128;
   int nw = pieces >= 32 ? 8 : (pieces >= 16 ? 4 : (pieces >= 8 ? 2 : 1));
   if (force_nw) nw = force_nw;
-  if (nw == 8) launch_skinny_nw<T, 8, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
-  else if (nw == 4) launch_skinny_nw<T, 4, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
-  else if (nw == 2) launch_skinny_nw<T, 2, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
-  else launch_skinny_nw<T, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  // many rows: each block takes 2 or 4 groups of 16, which divides the traffic of X (a function of N alone)
+  const bool wide = N >= 32768 && nw == 8, mid = N >= 8192 && nw == 8;
+  if (wide) launch_skinny_nw<T, 8, 4, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else if (mid) launch_skinny_nw<T, 8, 2, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else if (nw == 8) launch_skinny_nw<T, 8, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else if (nw == 4) launch_skinny_nw<T, 4, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else if (nw == 2) launch_skinny_nw<T, 2, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else launch_skinny_nw<T, 1, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
 }
 
 // ----------------------------------------------------------------------------

@@ -219,9 +219,10 @@ class Engine:
             raise EngineError(f"step: {why}")
         self.steps_run += 1
 
-        if (self.use_graphs and sink is None and len(entries) <= self.graph_max_batch
+        if (sink is None and len(entries) <= self.graph_max_batch
                 and all(n == 1 for n in q_lens) and all(list(e.want) == [0] for e in entries)):
-            return self._decode_step(entries, tokens, starts)
+            self.steps_run -= 1
+            return self.decode([e.slot for e in entries], tokens, checked=True)
 
         # wanted rows: (output row, flat row), in output order
         cu = np.concatenate([[0], np.cumsum(q_lens)])
@@ -299,36 +300,62 @@ class Engine:
             "cu_q": np.arange(b + 1, dtype=np.int32),
         }
 
-    def _decode_step(self, entries: Sequence[Entry], tokens: np.ndarray, starts: Sequence[int]) -> torch.Tensor:
-        b = len(entries)
-        slots = [e.slot for e in entries]
-        self.cache.reserve([(s, st + 1) for s, st in zip(slots, starts)])
-        self.cache.sync_tables()
+    def decode(self, slots: Sequence[int], tokens, checked: bool = False) -> torch.Tensor:
+        """One token for each of `slots`, logits [len(slots), vocab] for each (a view that the next decode
+        overwrites).  `tokens` are ids on the host, or an int32 tensor on the device in the order of `slots`
+        (the sampler's output: the ids need not come to the host before the next step starts)."""
+        b = len(slots)
+        slot_arr = np.asarray(slots, dtype=np.int64)
+        on_device = isinstance(tokens, torch.Tensor)
+        if not checked:
+            if b < 1 or b > self.graph_max_batch:
+                raise EngineError(f"decode: between 1 and {self.graph_max_batch} sequences, got {b}")
+            if len(set(slots)) != b or slot_arr.min() < 0 or slot_arr.max() >= self.cache.max_slots \
+                    or not self.cache._live[slot_arr].all():
+                raise EngineError("decode: slots must be distinct and in use")
+            if on_device:
+                if tokens.dtype != torch.int32 or tokens.dim() != 1 or tokens.shape[0] != b or tokens.device != self.device:
+                    raise EngineError("decode: device tokens must be one int32 id per slot on the engine's device")
+            else:
+                tok = np.asarray(tokens, dtype=np.int64)
+                if tok.shape != (b,) or tok.min() < 0 or tok.max() >= self.vocab:
+                    raise EngineError(f"decode: one token id inside the vocabulary of {self.vocab} per slot")
+        starts = self.cache.lengths[slot_arr]
+        if not checked:
+            if (starts + 1 > self.max_ctx).any():
+                raise EngineError(f"decode: a sequence would exceed the context of {self.max_ctx}")
+        if (starts % PAGE == 0).any() or self.cache.has_windows:
+            wants = [(int(s), int(st) + 1) for s, st in zip(slot_arr, starts)]
+            if not checked:
+                why = self.cache.can_reserve(wants)
+                if why:
+                    raise EngineError(f"decode: {why}")
+            self.cache.reserve(wants)
+            self.cache.sync_tables()
         st = self._static_arrays()
-        # a fixed layout per batch size inside the static buffer: one copy brings all arrays
-        fields = self._decode_fields(tokens, starts, slots)
-        width = sum((len(v) + 3) // 4 * 4 for v in fields.values())
-        if st["meta"].numel() < width:
-            raise EngineError("decode step: static arrays too small")   # cannot happen: sized for graph_max_batch
+        tok_host = np.zeros(b, dtype=np.int32) if on_device else np.asarray(tokens, dtype=np.int32)
+        fields = self._decode_fields(tok_host, starts, slot_arr)
         arrays = self._upload(fields, dest=st["meta"])
+        if on_device:
+            arrays["token_ids"].copy_(tokens)
         logits = self._static_logits[:b]
-        g = self._graphs.get(b)
+        g = self._graphs.get(b) if self.use_graphs else None
         if g is not None:
             g.graph.replay()
         else:
-            host = {"q_lens": np.ones(b, dtype=np.int64), "start_pos": np.asarray(starts, dtype=np.int64),
-                    "slots": np.asarray(slots, dtype=np.int64)}
+            host = {"q_lens": np.ones(b, dtype=np.int64), "start_pos": starts.astype(np.int64), "slots": slot_arr}
             ctx = StepContext(self, b, b, arrays, host)
             ctx.is_decode = True
-            ctx.max_pages_used = self.cache.max_pages_per_seq     # the recorded launch must cover any later length
+            if self.use_graphs:
+                ctx.max_pages_used = self.cache.max_pages_per_seq     # the recorded launch must cover any later length
             x = self.model.hidden(ctx, ctx.token_ids)
             self.model.logits(ctx, x, None, logits)
             # the second time a batch size is seen it is worth capturing
             self._graph_seen[b] = self._graph_seen.get(b, 0) + 1
-            if self._graph_seen[b] >= 2:
+            if self.use_graphs and self._graph_seen[b] >= 2:
                 self._capture(b, ctx, logits)
-        for s in slots:
-            self.cache.advance(s, 1)
+        self.cache.advance_many(slot_arr, 1)
+        self.steps_run += 1
         return logits
 
     def _capture(self, b: int, ctx: StepContext, logits: torch.Tensor) -> None:

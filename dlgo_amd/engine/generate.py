@@ -14,6 +14,15 @@ slots the last one freed.  Results come back in request order.
 The loop decides with host data only and talks to the engine and the sampler
 through four calls (open, close, step, choose), so its decisions can be tested
 with stand-ins.
+
+When the engine takes token ids from the device (`decode`) and the sampler can
+hand them over without waiting (`choose_async`), the loop runs one step ahead:
+the step that feeds the tokens just chosen is queued before those tokens reach
+the host, so the GPU does not wait for the host's bookkeeping.  Whether a
+sequence goes on after a token is then known one step late: a sequence that
+turns out to have stopped has been given one step too many, whose result is
+dropped and whose slot is given back as before.  Choices that depend on the
+tokens generated so far (the repetition penalty) keep the simple order.
 """
 from __future__ import annotations
 
@@ -80,6 +89,60 @@ def plan_batch(prompt_lens: Sequence[int], max_new: Sequence[int], free_slots: i
     return n
 
 
+def _decode_ahead(engine, sampler, live, logits, prompts, results, stats, on_token) -> None:
+    """The decode loop of one batch, one step ahead of the host (see the module's text)."""
+    def finish(l, reason):
+        results[l.index] = Result(l.tokens, reason, len(prompts[l.index]))
+        engine.close([l.slot])
+
+    while live:
+        # before a token is chosen: who may not go on at all
+        keep = []
+        for row, l in enumerate(live):
+            if len(l.tokens) >= l.config.max_tokens:
+                finish(l, "length")
+            elif l.pos >= engine.max_ctx - 1:
+                finish(l, "context")
+            else:
+                keep.append(row)
+        if not keep:
+            return
+        if len(keep) != len(live):
+            logits = logits[keep]
+            live = [live[r] for r in keep]
+        tok_dev, wait = sampler.choose_async(logits, [l.config.sampler for l in live],
+                                             [uniform(l.seed, l.index, len(l.tokens)) for l in live], None)
+        # queue the next step for every sequence that wants another token after this one, before knowing the ids
+        fed = [row for row, l in enumerate(live) if len(l.tokens) + 1 < l.config.max_tokens]
+        next_logits = None
+        if fed:
+            ids = tok_dev if len(fed) == len(live) else tok_dev[fed]
+            next_logits = engine.decode([live[r].slot for r in fed], ids)
+            stats.steps += 1
+        chosen = wait()
+        still = []
+        for row, (l, tok) in enumerate(zip(live, chosen)):
+            tok = int(tok)
+            if tok in l.stop:
+                finish(l, "stop")         # if it was fed, that step's row is dropped
+                continue
+            l.tokens.append(tok)
+            stats.output_tokens += 1
+            if on_token is not None:
+                on_token(l.index, tok)
+            if len(l.tokens) >= l.config.max_tokens:
+                finish(l, "length")
+                continue
+            still.append(row)
+        if not still:
+            return
+        rows = [fed.index(r) for r in still]          # every row in `still` was fed
+        logits = next_logits if len(rows) == len(fed) else next_logits[rows]
+        live = [live[r] for r in still]
+        for l in live:
+            l.pos += 1
+
+
 def generate(engine, sampler, prompts: Sequence[Sequence[int]], configs: Sequence[GenerateConfig],
              default_stop: Sequence[int] = (), on_token: Optional[Callable[[int, int], None]] = None,
              max_batch: int = 64, sync: Optional[Callable[[], None]] = None):
@@ -123,6 +186,11 @@ def generate(engine, sampler, prompts: Sequence[Sequence[int]], configs: Sequenc
             stats.prefill_ms += (t1 - t0) * 1000.0
             stats.prompt_tokens += sum(len(prompts[l.index]) for l in live)
             stats.steps += 1
+            ahead = (hasattr(engine, "decode") and hasattr(sampler, "choose_async")
+                     and not sampler.needs_recent([l.config.sampler for l in live]))
+            if ahead:
+                _decode_ahead(engine, sampler, live, logits, prompts, results, stats, on_token)
+                live = []
             while live:
                 # sequences that may not go on leave before a token is chosen for them
                 keep_rows = []

@@ -19,6 +19,8 @@ class Sampler:
         self.device = torch.device(device)
         self.max_rows = max_rows
         self._out = torch.empty(max_rows, dtype=torch.int32, device=self.device)
+        self._pinned = [torch.empty(max_rows, dtype=torch.int32, pin_memory=True) for _ in range(4)]
+        self._pin_next = 0
         self._work: Optional[torch.Tensor] = None
         self._e: Optional[torch.Tensor] = None
 
@@ -30,6 +32,35 @@ class Sampler:
     def choose(self, logits: torch.Tensor, configs: Sequence[SamplerConfig], uniforms: Sequence[float],
                recent: Optional[Sequence[Sequence[int]]] = None) -> List[int]:
         """logits [rows, vocab] float32 on the device -> one token id per row (host list)."""
+        return self.choose_device(logits, configs, uniforms, recent).tolist()
+
+    def choose_async(self, logits: torch.Tensor, configs: Sequence[SamplerConfig], uniforms: Sequence[float],
+                     recent: Optional[Sequence[Sequence[int]]] = None):
+        """The ids as a device tensor (valid until the next call) and a function that waits for them and
+        returns them as a host list; work can be queued behind the choice before the ids are awaited."""
+        out = self.choose_device(logits, configs, uniforms, recent)
+        n = out.shape[0]
+        i = self._pin_next
+        self._pin_next = (i + 1) % len(self._pinned)
+        host = self._pinned[i]
+        if host.shape[0] < n:
+            host = self._pinned[i] = torch.empty(max(n, 2 * host.shape[0]), dtype=torch.int32, pin_memory=True)
+        host[:n].copy_(out, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+
+        def wait() -> List[int]:
+            event.synchronize()
+            return host[:n].tolist()
+        return out, wait
+
+    def needs_recent(self, configs: Sequence[SamplerConfig]) -> bool:
+        """True if a row's choice depends on the tokens generated so far (the repetition penalty)."""
+        return any(c.repetition_penalty > 1.0 and not c.greedy for c in configs)
+
+    def choose_device(self, logits: torch.Tensor, configs: Sequence[SamplerConfig], uniforms: Sequence[float],
+                      recent: Optional[Sequence[Sequence[int]]] = None) -> torch.Tensor:
+        """logits [rows, vocab] float32 on the device -> int32 ids on the device (overwritten by the next call)."""
         n = logits.shape[0]
         if n != len(configs) or n != len(uniforms):
             raise ValueError("sampler: one configuration and one uniform number per row")
@@ -37,7 +68,7 @@ class Sampler:
         out = self._out[:n]
         if all(c.greedy for c in configs):
             ops.argmax(logits, out)
-            return out.tolist()
+            return out
         if self._work is None:
             rows = self._out.shape[0]
             self._work = torch.empty((rows, self.vocab), dtype=torch.float32, device=self.device)
@@ -57,4 +88,4 @@ class Sampler:
                 r[i, :len(toks)] = toks
             rec = torch.from_numpy(r).to(self.device)
         ops.sample(logits, self._work, self._e, fd[0], kd, fd[1], fd[2], fd[3], rec, fd[4], out)
-        return out.tolist()
+        return out

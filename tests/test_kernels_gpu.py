@@ -70,7 +70,8 @@ def test_rmsnorm_reference_vectors():
     close(out, w.double()[None] / math.sqrt(1 + 1e-5), 1e-6)
 
 
-GEMM_SHAPES = [(200, 37, 96), (130, 5, 40), (64, 1, 64), (388, 130, 352), (34, 8, 160), (512, 257, 128), (6, 3, 8)]
+GEMM_SHAPES = [(200, 37, 96), (130, 5, 40), (64, 1, 64), (388, 130, 352), (34, 8, 160), (512, 257, 128), (6, 3, 8),
+               (32790, 20, 2048)]      # wide enough for the kernel that gives a block four groups of rows
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
@@ -100,7 +101,7 @@ def test_gemm_store_and_accumulate(dtype, _, rel, kind, n, t, k):
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
 @pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5])
-@pytest.mark.parametrize("f,t,k", [(160, 5, 64), (352, 70, 128), (9, 2, 16), (1030, 200, 72), (40, 33, 2056), (8200, 64, 256)])
+@pytest.mark.parametrize("f,t,k", [(160, 5, 64), (352, 70, 128), (9, 2, 16), (1030, 200, 72), (40, 33, 2056), (8200, 64, 256), (16401, 9, 2048)])
 def test_gemm_swiglu(dtype, _, rel, kind, f, t, k):
     ops = _ops()
     if (kind == 1 and t > 8) or (kind == 5 and t > 64):
@@ -118,7 +119,7 @@ def test_gemm_swiglu(dtype, _, rel, kind, f, t, k):
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
-@pytest.mark.parametrize("n,t,k", [(200, 8, 96), (130, 1, 40), (96, 17, 2048), (388, 64, 352), (34, 48, 160)])
+@pytest.mark.parametrize("n,t,k", [(200, 8, 96), (130, 1, 40), (96, 17, 2048), (388, 64, 352), (34, 48, 160), (32780, 3, 2048)])
 def test_gemm_with_fused_rmsnorm(dtype, _, rel, n, t, k):
     """The product with the normed rows that are never written, in every epilogue."""
     ops = _ops()
