@@ -1,0 +1,59 @@
+// Shared by the two files of matrix products: the epilogues.
+//   store in the run dtype; add into the float32 residual stream; SwiGLU of interleaved gate/up rows
+//   (out[t, f] = silu(y[2f]) * y[2f+1], computerex/dlgo ops/activation.go:8-19,36-38); store float32 (logits).
+#pragma once
+#include "common.h"
+
+enum { EPI_STORE = 0, EPI_ACCUM_F32 = 1, EPI_SWIGLU = 2, EPI_STORE_F32 = 3 };
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
+
+// Four consecutive outputs n..n+3 of token t.
+template <typename T, int EPI>
+__device__ __forceinline__ void epilogue4(void* __restrict__ Y, int ldy, int N, int t, int n, float v0, float v1, float v2,
+                                          float v3) {
+  if (n >= N) return;
+  const bool full = n + 3 < N;
+  if (EPI == EPI_STORE) {
+    T* y = (T*)Y + (size_t)t * ldy + n;
+    if (full && (ldy & 3) == 0) {
+      if (sizeof(T) == 4) {
+        *(float4*)y = make_float4(v0, v1, v2, v3);
+      } else {
+        uint2 p;
+        p.x = (uint32_t)f32_to_bf16(v0) | ((uint32_t)f32_to_bf16(v1) << 16);
+        p.y = (uint32_t)f32_to_bf16(v2) | ((uint32_t)f32_to_bf16(v3) << 16);
+        *(uint2*)y = p;
+      }
+    } else {
+      const float v[4] = {v0, v1, v2, v3};
+      for (int r = 0; r < 4 && n + r < N; ++r) Elem<T>::store(y + r, v[r]);
+    }
+  } else if (EPI == EPI_ACCUM_F32 || EPI == EPI_STORE_F32) {
+    float* y = (float*)Y + (size_t)t * ldy + n;
+    if (full && (ldy & 3) == 0) {
+      float4 o = make_float4(v0, v1, v2, v3);
+      if (EPI == EPI_ACCUM_F32) {
+        const float4 old = *(float4*)y;
+        o.x += old.x;
+        o.y += old.y;
+        o.z += old.z;
+        o.w += old.w;
+      }
+      *(float4*)y = o;
+    } else {
+      const float v[4] = {v0, v1, v2, v3};
+      for (int r = 0; r < 4 && n + r < N; ++r) y[r] = (EPI == EPI_ACCUM_F32 ? y[r] : 0.f) + v[r];
+    }
+  } else {   // EPI_SWIGLU: rows (n, n+1) and (n+2, n+3) are (gate, up) pairs; N is even
+    T* y = (T*)Y + (size_t)t * ldy + (n >> 1);
+    if (n + 3 < N && (ldy & 1) == 0) {     // both halves at once
+      if (sizeof(T) == 4) *(float2*)y = make_float2(silu_f(v0) * v1, silu_f(v2) * v3);
+      else *(uint32_t*)y = (uint32_t)f32_to_bf16(silu_f(v0) * v1) | ((uint32_t)f32_to_bf16(silu_f(v2) * v3) << 16);
+    } else {
+      Elem<T>::store(y, silu_f(v0) * v1);
+      if (n + 3 < N) Elem<T>::store(y + 1, silu_f(v2) * v3);
+    }
+  }
+}
+

@@ -1,0 +1,374 @@
+// Matrix products for a few rows of X (decode): Y[t, n] = sum_k X[t, k] * W[n, k] with up to 64 tokens t, where the
+// time goes to streaming W once.  computerex/dlgo's mat-vec shader gives 4 rows of W to a workgroup and splits k over
+// lanes (gpu/shaders/matvec_f32.comp:17-47); here:
+//
+//  * skinny_kernel: 16 (or 32, 64) rows of W per block, k split over the block's waves, 16x16 MFMA with W as the
+//    row operand and the tokens as the column operand (bfloat16: v_mfma_f32_16x16x32_bf16; float32:
+//    v_mfma_f32_16x16x4_f32, a true float32 product).  Optionally the RMSNorm of the float32 residual rows rides in
+//    the product, so that the normed rows are never written.
+//  * gemv_kernel: up to 8 tokens on the vector units; a wave streams whole rows of W.
+//
+// Every reduction order is a function of N and K alone: a row of Y never depends on the other rows of the step.
+#include "gemm_common.h"
+
+// ----------------------------------------------------------------------------
+// weight-streaming kernel for up to 8 tokens
+// ----------------------------------------------------------------------------
+template <typename T> struct Chunk;
+template <> struct Chunk<bf16_t> {
+  static constexpr int E = 8;
+  static __device__ __forceinline__ void unpack(const uint4& u, float* f) {
+    f[0] = __uint_as_float(u.x << 16);
+    f[1] = __uint_as_float(u.x & 0xffff0000u);
+    f[2] = __uint_as_float(u.y << 16);
+    f[3] = __uint_as_float(u.y & 0xffff0000u);
+    f[4] = __uint_as_float(u.z << 16);
+    f[5] = __uint_as_float(u.z & 0xffff0000u);
+    f[6] = __uint_as_float(u.w << 16);
+    f[7] = __uint_as_float(u.w & 0xffff0000u);
+  }
+};
+template <> struct Chunk<float> {
+  static constexpr int E = 4;
+  static __device__ __forceinline__ void unpack(const uint4& u, float* f) {
+    f[0] = __uint_as_float(u.x);
+    f[1] = __uint_as_float(u.y);
+    f[2] = __uint_as_float(u.z);
+    f[3] = __uint_as_float(u.w);
+  }
+};
+
+#define GEMV_WAVES 4
+#define GEMV_ROWS 4   // rows of W per wave: two gate/up pairs
+
+template <typename T, int TM, int EPI>
+__global__ __launch_bounds__(GEMV_WAVES* WAVE) void gemv_kernel(const T* __restrict__ W, const T* __restrict__ X,
+                                                                 void* __restrict__ Y, int N, int Tn, int K, int ldw, int ldx,
+                                                                 int ldy) {
+  constexpr int E = Chunk<T>::E;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n0 = (blockIdx.x * GEMV_WAVES + wave) * GEMV_ROWS;
+  if (n0 >= N) return;
+  const T* wrow[GEMV_ROWS];
+#pragma unroll
+  for (int r = 0; r < GEMV_ROWS; ++r) wrow[r] = W + (size_t)(n0 + r < N ? n0 + r : N - 1) * ldw;
+  const T* xrow[TM];
+#pragma unroll
+  for (int m = 0; m < TM; ++m) xrow[m] = X + (size_t)(m < Tn ? m : Tn - 1) * ldx;
+
+  float acc[GEMV_ROWS][TM];
+#pragma unroll
+  for (int r = 0; r < GEMV_ROWS; ++r)
+#pragma unroll
+    for (int m = 0; m < TM; ++m) acc[r][m] = 0.f;
+
+  const int chunks = K / E;
+  for (int c = lane; c < chunks; c += WAVE) {
+    uint4 wv[GEMV_ROWS];
+#pragma unroll
+    for (int r = 0; r < GEMV_ROWS; ++r) wv[r] = *(const uint4*)(wrow[r] + (size_t)c * E);
+    float xf[TM][E];
+#pragma unroll
+    for (int m = 0; m < TM; ++m) {
+      const uint4 xv = *(const uint4*)(xrow[m] + (size_t)c * E);
+      Chunk<T>::unpack(xv, xf[m]);
+    }
+#pragma unroll
+    for (int r = 0; r < GEMV_ROWS; ++r) {
+      float wf[E];
+      Chunk<T>::unpack(wv[r], wf);
+#pragma unroll
+      for (int m = 0; m < TM; ++m)
+#pragma unroll
+        for (int e = 0; e < E; ++e) acc[r][m] = fmaf(wf[e], xf[m][e], acc[r][m]);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < GEMV_ROWS; ++r)
+#pragma unroll
+    for (int m = 0; m < TM; ++m) acc[r][m] = wave_sum(acc[r][m]);
+  // lane m writes token m
+#pragma unroll
+  for (int m = 0; m < TM; ++m)
+    if (lane == m && m < Tn) epilogue4<T, EPI>(Y, ldy, N, m, n0, acc[0][m], acc[1][m], acc[2][m], acc[3][m]);
+}
+
+// ----------------------------------------------------------------------------
+// MFMA kernel for a few rows of X (decode): 16 rows of W per block, k split over the waves
+// ----------------------------------------------------------------------------
+// A block owns 16 consecutive rows of W and every token of the step (up to 16 * TB).  Its NW waves take
+// the 128-byte pieces of those rows in turn (wave w: pieces w, w + NW, ...), so together they stream the
+// rows front to back; each piece is two 16x16 MFMA steps with W as the row operand and X as the column
+// operand.  The waves' partial tiles are summed through LDS in wave order, then wave 0 runs the epilogue:
+// a lane holds four consecutive n of one token, as in the tiled kernel.
+//
+// NORM: X is the float32 residual stream and the product is taken with rmsnorm(X) * norm_w without
+// writing the normed rows: the column operand is X[t,k] * norm_w[k], the sum of squares of each token is
+// gathered on the way, and 1/sqrt(mean + eps) multiplies the finished sums (it is a scalar per token).
+template <typename T> struct Mma16;
+template <> struct Mma16<bf16_t> {
+  static __device__ __forceinline__ void run(const uint4& a, const uint4& b, f32x4_t& c) {
+    union { uint4 u; bf16x8_t v; } ua, ub;
+    ua.u = a;
+    ub.u = b;
+    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ua.v, ub.v, c, 0, 0, 0);
+  }
+  // 8 floats -> one 16-byte operand
+  static __device__ __forceinline__ uint4 pack(const float* f) {
+    union { uint4 u; bf16x8_t v; } x;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x.v[e] = (__bf16)f[e];
+    return x.u;
+  }
+};
+template <> struct Mma16<float> {
+  static __device__ __forceinline__ void run(const uint4& a, const uint4& b, f32x4_t& c) {
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint4 pack(const float* f) {
+    return make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3]));
+  }
+};
+
+template <typename T, int NW, int R, int TB, int EPI, bool NORM>
+__global__ __launch_bounds__(NW* WAVE) void skinny_kernel(const T* __restrict__ W, const void* __restrict__ Xv,
+                                                           const float* __restrict__ norm_w, float eps, void* __restrict__ Y,
+                                                           int N, int Tn, int K, int ldw, int ldx, int ldy) {
+  constexpr int EPC = 16 / sizeof(T);          // elements of a 16-byte operand
+  constexpr int PIECE = 8 * EPC;               // elements of a 128-byte piece of a row
+  __shared__ float red[NW][16][17];
+  __shared__ float ssq[NW][TB][16];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int j = lane & 15, G = lane >> 4;
+  const int n0 = blockIdx.x * 16 * R;          // R groups of 16 rows share every load of X
+  const T* wrow[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) wrow[r] = W + (size_t)(n0 + r * 16 + j < N ? n0 + r * 16 + j : N - 1) * ldw;
+
+  f32x4_t acc[R][TB];
+  float ss[TB];
+#pragma unroll
+  for (int c = 0; c < TB; ++c) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    ss[c] = 0.f;
+  }
+  const int pieces = (K + PIECE - 1) / PIECE;
+  // blocks start at different places of their rows, so that at any moment they ask different memory channels
+  const int rot = (int)((blockIdx.x * 7u) % (unsigned)pieces);
+#pragma unroll 4
+  for (int pi = wave; pi < pieces; pi += NW) {
+    const int p = pi + rot < pieces ? pi + rot : pi + rot - pieces;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {            // the two 64-byte halves of the piece
+      const int k = p * PIECE + h * 4 * EPC + G * EPC;
+      const bool in = k < K;
+      uint4 a[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) a[r] = in ? *(const uint4*)(wrow[r] + k) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int c = 0; c < TB; ++c) {
+        const int t = c * 16 + j;
+        uint4 b = make_uint4(0, 0, 0, 0);
+        if (in && t < Tn) {
+          if (NORM) {
+            const float* xr = (const float*)Xv + (size_t)t * ldx + k;
+            float f[EPC];
+#pragma unroll
+            for (int e = 0; e < EPC; e += 4) {
+              const float4 x4 = *(const float4*)(xr + e);
+              const float4 w4 = *(const float4*)(norm_w + k + e);
+              ss[c] = fmaf(x4.x, x4.x, ss[c]);
+              ss[c] = fmaf(x4.y, x4.y, ss[c]);
+              ss[c] = fmaf(x4.z, x4.z, ss[c]);
+              ss[c] = fmaf(x4.w, x4.w, ss[c]);
+              f[e] = x4.x * w4.x;
+              f[e + 1] = x4.y * w4.y;
+              f[e + 2] = x4.z * w4.z;
+              f[e + 3] = x4.w * w4.w;
+            }
+            b = Mma16<T>::pack(f);
+          } else {
+            b = *(const uint4*)((const T*)Xv + (size_t)t * ldx + k);
+          }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) Mma16<T>::run(a[r], b, acc[r][c]);
+      }
+    }
+  }
+  // lane: token = 16 c + j, rows 16 r + 4 G + v.  Tile by tile the partial sums go to LDS and wave 0 adds them in
+  // wave order and runs the epilogue.
+  float scale[TB];
+  if (NORM) {
+#pragma unroll
+    for (int c = 0; c < TB; ++c) {
+      float s = ss[c];
+      s += __shfl_xor(s, 16, WAVE);
+      s += __shfl_xor(s, 32, WAVE);
+      if (G == 0) ssq[wave][c][j] = s;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < TB; ++c) {
+      float s = 0.f;
+      for (int w = 0; w < NW; ++w) s += ssq[w][c][j];
+      scale[c] = 1.0f / sqrtf(s / (float)K + eps);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int c = 0; c < TB; ++c) {
+      if (NW > 1) {
+        if (r + c) __syncthreads();          // wave 0 has read the tile before
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave][4 * G + v][j] = acc[r][c][v];
+        __syncthreads();
+      }
+      if (wave == 0) {
+        float v[4];
+        if (NW > 1) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] = 0.f;
+          for (int w = 0; w < NW; ++w)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] += red[w][4 * G + q][j];
+        } else {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] = acc[r][c][q];
+        }
+        if (NORM) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] *= scale[c];
+        }
+        const int t = c * 16 + j;
+        if (t < Tn) epilogue4<T, EPI>(Y, ldy, N, t, n0 + r * 16 + 4 * G, v[0], v[1], v[2], v[3]);
+      }
+    }
+}
+
+template <typename T, int NW, int R, int EPI, bool NORM>
+static void launch_skinny_nw(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K, int ldw,
+                             int ldx, int ldy, hipStream_t stream) {
+  dim3 g((N + 16 * R - 1) / (16 * R)), b(NW * WAVE);
+  const int tb = (Tn + 15) / 16;
+#define SKINNY_GO(TB_) hipLaunchKernelGGL((skinny_kernel<T, NW, R, TB_, EPI, NORM>), g, b, 0, stream, (const T*)W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy)
+  if (tb <= 1) SKINNY_GO(1);
+  else if (tb == 2) SKINNY_GO(2);
+  else if (tb == 3) SKINNY_GO(3);
+  else SKINNY_GO(4);
+#undef SKINNY_GO
+}
+
+// The number of waves that share a block's rows is a function of K alone, so the order of the sums does not
+// depend on the step.  force_nw (1, 2, 4, 8) is for tuning and tests.
+template <typename T, int EPI, bool NORM>
+static void launch_skinny(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K, int ldw,
+                          int ldx, int ldy, hipStream_t stream, int force_nw = 0) {
+  const int pieces = (K * (int)sizeof(T) + 127) / 128;
+  int nw = pieces >= 32 ? 8 : (pieces >= 16 ? 4 : (pieces >= 8 ? 2 : 1));
+  if (force_nw) nw = force_nw;
+  // many rows: each block takes 2 or 4 groups of 16, which divides the traffic of X (a function of N alone)
+  const bool wide = N >= 32768 && nw == 8, mid = N >= 8192 && nw == 8;
+  if (wide) launch_skinny_nw<T, 8, 4, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else if (mid) launch_skinny_nw<T, 8, 2, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else if (nw == 8) launch_skinny_nw<T, 8, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else if (nw == 4) launch_skinny_nw<T, 4, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else if (nw == 2) launch_skinny_nw<T, 2, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else launch_skinny_nw<T, 1, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+}
+
+template <typename T, int EPI>
+static void launch_gemv(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy,
+                        hipStream_t stream) {
+  const int blocks = (N + GEMV_WAVES * GEMV_ROWS - 1) / (GEMV_WAVES * GEMV_ROWS);
+  dim3 g(blocks), b(GEMV_WAVES * WAVE);
+  if (Tn == 1) hipLaunchKernelGGL((gemv_kernel<T, 1, EPI>), g, b, 0, stream, (const T*)W, (const T*)X, Y, N, Tn, K, ldw, ldx, ldy);
+  else if (Tn == 2) hipLaunchKernelGGL((gemv_kernel<T, 2, EPI>), g, b, 0, stream, (const T*)W, (const T*)X, Y, N, Tn, K, ldw, ldx, ldy);
+  else if (Tn <= 4) hipLaunchKernelGGL((gemv_kernel<T, 4, EPI>), g, b, 0, stream, (const T*)W, (const T*)X, Y, N, Tn, K, ldw, ldx, ldy);
+  else hipLaunchKernelGGL((gemv_kernel<T, 8, EPI>), g, b, 0, stream, (const T*)W, (const T*)X, Y, N, Tn, K, ldw, ldx, ldy);
+}
+
+template <typename T, int EPI>
+static void dispatch_rows(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy, int kind,
+                          hipStream_t stream) {
+  // kind: 0 = the MFMA kernel, 1 = the vector kernel (at most 8 rows), 6..9 = the MFMA kernel with 1, 2, 4, 8 waves per block
+  if (kind == 1) launch_gemv<T, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else launch_skinny<T, EPI, false>(W, X, nullptr, 0.f, Y, N, Tn, K, ldw, ldx, ldy, stream, kind == 0 ? 0 : 1 << (kind - 6));
+}
+
+template <typename T>
+static const char* rows_by_epilogue(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy,
+                                    int epi, int kind, hipStream_t stream) {
+  switch (epi) {
+    case EPI_STORE: dispatch_rows<T, EPI_STORE>(W, X, Y, N, Tn, K, ldw, ldx, ldy, kind, stream); break;
+    case EPI_ACCUM_F32: dispatch_rows<T, EPI_ACCUM_F32>(W, X, Y, N, Tn, K, ldw, ldx, ldy, kind, stream); break;
+    case EPI_SWIGLU: dispatch_rows<T, EPI_SWIGLU>(W, X, Y, N, Tn, K, ldw, ldx, ldy, kind, stream); break;
+    case EPI_STORE_F32: dispatch_rows<T, EPI_STORE_F32>(W, X, Y, N, Tn, K, ldw, ldx, ldy, kind, stream); break;
+    default: DLGO_FAIL("gemm_rows: unknown epilogue %d", epi);
+  }
+  return nullptr;
+}
+
+// Y[t, n] (epilogue) = sum_k X[t, k] W[n, k] for at most 64 rows of X.  ldy counts elements of Y's own type; for the
+// SwiGLU epilogue Y has N/2 columns.
+extern "C" const char* dlgo_gemm_rows(const void* W, const void* X, void* Y, int dtype, int N, int Tn, int K, int ldw, int ldx,
+                                      int ldy, int epilogue, int kind, hipStream_t stream) {
+  DLGO_REQUIRE(N > 0 && Tn >= 0 && Tn <= 64 && K > 0, "gemm_rows: bad sizes N=%d T=%d K=%d (at most 64 rows)", N, Tn, K);
+  DLGO_REQUIRE(dtype == DLGO_DTYPE_F32 || dtype == DLGO_DTYPE_BF16, "gemm_rows: unknown dtype code %d", dtype);
+  const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
+  DLGO_REQUIRE(K % epc == 0, "gemm: inner size %d must be a multiple of %d for 16-byte loads", K, epc);
+  DLGO_REQUIRE(ldw % epc == 0 && ldx % epc == 0 && ldw >= K && ldx >= K, "gemm: row strides (%d, %d) must be multiples of %d and at least K", ldw, ldx, epc);
+  DLGO_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && ((uintptr_t)Y & 15) == 0, "gemm: operands must be 16-byte aligned");
+  DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm: SwiGLU epilogue needs an even N and ldy >= N/2");
+  DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm: ldy %d shorter than N %d", ldy, N);
+  DLGO_REQUIRE(kind == 0 || kind == 1 || (kind >= 6 && kind <= 9), "gemm_rows: unknown kernel choice %d", kind);
+  DLGO_REQUIRE(kind != 1 || Tn <= 8, "gemm: the vector kernel takes at most 8 rows, got %d", Tn);
+  if (Tn == 0) return nullptr;
+  const char* err = dtype == DLGO_DTYPE_F32 ? rows_by_epilogue<float>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, kind, stream)
+                                            : rows_by_epilogue<bf16_t>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, kind, stream);
+  if (err) return err;
+  DLGO_LAUNCH_CHECK("gemm_rows");
+  return nullptr;
+}
+
+// Y (epilogue)= (rmsnorm(X) * norm_w) W^T for up to 64 rows of the float32 residual stream X [T, K], without
+// writing the normed rows.  Epilogues as dlgo_gemm.
+extern "C" const char* dlgo_gemm_rmsnorm(const void* W, const float* X, const float* norm_w, float eps, void* Y, int dtype, int N,
+                                         int Tn, int K, int ldw, int ldx, int ldy, int epilogue, hipStream_t stream) {
+  DLGO_REQUIRE(N > 0 && Tn >= 0 && Tn <= 64 && K > 0, "gemm_rmsnorm: bad sizes N=%d T=%d K=%d (at most 64 rows)", N, Tn, K);
+  DLGO_REQUIRE(dtype == DLGO_DTYPE_F32 || dtype == DLGO_DTYPE_BF16, "gemm_rmsnorm: unknown dtype code %d", dtype);
+  const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
+  DLGO_REQUIRE(K % epc == 0 && ldw % epc == 0 && ldx % 4 == 0 && ldw >= K && ldx >= K, "gemm_rmsnorm: K and the row strides must be multiples of %d", epc);
+  DLGO_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && ((uintptr_t)Y & 15) == 0 && ((uintptr_t)norm_w & 15) == 0,
+               "gemm_rmsnorm: operands must be 16-byte aligned");
+  DLGO_REQUIRE(eps > 0.f, "gemm_rmsnorm: eps must be positive");
+  DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm_rmsnorm: SwiGLU epilogue needs an even N and ldy >= N/2");
+  DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm_rmsnorm: ldy %d shorter than N %d", ldy, N);
+  if (Tn == 0) return nullptr;
+#define NORM_GO(T_, E_) launch_skinny<T_, E_, true>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream)
+  if (dtype == DLGO_DTYPE_F32) {
+    switch (epilogue) {
+      case EPI_STORE: NORM_GO(float, EPI_STORE); break;
+      case EPI_ACCUM_F32: NORM_GO(float, EPI_ACCUM_F32); break;
+      case EPI_SWIGLU: NORM_GO(float, EPI_SWIGLU); break;
+      case EPI_STORE_F32: NORM_GO(float, EPI_STORE_F32); break;
+      default: DLGO_FAIL("gemm_rmsnorm: unknown epilogue %d", epilogue);
+    }
+  } else {
+    switch (epilogue) {
+      case EPI_STORE: NORM_GO(bf16_t, EPI_STORE); break;
+      case EPI_ACCUM_F32: NORM_GO(bf16_t, EPI_ACCUM_F32); break;
+      case EPI_SWIGLU: NORM_GO(bf16_t, EPI_SWIGLU); break;
+      case EPI_STORE_F32: NORM_GO(bf16_t, EPI_STORE_F32); break;
+      default: DLGO_FAIL("gemm_rmsnorm: unknown epilogue %d", epilogue);
+    }
+  }
+#undef NORM_GO
+  DLGO_LAUNCH_CHECK("gemm_rmsnorm");
+  return nullptr;
+}

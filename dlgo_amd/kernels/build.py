@@ -49,7 +49,8 @@ def _hipcc() -> str:
 
 def _source_hash(module: str, defines: Defines) -> str:
     h = hashlib.sha256()
-    for name in (module + ".hip", "common.h"):
+    names = [module + ".hip"] + sorted(n for n in os.listdir(CSRC) if n.endswith(".h"))
+    for name in names:
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(f.read())
     h.update(repr(FLAGS).encode())
@@ -208,7 +209,7 @@ DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128)
 
 
 def all_variants(head_dims: Sequence[int] = DEFAULT_HEAD_DIMS) -> list[Variant]:
-    out: list[Variant] = [(m, ()) for m in ("embed", "rmsnorm", "rope_kv", "gemm", "sampling")]
+    out: list[Variant] = [(m, ()) for m in ("embed", "rmsnorm", "rope_kv", "gemm", "gemm_rows", "sampling")]
     out += [("attention", (("HEAD_DIM", hd),)) for hd in head_dims]
     return out
 

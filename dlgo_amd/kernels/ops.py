@@ -17,6 +17,8 @@ PAGE = 64   # tokens per cache page; the kernels are compiled with the same numb
 
 EPI_STORE, EPI_ACCUM_F32, EPI_SWIGLU, EPI_STORE_F32 = 0, 1, 2, 3
 GEMM_AUTO, GEMM_STREAM, GEMM_TILE128, GEMM_TILE64, GEMM_TILE32, GEMM_ROWS16 = 0, 1, 2, 3, 4, 5
+GEMM_TILE256X128, GEMM_TILE256 = 10, 11
+GEMM_FEW_ROWS = 64      # up to this many rows of x the weight-streaming kernels are chosen
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 
@@ -68,7 +70,7 @@ def _lib(module: str, defines=()):
     lib = build.load(module, defines)
     key = (module, tuple(defines))
     if key not in _protos_done:
-        for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_rmsnorm", "dlgo_attention_rows",
+        for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_attention_rows",
                      "dlgo_attention_prefill", "dlgo_attention_decode", "dlgo_argmax", "dlgo_sample"):
             if hasattr(lib, name):
                 getattr(lib, name).restype = ctypes.c_char_p
@@ -129,9 +131,14 @@ def gemm(weight: torch.Tensor, x: torch.Tensor, out: torch.Tensor, epilogue: int
     cols = n // 2 if epilogue == EPI_SWIGLU else n
     if tuple(out.shape) != (t, cols):
         raise KernelError(f"gemm: output {tuple(out.shape)}, expected {(t, cols)}")
-    _check(_lib("gemm").dlgo_gemm(_ptr(weight), _ptr(x), _ptr(out), dtype_code(weight.dtype), n, t, k,
-                                  _rows(weight, "gemm weight"), _rows(x, "gemm input"), _rows(out, "gemm output"),
-                                  epilogue, kind, _stream()))
+    rows_kernel = kind in (GEMM_STREAM, 5, 6, 7, 8, 9) or (kind == GEMM_AUTO and t <= GEMM_FEW_ROWS)
+    if rows_kernel:
+        fn = _lib("gemm_rows").dlgo_gemm_rows
+        kind = 0 if kind in (GEMM_AUTO, GEMM_ROWS16) else kind
+    else:
+        fn = _lib("gemm").dlgo_gemm
+    _check(fn(_ptr(weight), _ptr(x), _ptr(out), dtype_code(weight.dtype), n, t, k, _rows(weight, "gemm weight"),
+              _rows(x, "gemm input"), _rows(out, "gemm output"), epilogue, kind, _stream()))
     return out
 
 
@@ -154,7 +161,7 @@ def gemm_rmsnorm(weight: torch.Tensor, x: torch.Tensor, norm_weight: torch.Tenso
     cols = n // 2 if epilogue == EPI_SWIGLU else n
     if tuple(out.shape) != (t, cols):
         raise KernelError(f"gemm_rmsnorm: output {tuple(out.shape)}, expected {(t, cols)}")
-    _check(_lib("gemm").dlgo_gemm_rmsnorm(_ptr(weight), _ptr(x), _ptr(norm_weight), ctypes.c_float(eps), _ptr(out),
+    _check(_lib("gemm_rows").dlgo_gemm_rmsnorm(_ptr(weight), _ptr(x), _ptr(norm_weight), ctypes.c_float(eps), _ptr(out),
                                           dtype_code(weight.dtype), n, t, k, _rows(weight, "gemm weight"),
                                           _rows(x, "residual rows"), _rows(out, "gemm output"), epilogue, _stream()))
     return out

@@ -51,7 +51,7 @@ class Mixer(Part):
 
 
 class Attention(Mixer):
-    kernel_modules = ("gemm", "rope_kv")
+    kernel_modules = ("gemm", "gemm_rows", "rope_kv")
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PositionEncoding,
                  window: Optional[int] = None, scale: Optional[float] = None):
@@ -76,7 +76,7 @@ class Attention(Mixer):
         }
 
     def kernel_variants(self, dtype):
-        return (("gemm", ()), ("rope_kv", ()), ("attention", (("HEAD_DIM", self.head_dim),)))
+        return (("gemm", ()), ("gemm_rows", ()), ("rope_kv", ()), ("attention", (("HEAD_DIM", self.head_dim),)))
 
     def cache_needs(self) -> List[CacheNeed]:
         return [CacheNeed(kind="kv", kv_heads=self.n_kv_heads, head_dim=self.head_dim, window=self.window)]

@@ -31,7 +31,7 @@ class Embedding(Part):
 
 
 class OutputHead(Part):
-    kernel_modules = ("gemm",)
+    kernel_modules = ("gemm", "gemm_rows")
 
     def __init__(self, vocab: int, width: int, tied_to: Optional[Embedding] = None):
         self.vocab, self.width = vocab, width

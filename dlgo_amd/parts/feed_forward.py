@@ -26,7 +26,7 @@ class FeedForward(Part):
 
 
 class GatedFeedForward(FeedForward):
-    kernel_modules = ("gemm",)
+    kernel_modules = ("gemm", "gemm_rows")
 
     def __init__(self, width: int, inner: int, activation: str = "silu"):
         if activation != "silu":
