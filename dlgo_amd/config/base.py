@@ -122,7 +122,14 @@ def register_architecture(name: str, config_class: Type[ModelConfig], build: Cal
     _ARCHITECTURES[name] = Architecture(name, config_class, build)
 
 
+def _builtin() -> None:
+    """The architectures that ship with the library register themselves when their package is imported."""
+    import importlib
+    importlib.import_module("dlgo_amd.models")
+
+
 def known_architectures() -> list[str]:
+    _builtin()
     return sorted(_ARCHITECTURES)
 
 
@@ -133,6 +140,7 @@ def architecture_of(raw: Mapping[str, Any]) -> Architecture:
     if not names or not isinstance(names, (list, tuple)) or not isinstance(names[0], str):
         raise ConfigError('config.json: "architectures" must name the model class, e.g. ["LlamaForCausalLM"]')
     name = names[0]
+    _builtin()
     if name not in _ARCHITECTURES:
         raise ConfigError(f"config.json: unknown architecture {name!r}; known: {', '.join(known_architectures()) or '(none)'}")
     return _ARCHITECTURES[name]
@@ -164,6 +172,7 @@ def load_config(folder_or_file: str) -> ModelConfig:
 
 def build_model(config: ModelConfig):
     """The registry's second half: configuration -> model made of parts."""
+    _builtin()
     if config.architecture not in _ARCHITECTURES:
         raise ConfigError(f"unknown architecture {config.architecture!r}; known: {', '.join(known_architectures())}")
     return _ARCHITECTURES[config.architecture].build(config)

@@ -219,7 +219,7 @@ static const char* by_epilogue(const void* W, const void* X, void* Y, int N, int
 extern "C" const char* dlgo_gemm(const void* W, const void* X, void* Y, int dtype, int N, int Tn, int K, int ldw, int ldx,
                                  int ldy, int epilogue, int force_kind, hipStream_t stream) {
   DLGO_REQUIRE(N > 0 && Tn >= 0 && K > 0, "gemm: bad sizes N=%d T=%d K=%d", N, Tn, K);
-  DLGO_REQUIRE(dtype == DLGO_DTYPE_F32 || dtype == DLGO_DTYPE_BF16, "gemm: unknown dtype code %d", dtype);
+  DLGO_REQUIRE(dtype == DLGO_ELEM, "gemm: this library is built for dtype code %d, got %d", DLGO_ELEM, dtype);
   const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
   DLGO_REQUIRE(K % epc == 0, "gemm: inner size %d must be a multiple of %d for 16-byte loads", K, epc);
   DLGO_REQUIRE(ldw % epc == 0 && ldx % epc == 0 && ldw >= K && ldx >= K, "gemm: row strides (%d, %d) must be multiples of %d and at least K", ldw, ldx, epc);
@@ -229,8 +229,7 @@ extern "C" const char* dlgo_gemm(const void* W, const void* X, void* Y, int dtyp
   DLGO_REQUIRE(force_kind == 0 || (force_kind >= 2 && force_kind <= 4) || (force_kind >= 10 && force_kind <= 14),
                "gemm: unknown kernel choice %d", force_kind);
   if (Tn == 0) return nullptr;
-  const char* err = dtype == DLGO_DTYPE_F32 ? by_epilogue<float>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, force_kind, stream)
-                                            : by_epilogue<bf16_t>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, force_kind, stream);
+  const char* err = by_epilogue<elem_t>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, force_kind, stream);
   if (err) return err;
   DLGO_LAUNCH_CHECK("gemm");
   return nullptr;

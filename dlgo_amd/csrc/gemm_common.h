@@ -4,6 +4,18 @@
 #pragma once
 #include "common.h"
 
+// One library per element type: -DDLGO_ELEM=0 (float32) or 1 (bfloat16), so that a model compiles what it runs in.
+#ifndef DLGO_ELEM
+#error "compile with -DDLGO_ELEM=0 (float32) or 1 (bfloat16)"
+#endif
+#if DLGO_ELEM == DLGO_DTYPE_F32
+typedef float elem_t;
+#elif DLGO_ELEM == DLGO_DTYPE_BF16
+typedef bf16_t elem_t;
+#else
+#error "DLGO_ELEM must be 0 or 1"
+#endif
+
 enum { EPI_STORE = 0, EPI_ACCUM_F32 = 1, EPI_SWIGLU = 2, EPI_STORE_F32 = 3 };
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }

@@ -319,7 +319,7 @@ static const char* rows_by_epilogue(const void* W, const void* X, void* Y, int N
 extern "C" const char* dlgo_gemm_rows(const void* W, const void* X, void* Y, int dtype, int N, int Tn, int K, int ldw, int ldx,
                                       int ldy, int epilogue, int kind, hipStream_t stream) {
   DLGO_REQUIRE(N > 0 && Tn >= 0 && Tn <= 64 && K > 0, "gemm_rows: bad sizes N=%d T=%d K=%d (at most 64 rows)", N, Tn, K);
-  DLGO_REQUIRE(dtype == DLGO_DTYPE_F32 || dtype == DLGO_DTYPE_BF16, "gemm_rows: unknown dtype code %d", dtype);
+  DLGO_REQUIRE(dtype == DLGO_ELEM, "gemm_rows: this library is built for dtype code %d, got %d", DLGO_ELEM, dtype);
   const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
   DLGO_REQUIRE(K % epc == 0, "gemm: inner size %d must be a multiple of %d for 16-byte loads", K, epc);
   DLGO_REQUIRE(ldw % epc == 0 && ldx % epc == 0 && ldw >= K && ldx >= K, "gemm: row strides (%d, %d) must be multiples of %d and at least K", ldw, ldx, epc);
@@ -329,8 +329,7 @@ extern "C" const char* dlgo_gemm_rows(const void* W, const void* X, void* Y, int
   DLGO_REQUIRE(kind == 0 || kind == 1 || (kind >= 6 && kind <= 9), "gemm_rows: unknown kernel choice %d", kind);
   DLGO_REQUIRE(kind != 1 || Tn <= 8, "gemm: the vector kernel takes at most 8 rows, got %d", Tn);
   if (Tn == 0) return nullptr;
-  const char* err = dtype == DLGO_DTYPE_F32 ? rows_by_epilogue<float>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, kind, stream)
-                                            : rows_by_epilogue<bf16_t>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, kind, stream);
+  const char* err = rows_by_epilogue<elem_t>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, kind, stream);
   if (err) return err;
   DLGO_LAUNCH_CHECK("gemm_rows");
   return nullptr;
@@ -341,7 +340,7 @@ extern "C" const char* dlgo_gemm_rows(const void* W, const void* X, void* Y, int
 extern "C" const char* dlgo_gemm_rmsnorm(const void* W, const float* X, const float* norm_w, float eps, void* Y, int dtype, int N,
                                          int Tn, int K, int ldw, int ldx, int ldy, int epilogue, hipStream_t stream) {
   DLGO_REQUIRE(N > 0 && Tn >= 0 && Tn <= 64 && K > 0, "gemm_rmsnorm: bad sizes N=%d T=%d K=%d (at most 64 rows)", N, Tn, K);
-  DLGO_REQUIRE(dtype == DLGO_DTYPE_F32 || dtype == DLGO_DTYPE_BF16, "gemm_rmsnorm: unknown dtype code %d", dtype);
+  DLGO_REQUIRE(dtype == DLGO_ELEM, "gemm_rmsnorm: this library is built for dtype code %d, got %d", DLGO_ELEM, dtype);
   const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
   DLGO_REQUIRE(K % epc == 0 && ldw % epc == 0 && ldx % 4 == 0 && ldw >= K && ldx >= K, "gemm_rmsnorm: K and the row strides must be multiples of %d", epc);
   DLGO_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && ((uintptr_t)Y & 15) == 0 && ((uintptr_t)norm_w & 15) == 0,
@@ -350,23 +349,13 @@ extern "C" const char* dlgo_gemm_rmsnorm(const void* W, const float* X, const fl
   DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm_rmsnorm: SwiGLU epilogue needs an even N and ldy >= N/2");
   DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm_rmsnorm: ldy %d shorter than N %d", ldy, N);
   if (Tn == 0) return nullptr;
-#define NORM_GO(T_, E_) launch_skinny<T_, E_, true>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream)
-  if (dtype == DLGO_DTYPE_F32) {
-    switch (epilogue) {
-      case EPI_STORE: NORM_GO(float, EPI_STORE); break;
-      case EPI_ACCUM_F32: NORM_GO(float, EPI_ACCUM_F32); break;
-      case EPI_SWIGLU: NORM_GO(float, EPI_SWIGLU); break;
-      case EPI_STORE_F32: NORM_GO(float, EPI_STORE_F32); break;
-      default: DLGO_FAIL("gemm_rmsnorm: unknown epilogue %d", epilogue);
-    }
-  } else {
-    switch (epilogue) {
-      case EPI_STORE: NORM_GO(bf16_t, EPI_STORE); break;
-      case EPI_ACCUM_F32: NORM_GO(bf16_t, EPI_ACCUM_F32); break;
-      case EPI_SWIGLU: NORM_GO(bf16_t, EPI_SWIGLU); break;
-      case EPI_STORE_F32: NORM_GO(bf16_t, EPI_STORE_F32); break;
-      default: DLGO_FAIL("gemm_rmsnorm: unknown epilogue %d", epilogue);
-    }
+#define NORM_GO(E_) launch_skinny<elem_t, E_, true>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream)
+  switch (epilogue) {
+    case EPI_STORE: NORM_GO(EPI_STORE); break;
+    case EPI_ACCUM_F32: NORM_GO(EPI_ACCUM_F32); break;
+    case EPI_SWIGLU: NORM_GO(EPI_SWIGLU); break;
+    case EPI_STORE_F32: NORM_GO(EPI_STORE_F32); break;
+    default: DLGO_FAIL("gemm_rmsnorm: unknown epilogue %d", epilogue);
   }
 #undef NORM_GO
   DLGO_LAUNCH_CHECK("gemm_rmsnorm");

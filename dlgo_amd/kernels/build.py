@@ -204,12 +204,27 @@ def loaded_libraries() -> Sequence[str]:
     return sorted(_loaded)
 
 
+#: kernel files compiled once per element type (-DDLGO_ELEM=0 float32, 1 bfloat16)
+PER_ELEMENT_TYPE = ("gemm", "gemm_rows")
+_ELEM_CODE = {"torch.float32": 0, "torch.bfloat16": 1}
+
+
+def variant(module: str, dtype=None, defines: Defines = ()) -> Variant:
+    """The (module, defines) pair of a kernel file for a run dtype."""
+    if module in PER_ELEMENT_TYPE:
+        if str(dtype) not in _ELEM_CODE:
+            raise KernelBuildError(f"{module} is built for float32 or bfloat16, not {dtype}")
+        return module, (("DLGO_ELEM", _ELEM_CODE[str(dtype)]),) + tuple(defines)
+    return module, tuple(defines)
+
+
 #: head sizes compiled ahead by build_all(): those of the test configurations and of the benchmark shapes
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128)
 
 
 def all_variants(head_dims: Sequence[int] = DEFAULT_HEAD_DIMS) -> list[Variant]:
-    out: list[Variant] = [(m, ()) for m in ("embed", "rmsnorm", "rope_kv", "gemm", "gemm_rows", "sampling")]
+    out: list[Variant] = [(m, ()) for m in ("embed", "rmsnorm", "rope_kv", "sampling")]
+    out += [(m, (("DLGO_ELEM", code),)) for m in ("gemm", "gemm_rows") for code in (0, 1)]
     out += [("attention", (("HEAD_DIM", hd),)) for hd in head_dims]
     return out
 

@@ -133,10 +133,10 @@ def gemm(weight: torch.Tensor, x: torch.Tensor, out: torch.Tensor, epilogue: int
         raise KernelError(f"gemm: output {tuple(out.shape)}, expected {(t, cols)}")
     rows_kernel = kind in (GEMM_STREAM, 5, 6, 7, 8, 9) or (kind == GEMM_AUTO and t <= GEMM_FEW_ROWS)
     if rows_kernel:
-        fn = _lib("gemm_rows").dlgo_gemm_rows
+        fn = _lib("gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),)).dlgo_gemm_rows
         kind = 0 if kind in (GEMM_AUTO, GEMM_ROWS16) else kind
     else:
-        fn = _lib("gemm").dlgo_gemm
+        fn = _lib("gemm", (("DLGO_ELEM", dtype_code(weight.dtype)),)).dlgo_gemm
     _check(fn(_ptr(weight), _ptr(x), _ptr(out), dtype_code(weight.dtype), n, t, k, _rows(weight, "gemm weight"),
               _rows(x, "gemm input"), _rows(out, "gemm output"), epilogue, kind, _stream()))
     return out
@@ -161,7 +161,7 @@ def gemm_rmsnorm(weight: torch.Tensor, x: torch.Tensor, norm_weight: torch.Tenso
     cols = n // 2 if epilogue == EPI_SWIGLU else n
     if tuple(out.shape) != (t, cols):
         raise KernelError(f"gemm_rmsnorm: output {tuple(out.shape)}, expected {(t, cols)}")
-    _check(_lib("gemm_rows").dlgo_gemm_rmsnorm(_ptr(weight), _ptr(x), _ptr(norm_weight), ctypes.c_float(eps), _ptr(out),
+    _check(_lib("gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),)).dlgo_gemm_rmsnorm(_ptr(weight), _ptr(x), _ptr(norm_weight), ctypes.c_float(eps), _ptr(out),
                                           dtype_code(weight.dtype), n, t, k, _rows(weight, "gemm weight"),
                                           _rows(x, "residual rows"), _rows(out, "gemm output"), epilogue, _stream()))
     return out

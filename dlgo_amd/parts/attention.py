@@ -76,7 +76,8 @@ class Attention(Mixer):
         }
 
     def kernel_variants(self, dtype):
-        return (("gemm", ()), ("gemm_rows", ()), ("rope_kv", ()), ("attention", (("HEAD_DIM", self.head_dim),)))
+        from ..kernels.build import variant
+        return tuple(variant(m, dtype) for m in self.kernel_modules) + (variant("attention", dtype, (("HEAD_DIM", self.head_dim),)),)
 
     def cache_needs(self) -> List[CacheNeed]:
         return [CacheNeed(kind="kv", kv_heads=self.n_kv_heads, head_dim=self.head_dim, window=self.window)]

@@ -47,7 +47,8 @@ class Part:
 
     def kernel_variants(self, dtype: torch.dtype) -> Tuple[Tuple[str, Tuple[Tuple[str, int], ...]], ...]:
         """(module, defines) pairs to compile for this part at `dtype`."""
-        return tuple((m, ()) for m in self.kernel_modules)
+        from ..kernels.build import variant
+        return tuple(variant(m, dtype) for m in self.kernel_modules)
 
 
 def stored(t: torch.Tensor, spec: TensorSpec, device: torch.device, dtype: torch.dtype) -> torch.Tensor:
