@@ -28,7 +28,7 @@ __device__ __forceinline__ void epilogue4(void* __restrict__ Y, int ldy, int N, 
   const bool full = n + 3 < N;
   if (EPI == EPI_STORE) {
     T* y = (T*)Y + (size_t)t * ldy + n;
-    if (full && (ldy & 3) == 0) {
+    if (full && (ldy & 3) == 0 && ((uintptr_t)y & (4 * sizeof(T) - 1)) == 0) {
       if (sizeof(T) == 4) {
         *(float4*)y = make_float4(v0, v1, v2, v3);
       } else {
@@ -43,7 +43,7 @@ __device__ __forceinline__ void epilogue4(void* __restrict__ Y, int ldy, int N, 
     }
   } else if (EPI == EPI_ACCUM_F32 || EPI == EPI_STORE_F32) {
     float* y = (float*)Y + (size_t)t * ldy + n;
-    if (full && (ldy & 3) == 0) {
+    if (full && (ldy & 3) == 0 && ((uintptr_t)y & 15) == 0) {
       float4 o = make_float4(v0, v1, v2, v3);
       if (EPI == EPI_ACCUM_F32) {
         const float4 old = *(float4*)y;
@@ -59,7 +59,7 @@ __device__ __forceinline__ void epilogue4(void* __restrict__ Y, int ldy, int N, 
     }
   } else {   // EPI_SWIGLU: rows (n, n+1) and (n+2, n+3) are (gate, up) pairs; N is even
     T* y = (T*)Y + (size_t)t * ldy + (n >> 1);
-    if (n + 3 < N && (ldy & 1) == 0) {     // both halves at once
+    if (n + 3 < N && (ldy & 1) == 0 && ((uintptr_t)y & (2 * sizeof(T) - 1)) == 0) {     // both halves at once
       if (sizeof(T) == 4) *(float2*)y = make_float2(silu_f(v0) * v1, silu_f(v2) * v3);
       else *(uint32_t*)y = (uint32_t)f32_to_bf16(silu_f(v0) * v1) | ((uint32_t)f32_to_bf16(silu_f(v2) * v3) << 16);
     } else {

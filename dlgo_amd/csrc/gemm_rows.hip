@@ -264,17 +264,18 @@ static void launch_skinny_nw(const void* W, const void* X, const float* norm_w, 
 #undef SKINNY_GO
 }
 
-// The number of waves that share a block's rows is a function of K alone, so the order of the sums does not
-// depend on the step.  force_nw (1, 2, 4, 8) is for tuning and tests.
+// The number of waves that share a block's rows is a function of N and K alone, so the order of the sums does
+// not depend on the step (few rows of long k: 16 waves, so that the few blocks keep more loads in flight).  force_nw (1, 2, 4, 8) is for tuning and tests.
 template <typename T, int EPI, bool NORM>
 static void launch_skinny(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K, int ldw,
                           int ldx, int ldy, hipStream_t stream, int force_nw = 0) {
   const int pieces = (K * (int)sizeof(T) + 127) / 128;
-  int nw = pieces >= 32 ? 8 : (pieces >= 16 ? 4 : (pieces >= 8 ? 2 : 1));
+  int nw = pieces >= 128 && N <= 4096 ? 16 : (pieces >= 32 ? 8 : (pieces >= 16 ? 4 : (pieces >= 8 ? 2 : 1)));
   if (force_nw) nw = force_nw;
   // many rows: each block takes 2 or 4 groups of 16, which divides the traffic of X (a function of N alone)
   const bool wide = N >= 32768 && nw == 8, mid = N >= 8192 && nw == 8;
-  if (wide) launch_skinny_nw<T, 8, 4, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  if (nw == 16) launch_skinny_nw<T, 16, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  else if (wide) launch_skinny_nw<T, 8, 4, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
   else if (mid) launch_skinny_nw<T, 8, 2, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
   else if (nw == 8) launch_skinny_nw<T, 8, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
   else if (nw == 4) launch_skinny_nw<T, 4, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
@@ -323,7 +324,8 @@ extern "C" const char* dlgo_gemm_rows(const void* W, const void* X, void* Y, int
   const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
   DLGO_REQUIRE(K % epc == 0, "gemm: inner size %d must be a multiple of %d for 16-byte loads", K, epc);
   DLGO_REQUIRE(ldw % epc == 0 && ldx % epc == 0 && ldw >= K && ldx >= K, "gemm: row strides (%d, %d) must be multiples of %d and at least K", ldw, ldx, epc);
-  DLGO_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && ((uintptr_t)Y & 15) == 0, "gemm: operands must be 16-byte aligned");
+  DLGO_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0, "gemm: W and X must be 16-byte aligned");
+  DLGO_REQUIRE(((uintptr_t)Y & 3) == 0 || (dtype == DLGO_DTYPE_BF16 && ((uintptr_t)Y & 1) == 0), "gemm: Y must be aligned to its elements");
   DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm: SwiGLU epilogue needs an even N and ldy >= N/2");
   DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm: ldy %d shorter than N %d", ldy, N);
   DLGO_REQUIRE(kind == 0 || kind == 1 || (kind >= 6 && kind <= 9), "gemm_rows: unknown kernel choice %d", kind);
@@ -343,8 +345,8 @@ extern "C" const char* dlgo_gemm_rmsnorm(const void* W, const float* X, const fl
   DLGO_REQUIRE(dtype == DLGO_ELEM, "gemm_rmsnorm: this library is built for dtype code %d, got %d", DLGO_ELEM, dtype);
   const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
   DLGO_REQUIRE(K % epc == 0 && ldw % epc == 0 && ldx % 4 == 0 && ldw >= K && ldx >= K, "gemm_rmsnorm: K and the row strides must be multiples of %d", epc);
-  DLGO_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && ((uintptr_t)Y & 15) == 0 && ((uintptr_t)norm_w & 15) == 0,
-               "gemm_rmsnorm: operands must be 16-byte aligned");
+  DLGO_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && ((uintptr_t)norm_w & 15) == 0,
+               "gemm_rmsnorm: W, X and the norm weight must be 16-byte aligned");
   DLGO_REQUIRE(eps > 0.f, "gemm_rmsnorm: eps must be positive");
   DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm_rmsnorm: SwiGLU epilogue needs an even N and ldy >= N/2");
   DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm_rmsnorm: ldy %d shorter than N %d", ldy, N);

@@ -85,6 +85,11 @@ class Engine:
         self.max_ctx = min(x for x in (max_ctx, limit, pages_tokens) if x)
         self.max_step_tokens = max(1, min(max_step_tokens, pages_tokens))
         self.logits_rows = max(1, min(logits_rows, self.max_step_tokens))
+        for name, part in model.named_parts():
+            try:
+                part.check(self.dtype)
+            except ValueError as e:
+                raise EngineError(f"{name}: {e}") from None
         kernel_build.ensure_built(model.kernel_variants(self.dtype))
         self.cache = Cache(model.unit_needs, max_tokens, self.max_ctx, self.dtype, self.device, max_slots,
                            self.max_step_tokens)

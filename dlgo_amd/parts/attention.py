@@ -20,7 +20,7 @@ from typing import Dict, List, Optional
 import torch
 
 from ..kernels import ops
-from .base import CacheNeed, Part, TensorSpec, stored
+from .base import CacheNeed, Part, TensorSpec, check_inner, stored
 from .norm import RMSNorm
 from .position import PositionEncoding
 
@@ -74,6 +74,9 @@ class Attention(Mixer):
             "v_proj.weight": TensorSpec((self.kv_dim, self.width)),
             "o_proj.weight": TensorSpec((self.width, self.q_dim)),
         }
+
+    def check(self, dtype) -> None:
+        check_inner("attention", (("width", self.width), ("heads * head size", self.q_dim)), dtype)
 
     def kernel_variants(self, dtype):
         from ..kernels.build import variant

@@ -45,6 +45,9 @@ class Part:
         """Take the tensors named in tensor_specs() (CPU, as stored) and keep them on
         `device` the way the kernels want them."""
 
+    def check(self, dtype: torch.dtype) -> None:
+        """Raise ValueError if the kernels of this part cannot take its sizes at `dtype` (called before anything runs)."""
+
     def kernel_variants(self, dtype: torch.dtype) -> Tuple[Tuple[str, Tuple[Tuple[str, int], ...]], ...]:
         """(module, defines) pairs to compile for this part at `dtype`."""
         from ..kernels.build import variant
@@ -79,3 +82,12 @@ class CacheNeed:
     window: Optional[int] = None
     state_shape: Tuple[int, ...] = ()
     state_dtype: torch.dtype = torch.float32
+
+
+def check_inner(what: str, sizes, dtype: torch.dtype) -> None:
+    """The matrix products read 16 bytes at a time along their inner dimension."""
+    per = 4 if dtype == torch.float32 else 8
+    for name, n in sizes:
+        if n % per:
+            raise ValueError(f"{what}: {name} = {n} must be a multiple of {per} at {str(dtype).replace('torch.', '')} "
+                             f"(the products load 16 bytes at a time)")

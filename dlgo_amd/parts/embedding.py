@@ -9,7 +9,7 @@ from typing import Dict, Optional
 import torch
 
 from ..kernels import ops
-from .base import Part, TensorSpec, stored
+from .base import Part, TensorSpec, check_inner, stored
 from .norm import RMSNorm
 
 
@@ -44,6 +44,9 @@ class OutputHead(Part):
     def load(self, tensors, device, dtype) -> None:
         if self.tied_to is None:
             self._weight = stored(tensors["weight"], self.tensor_specs()["weight"], device, dtype)
+
+    def check(self, dtype) -> None:
+        check_inner("output head", (("width", self.width),), dtype)
 
     @property
     def weight(self) -> torch.Tensor:

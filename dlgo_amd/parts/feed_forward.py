@@ -10,7 +10,7 @@ from typing import Dict, Optional
 import torch
 
 from ..kernels import ops
-from .base import Part, TensorSpec, stored
+from .base import Part, TensorSpec, check_inner, stored
 from .norm import RMSNorm
 
 
@@ -41,6 +41,9 @@ class GatedFeedForward(FeedForward):
             "up_proj.weight": TensorSpec((self.inner, self.width)),
             "down_proj.weight": TensorSpec((self.width, self.inner)),
         }
+
+    def check(self, dtype) -> None:
+        check_inner("feed-forward", (("width", self.width), ("inner width", self.inner)), dtype)
 
     def load(self, tensors, device, dtype) -> None:
         spec = self.tensor_specs()

@@ -180,3 +180,37 @@ def test_errors_before_anything_runs(folders):
     assert eng.length(slot) == 0
     eng.step([Entry(slot, [1, 2, 3], [])])
     assert eng.length(slot) == 3
+
+
+def test_sizes_the_kernels_cannot_take_are_refused_at_once(tmp_path):
+    """A width that is no multiple of the products' 16-byte loads: a clear error when the engine is made, for the
+    dtype it concerns, not a wrong result later."""
+    from dlgo_amd.engine import Engine, EngineError
+    raw = dict(TINY_A, hidden_size=68, num_attention_heads=4, head_dim=16, intermediate_size=100)
+    folder = make_folder(raw, 1, tmp_path, dtype="float32")
+    with pytest.raises(EngineError, match="multiple of 8"):
+        Engine.from_folder(folder, "bfloat16", max_tokens=128)
+    eng = Engine.from_folder(folder, "float32", max_tokens=128)       # 68 and 100 are multiples of 4: float32 runs
+    from dlgo_amd.engine import Entry
+    (slot,) = eng.open(1)
+    tokens = [3, 9, 27, 81]
+    got = eng.step([Entry(slot, tokens, [0, 1, 2, 3])]).cpu().numpy()
+    cfg, w = plain.read_model(folder)
+    assert rel_err(got, plain.forward(cfg, w, tokens)) <= TOL["float32"]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_wanted_places_in_any_order_with_an_odd_vocabulary(folders, oracle, dtype):
+    """Logits only where they are wanted, in the order asked, from a step that is cut into pieces; the vocabulary of
+    this configuration (515) makes most rows of the output start at unaligned addresses."""
+    from dlgo_amd.engine import Entry
+    seqs = prompts_for(TINY_C, [90, 41, 7], seed=12)
+    eng = engine_for(folders["C", dtype], dtype, max_step_tokens=32)
+    slots = eng.open(3)
+    wants = [[89, 0, 40], [], [6, 5]]
+    out = eng.step([Entry(s, t, w) for s, t, w in zip(slots, seqs, wants)]).cpu().numpy()
+    assert out.shape == (5, 515)
+    rows = [(0, 89), (0, 0), (0, 40), (2, 6), (2, 5)]
+    for r, (i, p) in enumerate(rows):
+        assert rel_err(out[r], oracle("C", dtype, seqs[i])[p]) <= TOL[dtype], (r, i, p)
+    assert [eng.length(s) for s in slots] == [90, 41, 7]

@@ -337,6 +337,56 @@ def test_attention_over_pages(dtype, _, rel, H, KV, hd, window, seqs, kernel):
     close(out, torch.from_numpy(np.concatenate(want)), rel if dtype == torch.float32 else 2e-2, "attention")
 
 
+@pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("kernel", ["rows", "auto"])
+def test_attention_finds_a_far_key_and_respects_the_window_edge(dtype, _, rel, kernel):
+    """Random scores hide a key that is skipped or read twice.  Here one key among hundreds matches the query
+    so strongly that the output is that key's value: the first key, one in the middle of a page, the last key
+    of a page, the first of the next, the token itself; with a window, the key at its edge counts and the one just
+    outside does not."""
+    ops = _ops()
+    H, KV, hd = 4, 2, 32
+    length = 450
+    g = torch.Generator().manual_seed(9)
+    table, slots, storage, page_stride, unit_off, v_off = _paged_setup(dtype, [length], KV, hd, seed=4)
+    k = (0.05 * torch.randn(length, KV * hd, generator=g)).to(dtype)
+    v = torch.randn(length, KV * hd, generator=g).to(dtype)
+    probe = torch.zeros(hd)
+    probe[3] = 1.0
+    marks = [0, 37, 63, 64, 300, 449]
+    for i, t in enumerate(marks):
+        k[t, :hd] = 0
+        k[t, i] = 60.0                       # kv head 0: key t answers to a query along axis i
+    _fill_cache(storage, table, slots[0], k, v, KV, hd, page_stride, unit_off, v_off)
+    dev = lambda x, dt=torch.int32: torch.tensor(x, dtype=dt, device=DEV)
+
+    def run(queries, positions, window):
+        q = torch.zeros(len(queries), H * hd)
+        for r, axis in enumerate(queries):
+            q[r, axis] = 60.0                # head 0 (kv head 0)
+            q[r, hd + axis] = 60.0           # head 1 (kv head 0 too)
+        q = q.to(dtype).to(DEV)
+        out = torch.empty(len(queries), H * hd, dtype=dtype, device=DEV)
+        args = (q, out, H, KV, hd, dev(positions), dev([0] * len(queries)), dev(slots), table.to(DEV),
+                storage.to(DEV)[unit_off:], page_stride, v_off)
+        if kernel == "rows" or len(queries) > 1:
+            ops.attention_rows(*args, window=window)
+        else:
+            ops.attention(*args, q_lens=[1], start_pos=positions, window=window)
+        return out.float().cpu()
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    for i, t in enumerate(marks):            # a single row at the last position sees every marked key
+        out = run([i], [length - 1], 0)
+        assert torch.allclose(out[0, :hd], v[t, :hd].float(), atol=tol), (i, t)
+        assert torch.allclose(out[0, hd:2 * hd], v[t, :hd].float(), atol=tol)
+    # causality: a row before the marked key does not see it (its output is an average of many values)
+    out = run([4], [299], 0)
+    assert not torch.allclose(out[0, :hd], v[300, :hd].float(), atol=0.2)
+    # the window: at position 449 with window 150 the key at 300 is the oldest one seen; with 149 it is gone
+    assert torch.allclose(run([4], [449], 150)[0, :hd], v[300, :hd].float(), atol=tol)
+    assert not torch.allclose(run([4], [449], 149)[0, :hd], v[300, :hd].float(), atol=0.2)
+
+
 def test_attention_reference_vectors():
     """layers/gqa_test.go: one cached position gives V for every head of the group (:8-43);
     equal keys give the plain mean, with a window of 2 at position 3 of v = 0,1,2,3 that is 2.5 (:110-136)."""
