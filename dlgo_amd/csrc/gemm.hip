@@ -190,8 +190,9 @@ static const char* dispatch(const void* W, const void* X, void* Y, int N, int Tn
     const long b256 = (long)((N + 255) / 256) * ((Tn + 255) / 256);
     const long big = (long)((N + 127) / 128) * ((Tn + 127) / 128);
     const long mid = (long)((N + 63) / 64) * ((Tn + 63) / 64);
-    // the largest tile that still gives every compute unit a block
-    kind = b256 >= 256 ? 12 : (big >= 256 ? 2 : (mid >= 256 ? 3 : 4));
+    const long tall = (long)((N + 63) / 64) * ((Tn + 127) / 128);
+    // the largest tile that still gives every compute unit a block, and two where one block would leave a SIMD one wave
+    kind = b256 >= 256 ? 12 : (big >= 512 ? 2 : (tall >= 256 ? 14 : (big >= 256 ? 2 : (mid >= 256 ? 3 : 4))));
   }
   if (kind == 13) return launch_tiled<T, 128, 64, 2, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 14) return launch_tiled<T, 64, 128, 2, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
