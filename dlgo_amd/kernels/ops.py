@@ -18,7 +18,8 @@ PAGE = 64   # tokens per cache page; the kernels are compiled with the same numb
 EPI_STORE, EPI_ACCUM_F32, EPI_SWIGLU, EPI_STORE_F32 = 0, 1, 2, 3
 GEMM_AUTO, GEMM_STREAM, GEMM_TILE128, GEMM_TILE64, GEMM_TILE32, GEMM_ROWS16 = 0, 1, 2, 3, 4, 5
 GEMM_TILE256X128, GEMM_TILE256 = 10, 11
-GEMM_FEW_ROWS = 64      # up to this many rows of x the weight-streaming kernels are chosen
+GEMM_FEW_ROWS = 64      # up to this many rows of x the weight-streaming kernels can be chosen
+GEMM_FEW_ROWS_WIDE = 16  # ... and up to this many when the weight has very many rows (there the tiled kernel is faster)
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 
@@ -131,7 +132,8 @@ def gemm(weight: torch.Tensor, x: torch.Tensor, out: torch.Tensor, epilogue: int
     cols = n // 2 if epilogue == EPI_SWIGLU else n
     if tuple(out.shape) != (t, cols):
         raise KernelError(f"gemm: output {tuple(out.shape)}, expected {(t, cols)}")
-    rows_kernel = kind in (GEMM_STREAM, 5, 6, 7, 8, 9) or (kind == GEMM_AUTO and t <= GEMM_FEW_ROWS)
+    rows_kernel = kind in (GEMM_STREAM, 5, 6, 7, 8, 9) or (
+        kind == GEMM_AUTO and (t <= GEMM_FEW_ROWS_WIDE or (t <= GEMM_FEW_ROWS and n < 16384)))
     if rows_kernel:
         fn = _lib("gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),)).dlgo_gemm_rows
         kind = 0 if kind in (GEMM_AUTO, GEMM_ROWS16) else kind
@@ -143,6 +145,7 @@ def gemm(weight: torch.Tensor, x: torch.Tensor, out: torch.Tensor, epilogue: int
 
 
 FUSED_NORM_ROWS = 64   # most rows of the residual stream that gemm_rmsnorm takes
+FUSED_NORM_PAYS = 16   # up to this many rows the fused norm is faster than a norm kernel and a plain product
 
 
 def gemm_rmsnorm(weight: torch.Tensor, x: torch.Tensor, norm_weight: torch.Tensor, eps: float, out: torch.Tensor,

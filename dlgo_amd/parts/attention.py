@@ -95,7 +95,7 @@ class Attention(Mixer):
         self.w_o = stored(tensors["o_proj.weight"], spec["o_proj.weight"], device, dtype)
 
     def fuses_norm(self, norm, ctx) -> bool:
-        return isinstance(norm, RMSNorm) and ctx.n_tokens <= ops.FUSED_NORM_ROWS
+        return isinstance(norm, RMSNorm) and ctx.n_tokens <= ops.FUSED_NORM_PAYS
 
     def forward(self, xn, ctx, unit, residual, owns_cache=True, norm=None) -> None:
         t = xn.shape[0]

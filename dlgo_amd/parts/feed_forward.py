@@ -53,7 +53,7 @@ class GatedFeedForward(FeedForward):
         self.w_down = stored(tensors["down_proj.weight"], spec["down_proj.weight"], device, dtype)
 
     def fuses_norm(self, norm, ctx) -> bool:
-        return isinstance(norm, RMSNorm) and ctx.n_tokens <= ops.FUSED_NORM_ROWS
+        return isinstance(norm, RMSNorm) and ctx.n_tokens <= ops.FUSED_NORM_PAYS
 
     def forward(self, xn, ctx, residual, norm=None) -> None:
         hid = ctx.buffer("feed_forward.hidden", (xn.shape[0], self.inner), ctx.dtype)
