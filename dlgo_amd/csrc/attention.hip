@@ -344,18 +344,60 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
     }
 }
 
+// Rotation of 8 consecutive elements d0..d0+7 of one head vector (bfloat16) at a position whose cos/sin rows are
+// given, as rope_kv.hip does it: split-half pairs (d, d + rot/2) or interleaved pairs (2i, 2i+1); elements from
+// `rot` on are copied.  rot is a multiple of 16, so the 8 elements lie in one half.
+__device__ __forceinline__ uint4 rotated8(const bf16_t* __restrict__ vec, int d0, const float* __restrict__ cs,
+                                          const float* __restrict__ sn, int rot, int interleaved) {
+  const uint4 raw = *(const uint4*)(vec + d0);
+  if (cs == nullptr || d0 >= rot) return raw;
+  float x[8], y[8];
+  Vec16<bf16_t>::load(vec + d0, x);
+  if (interleaved) {
+    const float4 c4 = *(const float4*)(cs + d0 / 2), s4 = *(const float4*)(sn + d0 / 2);
+    const float c[4] = {c4.x, c4.y, c4.z, c4.w}, sv[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      y[2 * i] = x[2 * i] * c[i] - x[2 * i + 1] * sv[i];
+      y[2 * i + 1] = x[2 * i] * sv[i] + x[2 * i + 1] * c[i];
+    }
+  } else {
+    const int half = rot / 2;
+    const bool low = d0 < half;
+    const int i0 = low ? d0 : d0 - half;
+    float p[8], c[8], sv[8];
+    Vec16<bf16_t>::load(vec + (low ? d0 + half : d0 - half), p);
+    *(float4*)c = *(const float4*)(cs + i0);
+    *(float4*)(c + 4) = *(const float4*)(cs + i0 + 4);
+    *(float4*)sv = *(const float4*)(sn + i0);
+    *(float4*)(sv + 4) = *(const float4*)(sn + i0 + 4);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = low ? x[e] * c[e] - p[e] * sv[e] : p[e] * sv[e] + x[e] * c[e];
+  }
+  union { uint4 u; bf16x8_t v; } o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o.v[e] = (__bf16)y[e];
+  return o.u;
+}
+
 // Decode: one token per sequence.  grid (splits, kv heads x head blocks of 16, sequences), NWV waves per block.
 // The pages that hold keys of a sequence's token are dealt evenly to the splits; a block's waves take its pages
 // in turn (wave w: the first page + w, + NWV, ...), all heads of the group at once as the MFMA's 16 columns, and are merged
 // through LDS in wave order.  With one split the block writes the finished rows; else it writes a partial per
 // head, part[((seq * H + head) * n_splits + split) * (HD + 4)] = weighted values [HD], max, sum (base-2
 // exponents), 2 unused, and attn_combine_kernel merges the partials in page order.
-template <int NWV>
+//
+// With cos/sin tables given, q holds the step's unrotated rows [q | k | v]: the query heads are rotated as they are
+// read, and (new_kv) the token's own key and value are taken from the row instead of the cache: the wave that
+// holds the token's page rotates the key, puts key and value into its operands and writes them to the cache for
+// the steps to come (rope_kv.hip's work, without its launch).
+template <int NWV, bool FUSED>
 __global__ __launch_bounds__(NWV* WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, float* __restrict__ part,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, const int32_t* __restrict__ page_table,
-    int max_pages, const bf16_t* __restrict__ cache, long long page_stride, long long v_off, int n_heads, int group,
-    int head_blocks, int n_splits, int window, float scale_log2e) {
+    int max_pages, bf16_t* __restrict__ cache, long long page_stride, long long v_off, int n_heads, int group,
+    int head_blocks, int n_splits, int window, float scale_log2e, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, int rot, int interleaved, int new_kv, int k_col, int v_col) {
   constexpr int HD = HEAD_DIM;
   constexpr int KS = (HD + 31) / 32;   // k steps of K Q^T (16x16x32)
   constexpr int DT = HD / 16;          // 16-row tiles of the output's head dimension
@@ -378,23 +420,21 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_kernel(
   const bool head_ok = j < heads_here;
   const int head = kvh * group + hig;
 
+  const float* cs = cos_t ? cos_t + (size_t)pos * (rot / 2) : nullptr;
+  const float* sn = cos_t ? sin_t + (size_t)pos * (rot / 2) : nullptr;
   uint4 qf[KS];
-  {
-    const bf16_t* qrow = q + (size_t)seq * ldq + (size_t)(head_ok ? head : kvh * group) * HD;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      qf[ks] = (head_ok && ks * 32 + G * 8 < HD) ? *(const uint4*)(qrow + ks * 32 + G * 8) : make_uint4(0, 0, 0, 0);
-  }
+  bool have_q = false;                 // the queries are read (and rotated) behind the first page's loads
   f32x4_t o[DT];
 #pragma unroll
   for (int d = 0; d < DT; ++d) o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
+  const int own = pos % PAGE;          // the token's own row in its page
 
   for (int pg = pg0 + wave; pg <= pg1; pg += NWV) {
     const int page = page_table[(size_t)slot * max_pages + pg];
     if (page < 0) continue;
-    const bf16_t* kpage = cache + (size_t)page * page_stride + (size_t)kvh * PAGE * HD;
-    const bf16_t* vpage = cache + v_off + (size_t)page * page_stride + (size_t)kvh * HD * PAGE;
+    bf16_t* kpage = cache + (size_t)page * page_stride + (size_t)kvh * PAGE * HD;
+    bf16_t* vpage = cache + v_off + (size_t)page * page_stride + (size_t)kvh * HD * PAGE;
     const int key0 = pg * PAGE;
     // every load of the page is issued before the first product
     uint4 kf[4][KS];
@@ -413,6 +453,55 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_kernel(
         vf[u][d][0] = *(const uint2*)(vrow);
         vf[u][d][1] = *(const uint2*)(vrow + 16);
       }
+    if (!have_q) {
+      have_q = true;
+      const bf16_t* qrow = q + (size_t)seq * ldq + (size_t)(head_ok ? head : kvh * group) * HD;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        qf[ks] = !(head_ok && ks * 32 + G * 8 < HD) ? make_uint4(0, 0, 0, 0)
+                 : (FUSED ? rotated8(qrow, ks * 32 + G * 8, cs, sn, rot, interleaved) : *(const uint4*)(qrow + ks * 32 + G * 8));
+    }
+    if (FUSED && new_kv && pg == last_pg) {
+      // the token's own key and value come from the step's row, not from the cache; head block 0 stores them
+      const bf16_t* row = q + (size_t)seq * ldq;
+      const bf16_t* krow_new = row + k_col + (size_t)kvh * HD;
+      const bf16_t* vrow_new = row + v_col + (size_t)kvh * HD;
+      if (j == own % 16) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          if (t == own / 16) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+              if (ks * 32 + G * 8 < HD) {
+                kf[t][ks] = rotated8(krow_new, ks * 32 + G * 8, cs, sn, rot, interleaved);
+                if (hb == 0) *(uint4*)(kpage + (size_t)own * HD + ks * 32 + G * 8) = kf[t][ks];
+              }
+          }
+      }
+      const int rr = own % 32;
+      if (G == (rr % 16) / 4) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+          if (u == own / 32) {
+#pragma unroll
+            for (int d = 0; d < DT; ++d) {
+              const bf16_t val = vrow_new[d * 16 + j];
+              const int e = rr % 4;
+#pragma unroll
+              for (int h = 0; h < 2; ++h)
+                if (h == rr / 16) {
+                  uint32_t lo32 = vf[u][d][h].x, hi32 = vf[u][d][h].y;
+                  if (e == 0) lo32 = (lo32 & 0xffff0000u) | val;
+                  else if (e == 1) lo32 = (lo32 & 0x0000ffffu) | ((uint32_t)val << 16);
+                  else if (e == 2) hi32 = (hi32 & 0xffff0000u) | val;
+                  else hi32 = (hi32 & 0x0000ffffu) | ((uint32_t)val << 16);
+                  vf[u][d][h] = make_uint2(lo32, hi32);
+                }
+              if (hb == 0) vpage[(size_t)(d * 16 + j) * PAGE + own] = val;
+            }
+          }
+      }
+    }
     f32x4_t s[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
@@ -614,13 +703,18 @@ extern "C" const char* dlgo_attention_prefill(const void* q, int ldq, void* out,
   return nullptr;
 }
 
-// bfloat16, one row per sequence.  max_pages_used bounds the pages of any sequence of the step (a recorded
+// bfloat16, one row per sequence.  With cos_t/sin_t ([table_rows, rot/2]) the rows q are unrotated and are rotated
+// here; with new_kv they are [q | k | v] rows whose key (rotated) and value enter the product and the cache here.
+// max_pages_used bounds the pages of any sequence of the step (a recorded
 // launch passes the context's bound).  part: float32 scratch, used when the pages are split over several
 // blocks: n_seq * n_heads * n_splits * (hd + 4) with n_splits = dlgo_attention_decode_splits(...).
-static void decode_plan(int n_pairs, int group, int max_pages_used, int* nwv, int* n_splits) {
+static void decode_plan(int n_pairs, int group, int max_pages_used, bool fused, int* nwv, int* n_splits) {
   const int heads_here = group < 16 ? group : 16;
   const int per_wave = heads_here * (HEAD_DIM + 2) * 4;      // bytes of LDS a wave needs for the merge
-  int w = 16;
+  // the registers a wave needs grow with the head size (a page's keys and values are held at once), and a block
+  // of w waves leaves each 2048 / w of them; the variant that rotates needs about a third more
+  int w = HEAD_DIM <= 64 ? 16 : (HEAD_DIM <= 128 ? 8 : 4);
+  if (fused) w >>= 1;
   while (w > 1 && w * per_wave > 60 * 1024) w >>= 1;
   // enough blocks to fill the chip: with few (sequence, kv head) pairs each pair's pages go to several blocks
   int splits = n_pairs >= 256 ? 1 : (256 + n_pairs - 1) / n_pairs;
@@ -631,29 +725,35 @@ static void decode_plan(int n_pairs, int group, int max_pages_used, int* nwv, in
   *n_splits = splits;
 }
 
-extern "C" int dlgo_attention_decode_splits(int n_seq, int n_heads, int n_kv, int max_pages_used) {
+extern "C" int dlgo_attention_decode_splits(int n_seq, int n_heads, int n_kv, int max_pages_used, int fused) {
   int nwv, n_splits;
   const int group = n_heads / n_kv;
-  decode_plan(n_seq * n_kv * ((group + 15) / 16), group, max_pages_used, &nwv, &n_splits);
+  decode_plan(n_seq * n_kv * ((group + 15) / 16), group, max_pages_used, fused != 0, &nwv, &n_splits);
   return n_splits;
 }
 
 extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, int ldo, float* part, long long part_elems,
                                              int n_seq, int n_heads, int n_kv, int head_dim, const int32_t* positions,
                                              const int32_t* slots, const int32_t* page_table, int max_pages,
-                                             int max_pages_used, const void* cache, long long page_stride, long long v_off,
-                                             int window, float scale, hipStream_t stream) {
+                                             int max_pages_used, void* cache, long long page_stride, long long v_off,
+                                             int window, float scale, const float* cos_t, const float* sin_t, int table_rows,
+                                             int rot, int interleaved, int new_kv, hipStream_t stream) {
   DLGO_REQUIRE(head_dim == HEAD_DIM, "attention: this library is built for head size %d, got %d", HEAD_DIM, head_dim);
   DLGO_REQUIRE(HEAD_DIM <= 256, "attention: the split kernel takes head sizes up to 256");
   DLGO_REQUIRE(n_seq >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention: bad sizes");
   DLGO_REQUIRE(max_pages_used >= 1 && max_pages_used <= max_pages, "attention: bad bound on the pages of a sequence");
+  DLGO_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attention: cos and sin tables come together");
+  DLGO_REQUIRE(cos_t == nullptr || (rot % 16 == 0 && rot > 0 && rot <= head_dim && table_rows > 0),
+               "attention: the fused rotation takes a rotated width that is a multiple of 16, got %d", rot);
+  DLGO_REQUIRE(!new_kv || ldq >= (n_heads + 2 * n_kv) * head_dim, "attention: rows with new keys and values hold [q | k | v]");
   DLGO_REQUIRE(ldq >= n_heads * head_dim && ldo >= n_heads * head_dim && ldq % 8 == 0, "attention: row strides");
   DLGO_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)cache & 15) == 0 && page_stride % 8 == 0 && v_off % 8 == 0,
                "attention: operands must be 16-byte aligned");
   const int group = n_heads / n_kv;
   const int head_blocks = (group + 15) / 16;
   int nwv, n_splits;
-  decode_plan(n_seq * n_kv * head_blocks, group, max_pages_used, &nwv, &n_splits);
+  const bool fused = cos_t != nullptr || new_kv;
+  decode_plan(n_seq * n_kv * head_blocks, group, max_pages_used, fused, &nwv, &n_splits);
   DLGO_REQUIRE(n_splits == 1 || (part && part_elems >= (long long)n_seq * n_heads * n_splits * (HEAD_DIM + 4)),
                "attention: scratch for partial results too small");
   DLGO_REQUIRE((long long)n_kv * head_blocks <= 65535 && n_seq <= 65535 && n_heads <= 65535, "attention: grid too large");
@@ -661,15 +761,23 @@ extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, 
   const int heads_here = group < 16 ? group : 16;
   const size_t smem = (size_t)nwv * heads_here * (HEAD_DIM + 2) * 4;
   dim3 grid(n_splits, n_kv * head_blocks, n_seq);
-#define DECODE_GO(W_)                                                                                                          \
-  hipLaunchKernelGGL(attn_decode_kernel<W_>, grid, dim3(W_ * WAVE), smem, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo, part, \
-                     positions, slots, page_table, max_pages, (const bf16_t*)cache, page_stride, v_off, n_heads, group,      \
-                     head_blocks, n_splits, window, scale * LOG2E)
-  if (nwv == 16) DECODE_GO(16);
-  else if (nwv == 8) DECODE_GO(8);
-  else if (nwv == 4) DECODE_GO(4);
-  else if (nwv == 2) DECODE_GO(2);
-  else DECODE_GO(1);
+#define DECODE_GO(W_, F_)                                                                                                      \
+  hipLaunchKernelGGL((attn_decode_kernel<W_, F_>), grid, dim3(W_ * WAVE), smem, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo,  \
+                     part, positions, slots, page_table, max_pages, (bf16_t*)cache, page_stride, v_off, n_heads, group,        \
+                     head_blocks, n_splits, window, scale * LOG2E, cos_t, sin_t, rot, interleaved, new_kv,                    \
+                     n_heads * head_dim, (n_heads + n_kv) * head_dim)
+  if (fused) {
+    if (nwv == 8) DECODE_GO(8, true);
+    else if (nwv == 4) DECODE_GO(4, true);
+    else if (nwv == 2) DECODE_GO(2, true);
+    else DECODE_GO(1, true);
+  } else {
+    if (nwv == 16) DECODE_GO(16, false);
+    else if (nwv == 8) DECODE_GO(8, false);
+    else if (nwv == 4) DECODE_GO(4, false);
+    else if (nwv == 2) DECODE_GO(2, false);
+    else DECODE_GO(1, false);
+  }
 #undef DECODE_GO
   DLGO_LAUNCH_CHECK("attention_decode");
   if (n_splits > 1) {

@@ -228,12 +228,21 @@ def attention_rows(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, 
     return out
 
 
+def attention_fuses_rotation(dtype: torch.dtype, head_dim: int, group: int, max_q_len: int, rot_width: int,
+                             n_seq: int = 1) -> bool:
+    """True if attention() should rotate the queries and take in the new keys and values itself for such a step:
+    one row per sequence, bfloat16, a rotated width that is a multiple of 16 or no rotation at all, and few enough
+    sequences that a kernel launch costs more than the rotation repeated in every wave."""
+    return (dtype == torch.bfloat16 and head_dim <= 256 and group <= 128 and max_q_len == 1 and rot_width % 16 == 0
+            and n_seq <= 32)
+
+
 def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, positions: torch.Tensor,
               tok_seq: torch.Tensor, slots: torch.Tensor, page_table: torch.Tensor, cache: torch.Tensor, page_stride: int,
               v_off: int, q_lens: Sequence[int], start_pos: Sequence[int], window: int = 0,
               scale: Optional[float] = None, cu_q: Optional[torch.Tensor] = None,
               start_pos_dev: Optional[torch.Tensor] = None, scratch=None,
-              max_pages_used: Optional[int] = None, kernel: str = "auto") -> torch.Tensor:
+              max_pages_used: Optional[int] = None, kernel: str = "auto", rotation=None, new_kv: bool = False) -> torch.Tensor:
     """Attention of a step's query rows over the cache, with the kernel chosen by the step's shape and dtype.
 
     q_lens, start_pos: per sequence, on the host (rows of the step, and the length before it).  cu_q and
@@ -241,6 +250,9 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
     float32 buffer of at least n elements (partials of long sequences in decode).  max_pages_used bounds the pages any sequence
     of the step holds (default: from q_lens and start_pos; a captured step passes the context's bound).
     kernel: "auto", "rows", "tiled" (prefill) or "split" (decode).  All kernels compute the same thing.
+    rotation = (cos, sin, width, interleaved) and new_kv: only where attention_fuses_rotation() says so; then q
+    holds the step's unrotated [q | k | v] rows, which the kernel rotates, and with new_kv it also takes each
+    token's own key and value from its row and writes them to the cache (what rope_kv() does otherwise).
     """
     n_seq = len(q_lens)
     max_q = int(max(q_lens)) if n_seq else 0
@@ -248,6 +260,8 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
     fast_ok = q.dtype == torch.bfloat16 and head_dim <= 256 and group <= 128
     if kernel == "auto":
         kernel = "rows" if not fast_ok else ("split" if max_q == 1 else "tiled")
+    if (rotation is not None or new_kv) and not (kernel == "split" and fast_ok and max_q == 1):
+        raise KernelError("attention: only the split kernel rotates and stores by itself")
     if kernel == "rows" or n_seq == 0:
         return attention_rows(q, out, n_heads, n_kv, head_dim, positions, tok_seq, slots, page_table, cache, page_stride,
                               v_off, window, scale)
@@ -273,8 +287,16 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
         if max_pages_used is None:
             max_pages_used = (int(max(start_pos)) + 1 + PAGE - 1) // PAGE
         max_pages_used = max(1, min(max_pages_used, max_pages))
+        cos = sin = None
+        rot_width, interleaved = 0, False
+        if rotation is not None:
+            cos, sin, rot_width, interleaved = rotation
+            _need(cos, "cos table", torch.float32, 2)
+            _need(sin, "sin table", torch.float32, 2)
+            if cos.shape != sin.shape or cos.shape[1] != rot_width // 2 or not cos.is_contiguous() or not sin.is_contiguous():
+                raise KernelError(f"attention: tables {tuple(cos.shape)} do not fit a rotated width of {rot_width}")
         lib.dlgo_attention_decode_splits.restype = ctypes.c_int
-        n_splits = lib.dlgo_attention_decode_splits(n_seq, n_heads, n_kv, max_pages_used)
+        n_splits = lib.dlgo_attention_decode_splits(n_seq, n_heads, n_kv, max_pages_used, int(rotation is not None or new_kv))
         part = None
         if n_splits > 1:
             need = n_seq * n_heads * n_splits * (head_dim + 4)
@@ -284,7 +306,8 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
                                          ctypes.c_longlong(part.numel() if part is not None else 0), n_seq, n_heads, n_kv,
                                          head_dim, _ptr(positions), _ptr(slots), _ptr(page_table), max_pages, max_pages_used,
                                          _ptr(cache), ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(window),
-                                         ctypes.c_float(scale), _stream()))
+                                         ctypes.c_float(scale), _ptr(cos), _ptr(sin), cos.shape[0] if cos is not None else 0,
+                                         int(rot_width), int(interleaved), int(new_kv), _stream()))
         return out
     if kernel != "tiled":
         raise KernelError(f"attention: unknown kernel {kernel!r}")

@@ -108,18 +108,23 @@ class Attention(Mixer):
             ops.gemm(self.w_qkv[:cols], xn, qkv[:, :cols])
         kv = ctx.cache.kv_view(unit)
         rot = self.position.rotation()
-        ops.rope_kv(qkv, self.n_heads, n_kv, self.head_dim, rot.width if rot else 0, rot.interleaved if rot else False,
-                    rot.cos if rot else None, rot.sin if rot else None, ctx.positions,
-                    ctx.tok_seq, ctx.slots, kv.page_table, kv.cache, kv.page_stride, kv.v_off, write_kv=owns_cache)
+        # a step of single tokens: the attention kernel rotates and stores by itself; else a kernel of its own does
+        fused = ops.attention_fuses_rotation(ctx.dtype, self.head_dim, self.n_heads // self.n_kv_heads, ctx.max_q_len,
+                                             rot.width if rot else 0, ctx.n_seq)
+        if not fused:
+            ops.rope_kv(qkv, self.n_heads, n_kv, self.head_dim, rot.width if rot else 0, rot.interleaved if rot else False,
+                        rot.cos if rot else None, rot.sin if rot else None, ctx.positions,
+                        ctx.tok_seq, ctx.slots, kv.page_table, kv.cache, kv.page_stride, kv.v_off, write_kv=owns_cache)
         out = ctx.buffer("attention.out", (t, self.q_dim), ctx.dtype)
-        self.attend(qkv, out, ctx, kv)
+        self.attend(qkv, out, ctx, kv, rotation=(rot.cos, rot.sin, rot.width, rot.interleaved) if fused and rot else None,
+                    new_kv=fused and owns_cache)
         ops.gemm(self.w_o, out, residual, ops.EPI_ACCUM_F32)
 
-    def attend(self, q, out, ctx, kv) -> None:
+    def attend(self, q, out, ctx, kv, rotation=None, new_kv=False) -> None:
         """Attention of the step's (rotated) query rows over the cache; the kernel is chosen by the
         step's shape and the run dtype, the arithmetic is the same."""
         ops.attention(q, out, self.n_heads, self.n_kv_heads, self.head_dim, ctx.positions, ctx.tok_seq, ctx.slots,
                       kv.page_table, kv.cache, kv.page_stride, kv.v_off, ctx.host["q_lens"], ctx.host["start_pos"],
                       window=self.window or 0, scale=self.scale, cu_q=ctx.cu_q, start_pos_dev=ctx.start_pos,
                       scratch=lambda n: ctx.scratch("attention.partials", n, torch.float32),
-                      max_pages_used=ctx.max_pages_used)
+                      max_pages_used=ctx.max_pages_used, rotation=rotation, new_kv=new_kv)

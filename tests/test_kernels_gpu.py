@@ -387,6 +387,50 @@ def test_attention_finds_a_far_key_and_respects_the_window_edge(dtype, _, rel, k
     assert not torch.allclose(run([4], [449], 149)[0, :hd], v[300, :hd].float(), atol=0.2)
 
 
+@pytest.mark.parametrize("H,KV,hd,rot,inter,window", [(4, 2, 16, 16, False, 0), (32, 8, 64, 64, False, 0), (6, 3, 48, 32, True, 0),
+                                                       (40, 2, 32, 32, False, 0), (8, 8, 128, 128, True, 50), (4, 1, 80, 0, False, 0)])
+def test_decode_attention_that_rotates_and_stores_by_itself(H, KV, hd, rot, inter, window):
+    """One row per sequence: the split kernel given unrotated [q | k | v] rows against the two-kernel way
+    (rotate and store, then attend): the same output, the same cache afterwards."""
+    ops = _ops()
+    from dlgo_amd.parts import rotary_frequencies
+    dtype = torch.bfloat16
+    lens = [70, 3, 129, 64, 65, 1, 2000]
+    table, slots, storage, page_stride, unit_off, v_off = _paged_setup(dtype, lens, KV, hd, seed=rot + hd)
+    g = torch.Generator().manual_seed(H + hd)
+    for i, n in enumerate(lens):                       # what the sequences hold before this step
+        if n > 1:
+            k = torch.randn(n - 1, KV * hd, generator=g).to(dtype)
+            v = torch.randn(n - 1, KV * hd, generator=g).to(dtype)
+            _fill_cache(storage, table, slots[i], k, v, KV, hd, page_stride, unit_off, v_off)
+    storage = torch.nan_to_num(storage.float(), nan=7.0).to(dtype)      # so that the caches can be compared
+    qkv = torch.randn(len(lens), (H + 2 * KV) * hd, generator=g).to(dtype)
+    cos = sin = None
+    if rot:
+        ang = np.arange(2048)[:, None] * rotary_frequencies(rot, 10000.0)[None]
+        cos, sin = (torch.from_numpy(f(ang).astype(np.float32)).to(DEV) for f in (np.cos, np.sin))
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    positions, tok_seq, dslots = dev([n - 1 for n in lens]), dev(list(range(len(lens)))), dev(slots)
+    outs, caches = [], []
+    for fused in (False, True):
+        store = storage.clone().to(DEV)
+        rows = qkv.clone().to(DEV)
+        out = torch.empty(len(lens), H * hd, dtype=dtype, device=DEV)
+        common = dict(q_lens=[1] * len(lens), start_pos=[n - 1 for n in lens], window=window, kernel="split")
+        if fused:
+            ops.attention(rows, out, H, KV, hd, positions, tok_seq, dslots, table.to(DEV), store[unit_off:], page_stride, v_off,
+                          rotation=(cos, sin, rot, inter) if rot else None, new_kv=True, **common)
+        else:
+            ops.rope_kv(rows, H, KV, hd, rot, inter, cos, sin, positions, tok_seq, dslots, table.to(DEV), store[unit_off:],
+                        page_stride, v_off)
+            ops.attention(rows, out, H, KV, hd, positions, tok_seq, dslots, table.to(DEV), store[unit_off:], page_stride, v_off,
+                          **common)
+        outs.append(out.float().cpu())
+        caches.append(store.cpu())
+    assert torch.equal(caches[0], caches[1])
+    assert torch.allclose(outs[0], outs[1], atol=1e-6, rtol=0)
+
+
 def test_attention_reference_vectors():
     """layers/gqa_test.go: one cached position gives V for every head of the group (:8-43);
     equal keys give the plain mean, with a window of 2 at position 3 of v = 0,1,2,3 that is 2.5 (:110-136)."""
