@@ -70,6 +70,106 @@ __global__ __launch_bounds__(WAVE) void rope_kv_kernel(T* __restrict__ qkv, int 
     for (int i = rot + lane; i < hd; i += WAVE) kdst[i] = src[i];
 }
 
+// The same work in 16-byte pieces, one thread per piece of a token's [q | k | v] row, for rotated widths whose halves
+// are whole pieces (every model of a usual shape): a piece is read once, rotated against its partner piece, and
+// written once (queries in place, keys as one 16-byte store, values scattered into their transposed page).
+template <typename T> struct Piece;
+template <> struct Piece<float> {
+  static constexpr int E = 4;
+  static __device__ __forceinline__ void load(const float* p, float* f) { *(float4*)f = *(const float4*)p; }
+  static __device__ __forceinline__ void store(float* p, const float* f) { *(float4*)p = *(const float4*)f; }
+};
+template <> struct Piece<bf16_t> {
+  static constexpr int E = 8;
+  static __device__ __forceinline__ void load(const bf16_t* p, float* f) {
+    const uint4 u = *(const uint4*)p;
+    f[0] = __uint_as_float(u.x << 16); f[1] = __uint_as_float(u.x & 0xffff0000u);
+    f[2] = __uint_as_float(u.y << 16); f[3] = __uint_as_float(u.y & 0xffff0000u);
+    f[4] = __uint_as_float(u.z << 16); f[5] = __uint_as_float(u.z & 0xffff0000u);
+    f[6] = __uint_as_float(u.w << 16); f[7] = __uint_as_float(u.w & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float* f) {
+    uint4 u;
+    u.x = (uint32_t)f32_to_bf16(f[0]) | ((uint32_t)f32_to_bf16(f[1]) << 16);
+    u.y = (uint32_t)f32_to_bf16(f[2]) | ((uint32_t)f32_to_bf16(f[3]) << 16);
+    u.z = (uint32_t)f32_to_bf16(f[4]) | ((uint32_t)f32_to_bf16(f[5]) << 16);
+    u.w = (uint32_t)f32_to_bf16(f[6]) | ((uint32_t)f32_to_bf16(f[7]) << 16);
+    *(uint4*)p = u;
+  }
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_pieces_kernel(T* __restrict__ qkv, int ld, int n_tokens, int n_heads, int n_kv, int hd,
+                                                             int rot, int interleaved, const float* __restrict__ cos_t,
+                                                             const float* __restrict__ sin_t,
+                                                             const int32_t* __restrict__ positions,
+                                                             const int32_t* __restrict__ tok_seq,
+                                                             const int32_t* __restrict__ slots,
+                                                             const int32_t* __restrict__ page_table, int max_pages,
+                                                             T* __restrict__ cache, long long page_stride, long long v_off,
+                                                             int write_kv) {
+  constexpr int E = Piece<T>::E;
+  const int per_head = hd / E;
+  const int heads = n_heads + (write_kv ? 2 * n_kv : 0);
+  const int per_token = heads * per_head;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long long)n_tokens * per_token) return;
+  const int t = (int)(idx / per_token), c = (int)(idx % per_token);
+  const int head = c / per_head, d0 = (c % per_head) * E;
+  const int pos = positions[t];
+  T* src = qkv + (size_t)t * ld + (size_t)head * hd;
+  const bool is_q = head < n_heads, is_k = !is_q && head < n_heads + n_kv;
+  const bool rotates = (is_q || is_k) && cos_t && d0 < rot;
+  const int half = rot / 2;
+  if (rotates && !interleaved && d0 >= half) return;   // done by the thread of the partner piece
+  // where the (rotated) pieces go
+  T* dst = src;            // queries: in place
+  T* vcol = nullptr;       // values: a column of the transposed page
+  if (!is_q) {
+    const int slot = slots[tok_seq[t]];
+    const int page = page_table[(size_t)slot * max_pages + pos / PAGE];
+    if (page < 0) return;
+    const int in_page = pos % PAGE;
+    if (is_k) dst = cache + (size_t)page * page_stride + ((size_t)(head - n_heads) * PAGE + in_page) * hd;
+    else vcol = cache + v_off + (size_t)page * page_stride + (size_t)(head - n_heads - n_kv) * hd * PAGE + in_page;
+  }
+  float x[E];
+  Piece<T>::load(src + d0, x);
+  if (vcol) {
+#pragma unroll
+    for (int e = 0; e < E; ++e) Elem<T>::store(vcol + (size_t)(d0 + e) * PAGE, x[e]);
+    return;
+  }
+  if (!rotates) {
+    if (!is_q) Piece<T>::store(dst + d0, x);      // the part of a key beyond the rotated width is copied
+    return;
+  }
+  const float* cs = cos_t + (size_t)pos * half;
+  const float* sn = sin_t + (size_t)pos * half;
+  if (interleaved) {
+    float y[E];
+#pragma unroll
+    for (int i = 0; i < E / 2; ++i) {
+      const float c_ = cs[d0 / 2 + i], s_ = sn[d0 / 2 + i];
+      y[2 * i] = x[2 * i] * c_ - x[2 * i + 1] * s_;
+      y[2 * i + 1] = x[2 * i] * s_ + x[2 * i + 1] * c_;
+    }
+    Piece<T>::store(dst + d0, y);
+  } else {
+    // this thread owns the pieces at d0 and d0 + half: both are read before either is written
+    float p[E], y0[E], y1[E];
+    Piece<T>::load(src + d0 + half, p);
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const float c_ = cs[d0 + e], s_ = sn[d0 + e];
+      y0[e] = x[e] * c_ - p[e] * s_;
+      y1[e] = x[e] * s_ + p[e] * c_;
+    }
+    Piece<T>::store(dst + d0, y0);
+    Piece<T>::store(dst + d0 + half, y1);
+  }
+}
+
 extern "C" const char* dlgo_rope_kv(void* qkv, int dtype, int n_tokens, int ld, int n_heads, int n_kv, int hd, int rot,
                                     int interleaved, const float* cos_t, const float* sin_t, int table_rows,
                                     const int32_t* positions, const int32_t* tok_seq, const int32_t* slots,
@@ -82,6 +182,25 @@ extern "C" const char* dlgo_rope_kv(void* qkv, int dtype, int n_tokens, int ld, 
   DLGO_REQUIRE(cos_t == nullptr || table_rows > 0, "rope_kv: empty rotation table");
   DLGO_REQUIRE(!write_kv || (cache && page_table && slots && tok_seq && max_pages > 0), "rope_kv: cache arguments missing");
   if (n_tokens == 0) return nullptr;
+  const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
+  const bool pieces = hd % epc == 0 && rot % (2 * epc) == 0 && ld % epc == 0 && ((uintptr_t)qkv & 15) == 0 &&
+                      (!write_kv || (((uintptr_t)cache & 15) == 0 && page_stride % epc == 0 && v_off % epc == 0));
+  if (pieces) {
+    const long long items = (long long)n_tokens * (n_heads + (write_kv ? 2 * n_kv : 0)) * (hd / epc);
+    dim3 g((unsigned)((items + 255) / 256));
+    if (dtype == DLGO_DTYPE_F32)
+      hipLaunchKernelGGL(rope_kv_pieces_kernel<float>, g, dim3(256), 0, stream, (float*)qkv, ld, n_tokens, n_heads, n_kv, hd, rot,
+                         interleaved, cos_t, sin_t, positions, tok_seq, slots, page_table, max_pages, (float*)cache, page_stride,
+                         v_off, write_kv);
+    else if (dtype == DLGO_DTYPE_BF16)
+      hipLaunchKernelGGL(rope_kv_pieces_kernel<bf16_t>, g, dim3(256), 0, stream, (bf16_t*)qkv, ld, n_tokens, n_heads, n_kv, hd, rot,
+                         interleaved, cos_t, sin_t, positions, tok_seq, slots, page_table, max_pages, (bf16_t*)cache, page_stride,
+                         v_off, write_kv);
+    else
+      DLGO_FAIL("rope_kv: unknown dtype code %d", dtype);
+    DLGO_LAUNCH_CHECK("rope_kv");
+    return nullptr;
+  }
   dim3 grid(n_tokens, n_heads + 2 * n_kv);
   if (dtype == DLGO_DTYPE_F32)
     hipLaunchKernelGGL(rope_kv_kernel<float>, grid, dim3(WAVE), 0, stream, (float*)qkv, ld, n_heads, n_kv, hd, rot, interleaved,

@@ -213,7 +213,7 @@ def _rope_ref(v, pos, freqs, interleaved):
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
 @pytest.mark.parametrize("H,KV,hd,rot,inter", [(4, 2, 16, 16, False), (6, 3, 48, 48, True), (8, 1, 128, 64, False),
-                                               (2, 2, 32, 32, True)])
+                                               (2, 2, 32, 32, True), (4, 2, 16, 8, False), (3, 1, 32, 12, True)])
 def test_rope_kv_write(dtype, _, rel, H, KV, hd, rot, inter):
     ops = _ops()
     from dlgo_amd.cache import PAGE
