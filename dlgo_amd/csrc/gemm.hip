@@ -10,6 +10,10 @@
 // true float32 product with float32 accumulation.  Blocks are numbered so that the blocks one XCD runs share tiles
 // in that XCD's L2.
 //
+// gemm_direct_kernel: the same product for large shapes whose K is a whole number of 128-byte pieces.  Tiles go from
+// memory straight into LDS (global_load_lds_dwordx4), without registers in between and two to three tiles ahead of
+// the one being multiplied, so that neither the wait for memory nor the copy into LDS stands between the MFMAs.
+//
 // Every reduction order is a function of k alone: a row of Y never depends on the other rows of the step.
 #include "gemm_common.h"
 
@@ -163,6 +167,171 @@ __global__ __launch_bounds__(WN* WT* WAVE) void gemm_kernel(const T* __restrict_
   }
 }
 
+// 16 bytes per lane from base + voff into LDS at lds_base + lane * 16; lds_base is the same for the whole wave (it
+// travels in M0).  Written as assembly so that the compiler does not make every later LDS read wait for these loads;
+// wait_loads and the barrier below order them instead.
+static __device__ __forceinline__ void load_to_lds(const void* base, uint32_t voff, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(base) : "memory");
+}
+template <int N> static __device__ __forceinline__ void wait_loads() {   // until at most N of this wave's loads are in flight
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+template <typename T, int BN, int BT, int WN, int WT, int NS, int EPI>
+__global__ __launch_bounds__(WN* WT* WAVE) void gemm_direct_kernel(const T* __restrict__ W, const T* __restrict__ X,
+                                                                     void* __restrict__ Y, int N, int Tn, int K, int ldw, int ldx,
+                                                                     int ldy, int tiles_t) {
+  constexpr int NW = WN * WT;
+  constexpr int EPC = 16 / sizeof(T);
+  constexpr int BK = 128 / sizeof(T);
+  constexpr int MI = BN / WN / 32, NJ = BT / WT / 32;
+  constexpr int LA = BN / 8 / NW, LB = BT / 8 / NW;     // loads (8 rows of 128 bytes each) per wave and stage
+  constexpr int STAGE = (BN + BT) * 128;
+  static_assert(BN % (8 * NW) == 0 && BT % (8 * NW) == 0, "tile does not divide over the waves");
+  static_assert((NS - 2) * (LA + LB) < 64, "too many loads in flight for the counter");
+  extern __shared__ __attribute__((aligned(16))) char lds[];   // NS stages of (BN + BT) rows of 128 bytes
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wn = wave % WN, wt = wave / WN;
+  int bid = blockIdx.x;
+  const int nb = gridDim.x;
+  if ((nb & 7) == 0) bid = (bid & 7) * (nb >> 3) + (bid >> 3);     // as in gemm_kernel
+  const int tile_t = bid % tiles_t, tile_n = bid / tiles_t;
+  const int n0 = tile_n * BN, t0 = tile_t * BT;
+
+  f32x16_t acc[MI][NJ];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  // A load writes 1024 consecutive bytes of LDS: 8 rows without padding.  Row r therefore keeps its 16-byte piece p
+  // at slot p ^ ((r >> 1) & 7), which spreads the 16 rows that a quarter of a wave reads at once over all banks; the
+  // lane that fills slot s of row r fetches piece s ^ ((r >> 1) & 7).  Rows beyond the matrix repeat its last row.
+  uint32_t offA[LA], offB[LB];
+#pragma unroll
+  for (int q = 0; q < LA; ++q) {
+    const int r = (wave * LA + q) * 8 + (lane >> 3);
+    const int p = (lane & 7) ^ ((r >> 1) & 7);
+    int n = n0 + r;
+    n = n < N ? n : N - 1;
+    offA[q] = (uint32_t)(n - n0) * (uint32_t)ldw * (uint32_t)sizeof(T) + (uint32_t)p * 16u;
+  }
+#pragma unroll
+  for (int q = 0; q < LB; ++q) {
+    const int r = (wave * LB + q) * 8 + (lane >> 3);
+    const int p = (lane & 7) ^ ((r >> 1) & 7);
+    int t = t0 + r;
+    t = t < Tn ? t : Tn - 1;
+    offB[q] = (uint32_t)(t - t0) * (uint32_t)ldx * (uint32_t)sizeof(T) + (uint32_t)p * 16u;
+  }
+  const char* baseA = (const char*)(W + (size_t)n0 * ldw);
+  const char* baseB = (const char*)(X + (size_t)t0 * ldx);
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
+  const uint32_t ldsA = __builtin_amdgcn_readfirstlane(lds0 + wave * LA * 1024);
+  const uint32_t ldsB = __builtin_amdgcn_readfirstlane(lds0 + BN * 128 + wave * LB * 1024);
+
+  auto issue = [&](int kt, int stage) {
+    const char* a = baseA + (size_t)kt * 128;
+    const char* b = baseB + (size_t)kt * 128;
+#pragma unroll
+    for (int q = 0; q < LA; ++q) load_to_lds(a, offA[q], ldsA + stage * STAGE + q * 1024);
+#pragma unroll
+    for (int q = 0; q < LB; ++q) load_to_lds(b, offB[q], ldsB + stage * STAGE + q * 1024);
+  };
+
+  const int nk = K / BK;
+#pragma unroll
+  for (int s = 0; s < NS - 1; ++s)
+    if (s < nk) issue(s, s);
+
+  // operands: row lane%32 of a 32-row tile, pieces 2*slab + lane/32, found at slot (lane/32 ^ x) ^ 2*slab
+  const int s0 = (lane >> 5) ^ ((lane >> 1) & 7);
+  const int rowA = (wn * (BN / WN) + (lane & 31)) * 128, rowB = BN * 128 + (wt * (BT / WT) + (lane & 31)) * 128;
+  int stage = 0;
+  for (int kt = 0; kt < nk; ++kt) {
+    if (kt + NS - 2 < nk) wait_loads<(NS - 2) * (LA + LB)>();    // tile kt has arrived; the tiles after it may be on the way
+    else wait_loads<0>();
+    __syncthreads();        // ... for every wave, and every wave is done with tile kt-1, whose stage is filled next
+    if (kt + NS - 1 < nk) {
+      int ws = stage + NS - 1;
+      ws = ws >= NS ? ws - NS : ws;
+      issue(kt + NS - 1, ws);
+    }
+    const char* pa = lds + stage * STAGE + rowA;
+    const char* pb = lds + stage * STAGE + rowB;
+    uint4 a[2][MI], b[2][NJ];
+#pragma unroll
+    for (int i = 0; i < MI; ++i) a[0][i] = *(const uint4*)(pa + i * 32 * 128 + s0 * 16);
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) b[0][j] = *(const uint4*)(pb + j * 32 * 128 + s0 * 16);
+#pragma unroll
+    for (int slab = 0; slab < 4; ++slab) {
+      const int c = slab & 1, nx = c ^ 1;
+      if (slab < 3) {
+        const int so = (s0 ^ (2 * (slab + 1))) * 16;
+#pragma unroll
+        for (int i = 0; i < MI; ++i) a[nx][i] = *(const uint4*)(pa + i * 32 * 128 + so);
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) b[nx][j] = *(const uint4*)(pb + j * 32 * 128 + so);
+      }
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NJ; ++j) Mma<T>::run(a[c][i], b[c][j], acc[i][j]);
+    }
+    stage = stage + 1 == NS ? 0 : stage + 1;
+  }
+  __syncthreads();      // the stages are free: each wave turns its tiles through a piece of them, as in gemm_kernel
+
+  float* turn = (float*)(lds + wave * (32 * GEMM_ROWB));
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        *(float4*)(turn + (lane & 31) * (GEMM_ROWB / 4) + 8 * q + 4 * (lane >> 5)) =
+            make_float4(acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        const int tt = p * 8 + (lane >> 3), nn = (lane & 7) * 4;
+        const float4 v = *(const float4*)(turn + tt * (GEMM_ROWB / 4) + nn);
+        const int t = t0 + wt * (BT / WT) + j * 32 + tt;
+        const int n = n0 + wn * (BN / WN) + i * 32 + nn;
+        if (t < Tn) epilogue4<T, EPI>(Y, ldy, N, t, n, v.x, v.y, v.z, v.w);
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
+  }
+}
+
+template <typename T, int BN, int BT, int WN, int WT, int NS, int EPI>
+static const char* launch_direct(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy,
+                                 hipStream_t stream) {
+  const int tiles_t = (Tn + BT - 1) / BT, tiles_n = (N + BN - 1) / BN;
+  constexpr int smem = NS * (BN + BT) * 128;
+  static_assert(smem >= WN * WT * 32 * GEMM_ROWB, "the stages must hold the waves' turning space");
+  auto kernel = gemm_direct_kernel<T, BN, BT, WN, WT, NS, EPI>;
+  static bool raised = false;
+  if (smem > 64 * 1024 && !raised) {
+    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) DLGO_FAIL("gemm: cannot get %d bytes of LDS: %s", smem, hipGetErrorString(e));
+    raised = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(tiles_t * tiles_n)), dim3(WN * WT * WAVE), smem, stream, (const T*)W, (const T*)X, Y,
+                     N, Tn, K, ldw, ldx, ldy, tiles_t);
+  return nullptr;
+}
+
+// What gemm_direct_kernel asks of a product: whole 128-byte pieces along k, and row offsets within a tile that fit 32 bits.
+static bool direct_takes(int K, int ldw, int ldx, size_t elem) {
+  return K % (int)(128 / elem) == 0 && (size_t)256 * ldw * elem < (1ull << 32) && (size_t)256 * ldx * elem < (1ull << 32);
+}
+
 template <typename T, int BN, int BT, int WN, int WT, int EPI>
 static const char* launch_tiled(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy,
                                 hipStream_t stream) {
@@ -184,8 +353,20 @@ template <typename T, int EPI>
 static const char* dispatch(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy, int force,
                             hipStream_t stream) {
   // force: 0 = choose, 2 = 128x128 tiles, 3 = 64x64, 4 = 32x32, 10 = 256x128, 11 = 256x256, 12 = 256x256 with 8 waves,
-  // 13 = 128x64, 14 = 64x128
+  // 13 = 128x64, 14 = 64x128; direct loads into LDS: 20 = 256x256 with 16 waves, 21 = 128x128 with 8 waves and two
+  // blocks on a compute unit, 22 = 128x128 with 8 waves and three stages
   int kind = force;
+  const bool direct = direct_takes(K, ldw, ldx, sizeof(T));
+  if (kind >= 20 && !direct) DLGO_FAIL("gemm: kernel %d needs K %% %d == 0, got K=%d", kind, (int)(128 / sizeof(T)), K);
+  if (kind == 0 && direct && (long)((N + 127) / 128) * ((Tn + 127) / 128) >= 128) {
+    const long b256 = (long)((N + 255) / 256) * ((Tn + 255) / 256);
+    const long big = (long)((N + 127) / 128) * ((Tn + 127) / 128);
+    // the large tile when it fills the chip; else two blocks of 128x128 on a unit when there are that many; else one, deeper
+    kind = b256 >= 256 ? 20 : (big > 256 ? 21 : 22);
+  }
+  if (kind == 20) return launch_direct<T, 256, 256, 4, 4, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  if (kind == 21) return launch_direct<T, 128, 128, 2, 4, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  if (kind == 22) return launch_direct<T, 128, 128, 4, 2, 3, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 0) {
     const long b256 = (long)((N + 255) / 256) * ((Tn + 255) / 256);
     const long big = (long)((N + 127) / 128) * ((Tn + 127) / 128);
@@ -228,7 +409,8 @@ extern "C" const char* dlgo_gemm(const void* W, const void* X, void* Y, int dtyp
   DLGO_REQUIRE(((uintptr_t)Y & 3) == 0 || (dtype == DLGO_DTYPE_BF16 && ((uintptr_t)Y & 1) == 0), "gemm: Y must be aligned to its elements");
   DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm: SwiGLU epilogue needs an even N and ldy >= N/2");
   DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm: ldy %d shorter than N %d", ldy, N);
-  DLGO_REQUIRE(force_kind == 0 || (force_kind >= 2 && force_kind <= 4) || (force_kind >= 10 && force_kind <= 14),
+  DLGO_REQUIRE(force_kind == 0 || (force_kind >= 2 && force_kind <= 4) || (force_kind >= 10 && force_kind <= 14) ||
+                   (force_kind >= 20 && force_kind <= 22),
                "gemm: unknown kernel choice %d", force_kind);
   if (Tn == 0) return nullptr;
   const char* err = by_epilogue<elem_t>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, force_kind, stream);

@@ -100,6 +100,37 @@ def test_gemm_store_and_accumulate(dtype, _, rel, kind, n, t, k):
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("kind", [20, 21, 22])
+@pytest.mark.parametrize("n,t,k", [(300, 130, 64), (517, 259, 128), (128, 128, 192), (1030, 77, 1024), (250, 700, 2048)])
+def test_gemm_direct_to_lds(dtype, _, rel, kind, n, t, k):
+    """The kernels that load tiles straight into LDS: one k tile, fewer tiles than stages, many; edges in n and t;
+    every epilogue.  Row i of the weights is marked so that a row landing in another row's place shows."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(n + 7 * t + k)
+    w = torch.randn(n, k, generator=g)
+    w[:, 0] += torch.arange(n) % 7
+    w = w.to(dtype).to(DEV)
+    x = torch.randn(t, k, generator=g)
+    x[:, 0] += 1
+    x = x.to(dtype).to(DEV)
+    want = x.double() @ w.double().T
+    out = torch.empty(t, n, dtype=dtype, device=DEV)
+    ops.gemm(w, x, out, ops.EPI_STORE, kind)
+    close(out, want, rel, f"gemm store kind={kind}")
+    res = torch.randn(t, n, generator=g).to(DEV)
+    res0 = res.clone()
+    ops.gemm(w, x, res, ops.EPI_ACCUM_F32, kind)
+    close(res, res0.double() + want, 1e-5, f"gemm accumulate kind={kind}")
+    if n % 2 == 0:
+        sw = torch.empty(t, n // 2, dtype=dtype, device=DEV)
+        ops.gemm(w, x, sw, ops.EPI_SWIGLU, kind)
+        gd, ud = want[:, 0::2], want[:, 1::2]
+        close(sw, gd / (1 + torch.exp(-gd)) * ud, rel, f"swiglu kind={kind}")
+    with pytest.raises(ops.KernelError):
+        ops.gemm(w[:, :k - 8].contiguous(), x[:, :k - 8].contiguous(), out, ops.EPI_STORE, kind)
+
+
+@pytest.mark.parametrize("dtype,_,rel", DT)
 @pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("f,t,k", [(160, 5, 64), (352, 70, 128), (9, 2, 16), (1030, 200, 72), (40, 33, 2056), (8200, 64, 256), (16401, 9, 2048)])
 def test_gemm_swiglu(dtype, _, rel, kind, f, t, k):
