@@ -179,8 +179,8 @@ template <int N> static __device__ __forceinline__ void wait_loads() {   // unti
 
 template <typename T, int BN, int BT, int WN, int WT, int NS, int EPI>
 __global__ __launch_bounds__(WN* WT* WAVE) void gemm_direct_kernel(const T* __restrict__ W, const T* __restrict__ X,
-                                                                     void* __restrict__ Y, int N, int Tn, int K, int ldw, int ldx,
-                                                                     int ldy, int tiles_t) {
+                                                                     void* __restrict__ Yv, int N, int Tn, int K, int ldw, int ldx,
+                                                                     int ldy, int tiles_t, int nk_split, long long split_stride) {
   constexpr int NW = WN * WT;
   constexpr int EPC = 16 / sizeof(T);
   constexpr int BK = 128 / sizeof(T);
@@ -227,8 +227,12 @@ __global__ __launch_bounds__(WN* WT* WAVE) void gemm_direct_kernel(const T* __re
     t = t < Tn ? t : Tn - 1;
     offB[q] = (uint32_t)(t - t0) * (uint32_t)ldx * (uint32_t)sizeof(T) + (uint32_t)p * 16u;
   }
-  const char* baseA = (const char*)(W + (size_t)n0 * ldw);
-  const char* baseB = (const char*)(X + (size_t)t0 * ldx);
+  // blockIdx.y: which run of nk_split k tiles this block sums (one run = the whole of k, unless the caller split it)
+  const int kt0 = blockIdx.y * nk_split;
+  const int nk = K / BK - kt0 < nk_split ? K / BK - kt0 : nk_split;
+  void* Y = EPI == EPI_STORE_F32 ? (void*)((float*)Yv + (size_t)blockIdx.y * split_stride) : Yv;
+  const char* baseA = (const char*)(W + (size_t)n0 * ldw) + (size_t)kt0 * 128;
+  const char* baseB = (const char*)(X + (size_t)t0 * ldx) + (size_t)kt0 * 128;
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds;
   const uint32_t ldsA = __builtin_amdgcn_readfirstlane(lds0 + wave * LA * 1024);
   const uint32_t ldsB = __builtin_amdgcn_readfirstlane(lds0 + BN * 128 + wave * LB * 1024);
@@ -242,7 +246,6 @@ __global__ __launch_bounds__(WN* WT* WAVE) void gemm_direct_kernel(const T* __re
     for (int q = 0; q < LB; ++q) load_to_lds(b, offB[q], ldsB + stage * STAGE + q * 1024);
   };
 
-  const int nk = K / BK;
 #pragma unroll
   for (int s = 0; s < NS - 1; ++s)
     if (s < nk) issue(s, s);
@@ -311,8 +314,9 @@ __global__ __launch_bounds__(WN* WT* WAVE) void gemm_direct_kernel(const T* __re
 
 template <typename T, int BN, int BT, int WN, int WT, int NS, int EPI>
 static const char* launch_direct(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy,
-                                 hipStream_t stream) {
+                                 hipStream_t stream, int splits = 1, long long split_stride = 0) {
   const int tiles_t = (Tn + BT - 1) / BT, tiles_n = (N + BN - 1) / BN;
+  const int nk_all = K / (int)(128 / sizeof(T)), nk_split = (nk_all + splits - 1) / splits;
   constexpr int smem = NS * (BN + BT) * 128;
   static_assert(smem >= WN * WT * 32 * GEMM_ROWB, "the stages must hold the waves' turning space");
   auto kernel = gemm_direct_kernel<T, BN, BT, WN, WT, NS, EPI>;
@@ -322,8 +326,50 @@ static const char* launch_direct(const void* W, const void* X, void* Y, int N, i
     if (e != hipSuccess) DLGO_FAIL("gemm: cannot get %d bytes of LDS: %s", smem, hipGetErrorString(e));
     raised = true;
   }
-  hipLaunchKernelGGL(kernel, dim3((unsigned)(tiles_t * tiles_n)), dim3(WN * WT * WAVE), smem, stream, (const T*)W, (const T*)X, Y,
-                     N, Tn, K, ldw, ldx, ldy, tiles_t);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(tiles_t * tiles_n), (unsigned)((nk_all + nk_split - 1) / nk_split)), dim3(WN * WT * WAVE),
+                     smem, stream, (const T*)W, (const T*)X, Y, N, Tn, K, ldw, ldx, ldy, tiles_t, nk_split, split_stride);
+  return nullptr;
+}
+
+// The sums over the runs of k that a split product left in part[run][t][n], added in the order of the runs, go through
+// the epilogue.  A thread takes four consecutive n of one token.
+template <typename T, int EPI>
+__global__ __launch_bounds__(256) void split_sum_kernel(const float* __restrict__ part, int runs, long long run_stride,
+                                                        void* __restrict__ Y, int ldy, int N, int Tn) {
+  const int n4 = (N + 3) / 4;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long long)Tn * n4) return;
+  const int t = (int)(idx / n4), n = (int)(idx % n4) * 4;
+  const float* p = part + (size_t)t * N + n;
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  if ((N & 3) == 0) {
+    for (int r = 0; r < runs; ++r) {
+      const float4 x = *(const float4*)(p + (size_t)r * run_stride);
+      v[0] += x.x;
+      v[1] += x.y;
+      v[2] += x.z;
+      v[3] += x.w;
+    }
+  } else {
+    for (int r = 0; r < runs; ++r)
+      for (int e = 0; e < 4 && n + e < N; ++e) v[e] += p[(size_t)r * run_stride + e];
+  }
+  epilogue4<T, EPI>(Y, ldy, N, t, n, v[0], v[1], v[2], v[3]);
+}
+
+// Few rows of X and few rows of W leave a chip of 256 compute units idle unless k is shared out as well: the runs of
+// k go to blocks of their own (64x64 tiles), and split_sum_kernel adds their sums in a fixed order.
+template <typename T, int EPI, int BN = 64, int BT = 64, int WN = 2, int WT = 2, int NS = 4>
+static const char* launch_split(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy, int splits,
+                                float* part, hipStream_t stream) {
+  const long long plane = (long long)Tn * N;
+  const char* err = launch_direct<T, BN, BT, WN, WT, NS, EPI_STORE_F32>(W, X, part, N, Tn, K, ldw, ldx, N, stream, splits, plane);
+  if (err) return err;
+  const int nk_all = K / (int)(128 / sizeof(T)), nk_split = (nk_all + splits - 1) / splits;
+  const int runs = (nk_all + nk_split - 1) / nk_split;
+  const long long threads = (long long)Tn * ((N + 3) / 4);
+  hipLaunchKernelGGL((split_sum_kernel<T, EPI>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, part, runs, plane, Y,
+                     ldy, N, Tn);
   return nullptr;
 }
 
@@ -351,19 +397,41 @@ static const char* launch_tiled(const void* W, const void* X, void* Y, int N, in
 
 template <typename T, int EPI>
 static const char* dispatch(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy, int force,
-                            hipStream_t stream) {
+                            int splits, float* part, long long part_elems, hipStream_t stream) {
   // force: 0 = choose, 2 = 128x128 tiles, 3 = 64x64, 4 = 32x32, 10 = 256x128, 11 = 256x256, 12 = 256x256 with 8 waves,
   // 13 = 128x64, 14 = 64x128; direct loads into LDS: 20 = 256x256 with 16 waves, 21 = 128x128 with 8 waves and two
-  // blocks on a compute unit, 22 = 128x128 with 8 waves and three stages
+  // blocks on a compute unit, 22 = 128x128 with 8 waves and three stages, 23 = 64x64 with four stages.
+  // splits: 0 = choose, 1 = every block sums the whole of k, more = k in that many runs (64x64 tiles; needs part)
   int kind = force;
   const bool direct = direct_takes(K, ldw, ldx, sizeof(T));
-  if (kind >= 20 && !direct) DLGO_FAIL("gemm: kernel %d needs K %% %d == 0, got K=%d", kind, (int)(128 / sizeof(T)), K);
-  if (kind == 0 && direct && (long)((N + 127) / 128) * ((Tn + 127) / 128) >= 128) {
+  if ((kind >= 20 || splits > 1) && !direct) DLGO_FAIL("gemm: kernel %d needs K %% %d == 0, got K=%d", kind, (int)(128 / sizeof(T)), K);
+  const int nk_all = K / (int)(128 / sizeof(T));
+  if (splits == 0) {
+    splits = 1;
+    const long small = (long)((N + 63) / 64) * ((Tn + 63) / 64);
+    if (kind == 0 && direct && part && Tn <= 128 && small <= 64 && nk_all >= 32) {
+      splits = (int)(256 / small);                          // a block for every compute unit ...
+      if (splits > nk_all / 8) splits = nk_all / 8;         // ... of at least eight k tiles
+      if ((long long)splits * Tn * N > part_elems) splits = 1;
+    }
+  }
+  if (splits > 1) {
+    DLGO_REQUIRE(kind == 0 || kind == 23, "gemm: k is split for the 64x64 tiles only, not kernel %d", kind);
+    DLGO_REQUIRE(part && (long long)splits * Tn * N <= part_elems && ((uintptr_t)part & 15) == 0,
+                 "gemm: %d runs of k need %lld floats of scratch, got %lld", splits, (long long)splits * Tn * N, part_elems);
+    DLGO_REQUIRE(splits <= nk_all, "gemm: %d runs of k, but only %d tiles", splits, nk_all);
+    return launch_split<T, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, splits, part, stream);
+  }
+  if (kind == 0 && direct) {
     const long b256 = (long)((N + 255) / 256) * ((Tn + 255) / 256);
     const long big = (long)((N + 127) / 128) * ((Tn + 127) / 128);
-    // the large tile when it fills the chip; else two blocks of 128x128 on a unit when there are that many; else one, deeper
-    kind = b256 >= 256 ? 20 : (big > 256 ? 21 : 22);
+    // Few rows of X: the weights stream through small tiles.  Else the large tile when it fills the chip; else two blocks
+    // of 128x128 on a unit when there are that many; else one, deeper.  (Measured on the shapes of a 1B Llama.)
+    if (Tn <= 64) kind = 23;
+    else if (Tn <= 128) kind = N >= 32768 ? 21 : 23;
+    else if (big >= 128) kind = b256 >= 256 ? 20 : (big > 256 ? 21 : 22);
   }
+  if (kind == 23) return launch_direct<T, 64, 64, 2, 2, 4, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 20) return launch_direct<T, 256, 256, 4, 4, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 21) return launch_direct<T, 128, 128, 2, 4, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 22) return launch_direct<T, 128, 128, 4, 2, 3, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
@@ -387,19 +455,21 @@ static const char* dispatch(const void* W, const void* X, void* Y, int N, int Tn
 
 template <typename T>
 static const char* by_epilogue(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy, int epi,
-                               int force, hipStream_t stream) {
+                               int force, int splits, float* part, long long part_elems, hipStream_t stream) {
   switch (epi) {
-    case EPI_STORE: return dispatch<T, EPI_STORE>(W, X, Y, N, Tn, K, ldw, ldx, ldy, force, stream);
-    case EPI_ACCUM_F32: return dispatch<T, EPI_ACCUM_F32>(W, X, Y, N, Tn, K, ldw, ldx, ldy, force, stream);
-    case EPI_SWIGLU: return dispatch<T, EPI_SWIGLU>(W, X, Y, N, Tn, K, ldw, ldx, ldy, force, stream);
-    case EPI_STORE_F32: return dispatch<T, EPI_STORE_F32>(W, X, Y, N, Tn, K, ldw, ldx, ldy, force, stream);
+    case EPI_STORE: return dispatch<T, EPI_STORE>(W, X, Y, N, Tn, K, ldw, ldx, ldy, force, splits, part, part_elems, stream);
+    case EPI_ACCUM_F32: return dispatch<T, EPI_ACCUM_F32>(W, X, Y, N, Tn, K, ldw, ldx, ldy, force, splits, part, part_elems, stream);
+    case EPI_SWIGLU: return dispatch<T, EPI_SWIGLU>(W, X, Y, N, Tn, K, ldw, ldx, ldy, force, splits, part, part_elems, stream);
+    case EPI_STORE_F32: return dispatch<T, EPI_STORE_F32>(W, X, Y, N, Tn, K, ldw, ldx, ldy, force, splits, part, part_elems, stream);
     default: DLGO_FAIL("gemm: unknown epilogue %d", epi);
   }
 }
 
 // Y[t, n] (epilogue) = sum_k X[t, k] W[n, k].  ldy counts elements of Y's own type; for the SwiGLU epilogue Y has N/2 columns.
+// part (may be null): part_elems floats of scratch for products whose k is split over several blocks.
 extern "C" const char* dlgo_gemm(const void* W, const void* X, void* Y, int dtype, int N, int Tn, int K, int ldw, int ldx,
-                                 int ldy, int epilogue, int force_kind, hipStream_t stream) {
+                                 int ldy, int epilogue, int force_kind, int splits, float* part, long long part_elems,
+                                 hipStream_t stream) {
   DLGO_REQUIRE(N > 0 && Tn >= 0 && K > 0, "gemm: bad sizes N=%d T=%d K=%d", N, Tn, K);
   DLGO_REQUIRE(dtype == DLGO_ELEM, "gemm: this library is built for dtype code %d, got %d", DLGO_ELEM, dtype);
   const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
@@ -409,11 +479,12 @@ extern "C" const char* dlgo_gemm(const void* W, const void* X, void* Y, int dtyp
   DLGO_REQUIRE(((uintptr_t)Y & 3) == 0 || (dtype == DLGO_DTYPE_BF16 && ((uintptr_t)Y & 1) == 0), "gemm: Y must be aligned to its elements");
   DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm: SwiGLU epilogue needs an even N and ldy >= N/2");
   DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm: ldy %d shorter than N %d", ldy, N);
+  DLGO_REQUIRE(splits >= 0 && part_elems >= 0, "gemm: bad split %d", splits);
   DLGO_REQUIRE(force_kind == 0 || (force_kind >= 2 && force_kind <= 4) || (force_kind >= 10 && force_kind <= 14) ||
-                   (force_kind >= 20 && force_kind <= 22),
+                   (force_kind >= 20 && force_kind <= 23),
                "gemm: unknown kernel choice %d", force_kind);
   if (Tn == 0) return nullptr;
-  const char* err = by_epilogue<elem_t>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, force_kind, stream);
+  const char* err = by_epilogue<elem_t>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, force_kind, splits, part, part_elems, stream);
   if (err) return err;
   DLGO_LAUNCH_CHECK("gemm");
   return nullptr;

@@ -19,6 +19,8 @@ EPI_STORE, EPI_ACCUM_F32, EPI_SWIGLU, EPI_STORE_F32 = 0, 1, 2, 3
 GEMM_AUTO, GEMM_STREAM, GEMM_TILE128, GEMM_TILE64, GEMM_TILE32, GEMM_ROWS16 = 0, 1, 2, 3, 4, 5
 GEMM_TILE256X128, GEMM_TILE256 = 10, 11
 GEMM_FEW_ROWS = 64      # up to this many rows of x the weight-streaming kernels can be chosen
+GEMM_SPLIT_FLOATS = 1 << 20   # scratch that lets gemm() share the inner size of a product out over blocks
+GEMM_VERY_WIDE = 65536   # from this many weight rows on (a vocabulary) the tiled kernel is faster for any number of rows of x
 GEMM_FEW_ROWS_WIDE = 16  # ... and up to this many when the weight has very many rows (there the tiled kernel is faster)
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
@@ -114,8 +116,11 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
 
 
 def gemm(weight: torch.Tensor, x: torch.Tensor, out: torch.Tensor, epilogue: int = EPI_STORE,
-         kind: int = GEMM_AUTO) -> torch.Tensor:
+         kind: int = GEMM_AUTO, scratch: Optional[torch.Tensor] = None, splits: int = 0) -> torch.Tensor:
     """out (epilogue)= x @ weight.T with weight [N, K], x [T, K].
+
+    scratch: float32 of GEMM_SPLIT_FLOATS elements (optional).  With it, a product of few rows with a long inner
+    size may share k out over several blocks (splits: 0 = let the kernel choose, 1 = never, n = n runs of k).
 
     EPI_STORE: out [T, N] in the run dtype.  EPI_ACCUM_F32: out float32 [T, N], added to.
     EPI_SWIGLU: weight rows are (gate_0, up_0, gate_1, up_1, ...), out [T, N/2] = silu(gate) * up.
@@ -132,20 +137,41 @@ def gemm(weight: torch.Tensor, x: torch.Tensor, out: torch.Tensor, epilogue: int
     cols = n // 2 if epilogue == EPI_SWIGLU else n
     if tuple(out.shape) != (t, cols):
         raise KernelError(f"gemm: output {tuple(out.shape)}, expected {(t, cols)}")
-    rows_kernel = kind in (GEMM_STREAM, 5, 6, 7, 8, 9) or (
-        kind == GEMM_AUTO and (t <= GEMM_FEW_ROWS_WIDE or (t <= GEMM_FEW_ROWS and n < 16384)))
+    if scratch is not None:
+        _need(scratch, "gemm scratch", torch.float32, 1)
+    elif splits > 1:
+        raise KernelError("gemm: a split product needs scratch")
+    # k in 128-byte pieces, if it is a whole number of them (what the kernels that load tiles straight into LDS take)
+    piece = 128 // weight.element_size()
+    nk = k // piece if k % piece == 0 else 0
+    can_split = scratch is not None and splits != 1 and nk >= 32 and n <= 4096
+    if kind != GEMM_AUTO or splits > 1:
+        rows_kernel = kind in (GEMM_STREAM, 5, 6, 7, 8, 9)
+    elif t <= GEMM_FEW_ROWS_WIDE:       # measured on the shapes of a 1B Llama: a long inner size is better split,
+        rows_kernel = not (can_split and nk >= 64) and not (n >= GEMM_VERY_WIDE and nk > 0)   # a vocabulary better tiled
+    elif t <= GEMM_FEW_ROWS:
+        rows_kernel = n < 16384 and not (can_split and (nk >= 64 or t >= 24)) and (t <= 40 or nk == 0)
+    else:
+        rows_kernel = False
+    args = (_ptr(weight), _ptr(x), _ptr(out), dtype_code(weight.dtype), n, t, k, _rows(weight, "gemm weight"),
+            _rows(x, "gemm input"), _rows(out, "gemm output"), epilogue)
     if rows_kernel:
         fn = _lib("gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),)).dlgo_gemm_rows
-        kind = 0 if kind in (GEMM_AUTO, GEMM_ROWS16) else kind
+        _check(fn(*args, 0 if kind in (GEMM_AUTO, GEMM_ROWS16) else kind, _stream()))
     else:
         fn = _lib("gemm", (("DLGO_ELEM", dtype_code(weight.dtype)),)).dlgo_gemm
-    _check(fn(_ptr(weight), _ptr(x), _ptr(out), dtype_code(weight.dtype), n, t, k, _rows(weight, "gemm weight"),
-              _rows(x, "gemm input"), _rows(out, "gemm output"), epilogue, kind, _stream()))
+        _check(fn(*args, kind, splits, _ptr(scratch), ctypes.c_longlong(scratch.numel() if scratch is not None else 0), _stream()))
     return out
 
 
 FUSED_NORM_ROWS = 64   # most rows of the residual stream that gemm_rmsnorm takes
 FUSED_NORM_PAYS = 16   # up to this many rows the fused norm is faster than a norm kernel and a plain product
+
+
+def fused_norm_pays(weight: torch.Tensor, rows: int) -> bool:
+    """Whether gemm_rmsnorm beats a norm kernel followed by gemm for this weight and this many rows."""
+    tiled = weight.shape[0] >= GEMM_VERY_WIDE and weight.shape[1] % (128 // weight.element_size()) == 0
+    return rows <= FUSED_NORM_PAYS and not tiled
 
 
 def gemm_rmsnorm(weight: torch.Tensor, x: torch.Tensor, norm_weight: torch.Tensor, eps: float, out: torch.Tensor,

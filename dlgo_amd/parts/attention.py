@@ -95,17 +95,18 @@ class Attention(Mixer):
         self.w_o = stored(tensors["o_proj.weight"], spec["o_proj.weight"], device, dtype)
 
     def fuses_norm(self, norm, ctx) -> bool:
-        return isinstance(norm, RMSNorm) and ctx.n_tokens <= ops.FUSED_NORM_PAYS
+        return isinstance(norm, RMSNorm) and ops.fused_norm_pays(self.w_qkv, ctx.n_tokens)
 
     def forward(self, xn, ctx, unit, residual, owns_cache=True, norm=None) -> None:
         t = xn.shape[0]
         n_kv = self.n_kv_heads if owns_cache else 0
         cols = self.q_dim + 2 * n_kv * self.head_dim
         qkv = ctx.buffer("attention.qkv", (t, self.q_dim + 2 * self.kv_dim), ctx.dtype)
+        split = ctx.scratch("gemm.split", ops.GEMM_SPLIT_FLOATS, torch.float32)
         if norm is not None:      # xn are the float32 residual rows: the norm rides in the product
             ops.gemm_rmsnorm(self.w_qkv[:cols], xn, norm.weight, norm.eps, qkv[:, :cols])
         else:
-            ops.gemm(self.w_qkv[:cols], xn, qkv[:, :cols])
+            ops.gemm(self.w_qkv[:cols], xn, qkv[:, :cols], scratch=split)
         kv = ctx.cache.kv_view(unit)
         rot = self.position.rotation()
         # a step of single tokens: the attention kernel rotates and stores by itself; else a kernel of its own does
@@ -118,7 +119,7 @@ class Attention(Mixer):
         out = ctx.buffer("attention.out", (t, self.q_dim), ctx.dtype)
         self.attend(qkv, out, ctx, kv, rotation=(rot.cos, rot.sin, rot.width, rot.interleaved) if fused and rot else None,
                     new_kv=fused and owns_cache)
-        ops.gemm(self.w_o, out, residual, ops.EPI_ACCUM_F32)
+        ops.gemm(self.w_o, out, residual, ops.EPI_ACCUM_F32, scratch=split)
 
     def attend(self, q, out, ctx, kv, rotation=None, new_kv=False) -> None:
         """Attention of the step's (rotated) query rows over the cache; the kernel is chosen by the

@@ -53,7 +53,7 @@ class OutputHead(Part):
         return self.tied_to.weight if self.tied_to is not None else self._weight
 
     def fuses_norm(self, norm, ctx) -> bool:
-        return isinstance(norm, RMSNorm) and ctx.n_tokens <= ops.FUSED_NORM_PAYS
+        return isinstance(norm, RMSNorm) and ops.fused_norm_pays(self.weight, ctx.n_tokens)
 
     def __call__(self, xn: torch.Tensor, out: torch.Tensor, norm=None) -> torch.Tensor:
         """xn: normed rows (run dtype), or with `norm` the float32 residual rows; out: float32 [rows, vocab]."""

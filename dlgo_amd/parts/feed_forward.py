@@ -53,7 +53,7 @@ class GatedFeedForward(FeedForward):
         self.w_down = stored(tensors["down_proj.weight"], spec["down_proj.weight"], device, dtype)
 
     def fuses_norm(self, norm, ctx) -> bool:
-        return isinstance(norm, RMSNorm) and ctx.n_tokens <= ops.FUSED_NORM_PAYS
+        return isinstance(norm, RMSNorm) and ops.fused_norm_pays(self.w_gate_up, ctx.n_tokens)
 
     def forward(self, xn, ctx, residual, norm=None) -> None:
         hid = ctx.buffer("feed_forward.hidden", (xn.shape[0], self.inner), ctx.dtype)
@@ -61,4 +61,4 @@ class GatedFeedForward(FeedForward):
             ops.gemm_rmsnorm(self.w_gate_up, xn, norm.weight, norm.eps, hid, ops.EPI_SWIGLU)
         else:
             ops.gemm(self.w_gate_up, xn, hid, ops.EPI_SWIGLU)
-        ops.gemm(self.w_down, hid, residual, ops.EPI_ACCUM_F32)
+        ops.gemm(self.w_down, hid, residual, ops.EPI_ACCUM_F32, scratch=ctx.scratch("gemm.split", ops.GEMM_SPLIT_FLOATS, torch.float32))

@@ -100,7 +100,7 @@ def test_gemm_store_and_accumulate(dtype, _, rel, kind, n, t, k):
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
-@pytest.mark.parametrize("kind", [20, 21, 22])
+@pytest.mark.parametrize("kind", [20, 21, 22, 23])
 @pytest.mark.parametrize("n,t,k", [(300, 130, 64), (517, 259, 128), (128, 128, 192), (1030, 77, 1024), (250, 700, 2048)])
 def test_gemm_direct_to_lds(dtype, _, rel, kind, n, t, k):
     """The kernels that load tiles straight into LDS: one k tile, fewer tiles than stages, many; edges in n and t;
@@ -128,6 +128,47 @@ def test_gemm_direct_to_lds(dtype, _, rel, kind, n, t, k):
         close(sw, gd / (1 + torch.exp(-gd)) * ud, rel, f"swiglu kind={kind}")
     with pytest.raises(ops.KernelError):
         ops.gemm(w[:, :k - 8].contiguous(), x[:, :k - 8].contiguous(), out, ops.EPI_STORE, kind)
+
+
+@pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("n,t,k,splits", [(130, 20, 512, 2), (64, 64, 2048, 5), (257, 33, 1024, 8), (2048, 64, 8192, 0), (300, 17, 4096, 0),
+                                          (96, 40, 640, 3)])
+def test_gemm_with_split_inner_size(dtype, _, rel, n, t, k, splits):
+    """The inner size shared out over blocks whose sums are added in a fixed order: every epilogue, runs that do not
+    divide the tiles evenly, and twice the same bits."""
+    ops = _ops()
+    if dtype == torch.float32:
+        k //= 2         # the same number of 128-byte pieces
+    g = torch.Generator().manual_seed(n + 7 * t + k)
+    w = torch.randn(n, k, generator=g)
+    w[:, 0] += torch.arange(n) % 7
+    w = w.to(dtype).to(DEV)
+    x = torch.randn(t, k, generator=g).to(dtype).to(DEV)
+    want = x.double() @ w.double().T
+    scratch = torch.full((ops.GEMM_SPLIT_FLOATS,), float("nan"), device=DEV)
+    out = torch.empty(t, n, dtype=dtype, device=DEV)
+    ops.gemm(w, x, out, ops.EPI_STORE, scratch=scratch, splits=splits)
+    close(out, want, rel, "split store")
+    again = torch.empty_like(out)
+    ops.gemm(w, x, again, ops.EPI_STORE, scratch=scratch, splits=splits)
+    assert torch.equal(out, again)
+    res = torch.randn(t, n, generator=g).to(DEV)
+    res0 = res.clone()
+    ops.gemm(w, x, res, ops.EPI_ACCUM_F32, scratch=scratch, splits=splits)
+    close(res, res0.double() + want, 1e-5, "split accumulate")
+    out32 = torch.empty(t, n, dtype=torch.float32, device=DEV)
+    ops.gemm(w, x, out32, ops.EPI_STORE_F32, scratch=scratch, splits=splits)
+    close(out32, want, 1e-5, "split store f32")
+    if n % 2 == 0:
+        sw = torch.empty(t, n // 2, dtype=dtype, device=DEV)
+        ops.gemm(w, x, sw, ops.EPI_SWIGLU, scratch=scratch, splits=splits)
+        gd, ud = want[:, 0::2], want[:, 1::2]
+        close(sw, gd / (1 + torch.exp(-gd)) * ud, rel, "split swiglu")
+    if splits > 1:
+        with pytest.raises(ops.KernelError):
+            ops.gemm(w, x, out, ops.EPI_STORE, scratch=scratch[:splits * t * n - 1], splits=splits)
+        with pytest.raises(ops.KernelError):
+            ops.gemm(w, x, out, ops.EPI_STORE, splits=splits)
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
