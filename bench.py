@@ -28,6 +28,13 @@ LLAMA_1B = {
     "max_position_embeddings": 131072, "tie_word_embeddings": True, "initializer_range": 0.02,
     "hidden_act": "silu", "torch_dtype": "bfloat16", "bos_token_id": 128000, "eos_token_id": 128001,
 }
+# Other shapes of the family, for measurements beside the default: the same keys with other sizes.
+SHAPES = {
+    "llama-3.2-1b": LLAMA_1B,
+    "llama-3.2-3b": dict(LLAMA_1B, hidden_size=3072, num_hidden_layers=28, num_attention_heads=24, head_dim=128),
+    "llama-3.1-8b": dict(LLAMA_1B, hidden_size=4096, num_hidden_layers=32, intermediate_size=14336, head_dim=128,
+                         tie_word_embeddings=False, rope_scaling=dict(LLAMA_1B["rope_scaling"], factor=8.0)),
+}
 CONTEXT = 4096
 PROMPT = 2048
 HBM_PEAK = 8.0e12
@@ -38,7 +45,7 @@ def weight_bytes(cfg, elem):
     """Bytes a decode step must read of the weights: every matrix once (the tied table serves as the head)."""
     d, f = cfg.hidden_size, cfg.intermediate_size
     per_layer = (cfg.q_dim + 2 * cfg.kv_dim) * d + d * cfg.q_dim + 3 * d * f
-    head = cfg.vocab_size * d
+    head = cfg.vocab_size * d       # the output head; the embedding table gives only the step's rows
     norms = (2 * cfg.num_hidden_layers + 1) * d * 4
     return (cfg.num_hidden_layers * per_layer + head) * elem + norms
 
@@ -67,6 +74,7 @@ def main() -> int:
     ap.add_argument("--points", default="1,64", help="other batch sizes to report, comma separated ('' = none)")
     ap.add_argument("--point-steps", type=int, default=64)
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--shape", default="llama-3.2-1b", choices=sorted(SHAPES), help="layer sizes (default: the benchmark's)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -80,7 +88,7 @@ def main() -> int:
     from dlgo_amd.engine import Engine, Entry
     from dlgo_amd.sampling import Sampler, SamplerConfig
 
-    raw = dict(LLAMA_1B)
+    raw = dict(SHAPES[args.shape])
     full_layers = raw["num_hidden_layers"]
     if args.layers:
         raw["num_hidden_layers"] = args.layers
@@ -148,11 +156,11 @@ def main() -> int:
                    "frac": round(prefill_flops(cfg, PROMPT) / pt / FLOP_PEAK[args.dtype], 4)}
 
     line = {
-        "metric": f"decode tok/s @ batch {args.batch} (Llama 3.2 1B shape, {PROMPT}-token prompts, context {CONTEXT})",
+        "metric": f"decode tok/s @ batch {args.batch} ({args.shape} shape, {PROMPT}-token prompts, context {CONTEXT})",
         "value": round(value, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
-        "config": {"model": "llama-3.2-1b-shape", "layers": cfg.num_hidden_layers, "layers_of_model": full_layers,
+        "config": {"model": args.shape + "-shape", "layers": cfg.num_hidden_layers, "layers_of_model": full_layers,
                    "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                    "tied_embeddings": cfg.tie_word_embeddings, "global_batch": args.batch, "seq_len": CONTEXT,

@@ -1,6 +1,10 @@
-"""The layer sizes of Llama 3.2 1B (hidden 2048, 32 heads over 8 kv heads of 64, feed-forward 8192, vocabulary 128256,
-llama3 scaling with factor 32) with two layers: whole, last tokens one by one, and a batch of unequal lengths, against
-the plain implementation, in float32 and bfloat16."""
+"""Real layer sizes with one or two layers: whole, last tokens one by one, and a batch of unequal lengths, against the
+plain implementation, in float32 and bfloat16.
+
+  1b: Llama 3.2 1B (hidden 2048, 32 heads over 8 kv heads of 64, feed-forward 8192, vocabulary 128256, scaling factor 32)
+  3b: Llama 3.2 3B layers (hidden 3072, 24 heads over 8 kv heads of 128: three query heads a group, feed-forward 8192)
+  8b: Llama 3.1 8B layers (hidden 4096, 32 heads over 8 kv heads of 128, feed-forward 14336, untied head, factor 8)
+The two larger ones have one layer and a vocabulary of 32003 to keep the plain implementation quick."""
 import numpy as np
 import pytest
 
@@ -19,14 +23,20 @@ WIDE = {
     "max_position_embeddings": 131072, "tie_word_embeddings": True, "initializer_range": 0.02,
     "hidden_act": "silu", "torch_dtype": "bfloat16",
 }
+WIDE_3B = dict(WIDE, vocab_size=32003, hidden_size=3072, num_hidden_layers=1, num_attention_heads=24, head_dim=128)
+WIDE_8B = dict(WIDE, vocab_size=32003, hidden_size=4096, num_hidden_layers=1, intermediate_size=14336, head_dim=128,
+               tie_word_embeddings=False,
+               rope_scaling=dict(WIDE["rope_scaling"], factor=8.0))
+SHAPES = {"1b": WIDE, "3b": WIDE_3B, "8b": WIDE_8B}
 
 
-@pytest.fixture(scope="module")
-def wide(tmp_path_factory):
-    folder = make_folder(WIDE, 31, tmp_path_factory.mktemp("wide"), dtype="bfloat16")
+@pytest.fixture(scope="module", params=list(SHAPES))
+def wide(request, tmp_path_factory):
+    raw = SHAPES[request.param]
+    folder = make_folder(raw, 31, tmp_path_factory.mktemp("wide_" + request.param), dtype="bfloat16")
     cfg, w = plain.read_model(folder)
     rng = np.random.default_rng(2)
-    seqs = [rng.integers(0, WIDE["vocab_size"], size=n).tolist() for n in (70, 9)]
+    seqs = [rng.integers(0, raw["vocab_size"], size=n).tolist() for n in (70, 9)]
     # positions far into the context, where the scaled low frequencies matter
     want = [plain.forward(cfg, w, s) for s in seqs]
     return folder, seqs, want
