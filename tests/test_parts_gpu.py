@@ -1,6 +1,7 @@
 """Each part alone against the plain implementation, and the generality of the assembly: a toy
-mixer with state of its own, a toy position encoding, a windowed attention layer and a run order
-that names a layer twice and lets a run read another run's cache, all registered from here,
+mixer with state of its own, a toy feed-forward that routes each row to one of several experts, a toy
+position encoding, a windowed attention layer and a run order that names a layer twice and lets a
+run read another run's cache, all registered from here,
 built by the registry and stepped by the engine without a change to the library's files."""
 import math
 from dataclasses import dataclass
@@ -165,8 +166,8 @@ def test_attention_part_alone(dtype, window):
 # ---------------------------------------------------------------------------
 def _register_toy():
     from dlgo_amd.config import KeyReader, ModelConfig, register_architecture
-    from dlgo_amd.parts import (CacheNeed, DecoderModel, Embedding, LayerRun, Mixer, OutputHead, PositionEncoding,
-                                TensorSpec, make_part, register_part, stored)
+    from dlgo_amd.parts import (CacheNeed, DecoderModel, Embedding, FeedForward, LayerRun, Mixer, OutputHead,
+                                PositionEncoding, TensorSpec, make_part, register_part, stored)
 
     class DecayMixer(Mixer):
         """A mixer with state of its own: s_t = decay * s_{t-1} + x_t per sequence, out_t = W s_t.
@@ -197,6 +198,42 @@ def _register_toy():
                 state[int(slot)] = s
                 o += int(n)
 
+    class RoutedFeedForward(FeedForward):
+        """A feed-forward with routing: a float32 router scores the experts, each row goes to its best one.  The
+        experts are the library's gated feed-forwards, mounted under experts.<e>; every expert runs on every row and
+        the rows it was not chosen for are masked, which is slow and has no step that depends on the data."""
+
+        def __init__(self, width, inner, n_experts):
+            self.width, self.n_experts = width, n_experts
+            self.experts = [make_part("feed_forward", "gated", width, inner, "silu") for _ in range(n_experts)]
+
+        def tensor_specs(self):
+            specs = {"router.weight": TensorSpec((self.n_experts, self.width), kind="vector")}
+            for e, expert in enumerate(self.experts):
+                specs.update({f"experts.{e}.{n}": sp for n, sp in expert.tensor_specs().items()})
+            return specs
+
+        def kernel_variants(self, dtype):
+            return [v for expert in self.experts for v in expert.kernel_variants(dtype)]
+
+        def check(self, dtype):
+            for expert in self.experts:
+                expert.check(dtype)
+
+        def load(self, tensors, device, dtype):
+            self.router = stored(tensors["router.weight"], self.tensor_specs()["router.weight"], device, dtype)
+            for e, expert in enumerate(self.experts):
+                pre = f"experts.{e}."
+                expert.load({n[len(pre):]: t for n, t in tensors.items() if n.startswith(pre)}, device, dtype)
+
+        def forward(self, xn, ctx, residual, norm=None):
+            choice = (xn.float() @ self.router.T).argmax(-1)          # router logits in float32
+            for e, expert in enumerate(self.experts):
+                mine = ctx.buffer("toy.expert_out", tuple(residual.shape), torch.float32)
+                mine.zero_()
+                expert.forward(xn, ctx, mine)
+                residual += mine * (choice == e).unsqueeze(1)
+
     class LearnedPosition(PositionEncoding):
         """Another position encoding: a learned vector per position, added to the embedded rows."""
 
@@ -220,6 +257,7 @@ def _register_toy():
         kv_heads: int
         head_dim: int
         inner: int
+        experts: int
         eps: float
         decay: float
         window: int
@@ -232,7 +270,7 @@ def _register_toy():
             r = KeyReader(raw)
             vals = dict(architecture=raw["architectures"][0], vocab_size=r.integer("vocab_size"), width=r.integer("width"),
                         heads=r.integer("heads"), kv_heads=r.integer("kv_heads"), head_dim=r.integer("head_dim"),
-                        inner=r.integer("inner"), eps=r.number("eps"), decay=r.number("decay"), window=r.integer("window"),
+                        inner=r.integer("inner"), experts=r.integer("experts"), eps=r.number("eps"), decay=r.number("decay"), window=r.integer("window"),
                         max_position_embeddings=r.integer("max_position_embeddings"),
                         initializer_range=r.number("initializer_range"))
             r.finish()
@@ -252,8 +290,10 @@ def _register_toy():
             return make_part("mixer", "attention", d, cfg.heads, cfg.kv_heads, cfg.head_dim, make_part("position", "none"),
                              window=window)
         mixers = [attention(None), make_part("mixer", "toy_decay", d, cfg.decay), attention(cfg.window)]
-        layers = [(f"blocks.{i}", make_part("block", "pre_norm", ("n1", norm()), ("mixer", m), ("n2", norm()), ("ff", ffn())))
-                  for i, m in enumerate(mixers)]
+        # the layer with the state mixer routes its feed-forward; the attention layers have the dense one
+        ffns = [ffn(), make_part("feed_forward", "toy_routed", d, cfg.inner, cfg.experts), ffn()]
+        layers = [(f"blocks.{i}", make_part("block", "pre_norm", ("n1", norm()), ("mixer", m), ("n2", norm()), ("ff", f)))
+                  for i, (m, f) in enumerate(zip(mixers, ffns))]
         emb = Embedding(cfg.vocab_size, d)
         # layer 1 (state) runs twice, each run with state of its own; the last run is layer 0 again, reading the
         # keys and values that the first run stored
@@ -263,12 +303,16 @@ def _register_toy():
                             position=("positions", make_part("position", "toy_learned", cfg.max_position_embeddings, d)))
 
     register_part("mixer", "toy_decay", DecayMixer)
+    register_part("feed_forward", "toy_routed", RoutedFeedForward)
     register_part("position", "toy_learned", LearnedPosition)
     register_architecture("ToyForCausalLM", ToyConfig, build)
 
 
 TOY = {"architectures": ["ToyForCausalLM"], "vocab_size": 90, "width": 48, "heads": 3, "kv_heads": 1, "head_dim": 16, "inner": 72,
-       "eps": 1e-4, "decay": 0.8, "window": 20, "max_position_embeddings": 256, "initializer_range": 0.15}
+       "experts": 3, "eps": 1e-4, "decay": 0.8, "window": 20, "max_position_embeddings": 256, "initializer_range": 0.15}
+
+
+_EXPERTS_SEEN = set()        # the experts that the plain router chose, over all sequences of the test
 
 
 def _toy_plain(w, tokens):
@@ -288,7 +332,15 @@ def _toy_plain(w, tokens):
 
     def ffn(h, p):
         hn = plain.rmsnorm(h, w[p + "n2.weight"], c["eps"])
-        return h + plain.feed_forward(hn, w[p + "ff.gate_proj.weight"], w[p + "ff.up_proj.weight"], w[p + "ff.down_proj.weight"])
+        if p + "ff.router.weight" not in w:
+            return h + plain.feed_forward(hn, w[p + "ff.gate_proj.weight"], w[p + "ff.up_proj.weight"], w[p + "ff.down_proj.weight"])
+        choice = (hn @ w[p + "ff.router.weight"].T).argmax(-1)
+        _EXPERTS_SEEN.update(choice.tolist())
+        out = h.copy()
+        for t, e in enumerate(choice):
+            q = f"{p}ff.experts.{e}."
+            out[t] += plain.feed_forward(hn[t:t + 1], w[q + "gate_proj.weight"], w[q + "up_proj.weight"], w[q + "down_proj.weight"])[0]
+        return out
 
     def decay(x):
         p = "blocks.1."
@@ -320,6 +372,7 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path):
     rng = np.random.default_rng(0)
     seqs = [rng.integers(0, 90, size=n).tolist() for n in (90, 30, 1)]
     want = [_toy_plain(w, s) for s in seqs]
+    assert _EXPERTS_SEEN == set(range(TOY["experts"]))             # the routing is exercised: every expert gets rows
     # whole, in one batch of unequal lengths
     slots = eng.open(3)
     out = eng.step([Entry(s, t, list(range(len(t)))) for s, t in zip(slots, seqs)]).cpu().numpy()
