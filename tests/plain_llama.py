@@ -156,12 +156,9 @@ def attention(q, k, v, n_heads, n_kv_heads, head_dim, window=None):
         ks = slice(kvh * head_dim, (kvh + 1) * head_dim)
         for p in range(T):
             lo = 0 if window is None else max(0, p - window + 1)
-            scores = np.array([np.dot(q[p, qs], k[t, ks]) * scale for t in range(lo, p + 1)])
+            scores = (k[lo:p + 1, ks] @ q[p, qs]) * scale        # one dot product per visible key
             pr = softmax(scores)
-            acc = np.zeros(head_dim)
-            for j, t in enumerate(range(lo, p + 1)):
-                acc += pr[j] * v[t, ks]
-            out[p, qs] = acc
+            out[p, qs] = pr @ v[lo:p + 1, ks]                    # the values, weighted
     return out
 
 

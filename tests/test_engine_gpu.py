@@ -161,6 +161,40 @@ def test_step_cut_into_pieces_and_batch_mates(folders, oracle, dtype):
         o += len(t)
 
 
+LONG = dict(TINY_B, max_position_embeddings=8192, num_hidden_layers=2, num_key_value_heads=2,
+            rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                          "original_max_position_embeddings": 1024})
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_thousands_of_tokens(tmp_path, dtype):
+    """Prompts of thousands of tokens, cut into pieces of 1024 rows, then 40 tokens one by one from recorded steps:
+    dozens of pages a sequence, positions beyond the scaling's original length, pages dealt to several blocks.  The
+    first sequence repeats one rare token far back and near the end, so that the late queries lean on a far key."""
+    from dlgo_amd.engine import Entry
+    folder = make_folder(LONG, seed=5, path=tmp_path, dtype=dtype, norm_jitter=0.1, std=0.08)
+    cfg, w = plain.read_model(str(folder))
+    rng = np.random.default_rng(4)
+    lens, n_dec = [2500, 700, 65], 40
+    seqs = [rng.integers(1, LONG["vocab_size"], size=n + n_dec).tolist() for n in lens]
+    for at in (3, 2490, 2520):
+        seqs[0][at] = 0
+    want = [plain.forward(cfg, w, t) for t in seqs]
+    eng = engine_for(str(folder), dtype, max_tokens=4096, max_ctx=4096, max_step_tokens=1024)
+    slots = eng.open(3)
+    got = [[eng.step([Entry(s, t[:n], [n - 2, n - 1]) for s, t, n in zip(slots, seqs, lens)]).cpu().numpy()]]
+    for i in range(n_dec):
+        got.append([eng.step([Entry(s, [t[n + i]], [0]) for s, t, n in zip(slots, seqs, lens)]).cpu().numpy()])
+    tol = 5e-5 if dtype == "float32" else TOL[dtype]
+    first = got[0][0]
+    for j, (t, n) in enumerate(zip(seqs, lens)):
+        assert rel_err(first[2 * j:2 * j + 2], want[j][n - 2:n]) <= tol, (dtype, "prompt", j)
+        dec = np.stack([g[0][j] for g in got[1:]])
+        assert rel_err(dec, want[j][n:n + n_dec]) <= tol, (dtype, "decode", j)
+    eng.close(slots)
+    eng.cache.check_consistent()
+
+
 def test_errors_before_anything_runs(folders):
     from dlgo_amd.engine import EngineError, Entry
     eng = engine_for(folders["A", "float32"], "float32", max_tokens=128)
