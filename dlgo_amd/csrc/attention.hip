@@ -177,7 +177,12 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
 
   const int seq = blockIdx.y, kvh = blockIdx.z;
   const int q0 = cu_q[seq], qn = cu_q[seq + 1] - q0;
-  const int t0 = blockIdx.x * bq;
+  // Late tiles see more keys than early ones.  Blocks are handed to the compute units in the order of their linear
+  // index, 256 at a time: odd rounds walk the tiles forwards and even rounds backwards, so that the blocks that share
+  // a unit add up to about the same number of pages.
+  const int linear = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const int tile = (linear >> 8) & 1 ? blockIdx.x : gridDim.x - 1 - blockIdx.x;
+  const int t0 = tile * bq;
   if (t0 >= qn) return;
   const int t1 = t0 + bq < qn ? t0 + bq : qn;           // tokens [t0, t1) of the sequence's rows
   const int start = start_pos[seq];

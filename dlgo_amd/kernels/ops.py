@@ -37,7 +37,13 @@ def dtype_code(dtype: torch.dtype) -> int:
         raise KernelError(f"kernels run in float32 or bfloat16, not {dtype}") from None
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)    # the handle without a Stream object around it
+
+
 def _stream() -> ctypes.c_void_p:
+    """torch's current stream on the current device, as the launches take it."""
+    if _raw_stream is not None:
+        return ctypes.c_void_p(_raw_stream(torch.cuda.current_device()))
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
@@ -66,18 +72,19 @@ def _check(err: Optional[bytes]) -> None:
         raise KernelError(err.decode())
 
 
-_protos_done: set = set()
+_libs: dict = {}      # (module, defines) -> loaded library with its return types set; looked up at every launch
 
 
 def _lib(module: str, defines=()):
-    lib = build.load(module, defines)
     key = (module, tuple(defines))
-    if key not in _protos_done:
+    lib = _libs.get(key)
+    if lib is None:
+        lib = build.load(module, defines)
         for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_attention_rows",
                      "dlgo_attention_prefill", "dlgo_attention_decode", "dlgo_argmax", "dlgo_sample"):
             if hasattr(lib, name):
                 getattr(lib, name).restype = ctypes.c_char_p
-        _protos_done.add(key)
+        _libs[key] = lib
     return lib
 
 
