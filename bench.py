@@ -63,6 +63,53 @@ def prefill_flops(cfg, t):
     return linear + attn + head
 
 
+def ragged(args, cfg, full_layers, elem) -> int:
+    """Unequal prompts through the generation loop (the larger shapes' workloads): one batch, greedy, no stop tokens."""
+    import numpy as np
+    import torch
+
+    from dlgo_amd.engine import Engine
+    from dlgo_amd.engine.generate import generate
+    from dlgo_amd.sampling import Sampler, SamplerConfig
+    from dlgo_amd.sampling.options import GenerateConfig
+    n, lo, hi, new, ctx = (int(v) for v in args.ragged.split(":"))
+    rng = np.random.default_rng(0)
+    lens = rng.integers(lo, hi + 1, size=n)
+    prompts = [rng.integers(0, cfg.vocab_size, size=int(k)).tolist() for k in lens]
+    held = sum((int(k) + new + 63) // 64 * 64 for k in lens)
+    eng = Engine.from_random(cfg, seed=0, dtype=args.dtype, max_tokens=held, max_ctx=ctx, max_slots=n, graph_max_batch=n)
+    sampler = Sampler(eng.vocab, eng.device, max_rows=n)
+    conf = GenerateConfig(max_tokens=new, sampler=SamplerConfig(temperature=0.0), seed=1, ignore_eos=True)
+    runs = []
+    for _ in range(3):
+        _, st = generate(eng, sampler, prompts, [conf] * n, max_batch=n, sync=torch.cuda.synchronize)
+        runs.append(st)
+    st = sorted(runs, key=lambda r: r.generate_ms)[1]
+    steps = st.steps
+    mean_ctx = float(lens.mean()) + (new + 1) / 2.0
+    step_bytes = weight_bytes(cfg, elem) + n * mean_ctx * kv_bytes_per_token(cfg, elem)
+    achieved = step_bytes / (st.generate_ms / 1e3 / steps)
+    flops = sum(prefill_flops(cfg, int(k)) for k in lens)
+    line = {
+        "metric": f"decode tok/s, {n} requests with prompts of {lo}..{hi} tokens ({args.shape} shape, context {ctx})",
+        "value": round(st.tokens_per_sec, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": 1,
+        "ms_per_step": round(st.generate_ms / steps, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids and prompt lengths",
+        "config": {"model": args.shape + "-shape", "layers": cfg.num_hidden_layers, "layers_of_model": full_layers,
+                   "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+                   "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+                   "tied_embeddings": cfg.tie_word_embeddings, "global_batch": n, "seq_len": ctx,
+                   "prompt_tokens": int(lens.sum()), "new_tokens": new, "parallelism": "single-gpu",
+                   "kv_cache_dtype": args.dtype, "sampling": "greedy, through the generation loop"},
+        "prefill": {"value": round(st.prompt_tokens / st.prefill_ms * 1e3, 1), "tokens": int(st.prompt_tokens),
+                    "ms": round(st.prefill_ms, 3), "frac": round(flops / (st.prefill_ms / 1e3) / FLOP_PEAK[args.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK, 4)},
+    }
+    print(json.dumps(line))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -74,6 +121,9 @@ def main() -> int:
     ap.add_argument("--points", default="1,64", help="other batch sizes to report, comma separated ('' = none)")
     ap.add_argument("--point-steps", type=int, default=64)
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--ragged", default="", metavar="N:LO:HI:NEW:CTX",
+                    help="instead of the default run: N requests with prompts of LO..HI tokens (uniform, seeded), NEW "
+                         "generated tokens each, context CTX, through the generation loop")
     ap.add_argument("--shape", default="llama-3.2-1b", choices=sorted(SHAPES), help="layer sizes (default: the benchmark's)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -94,6 +144,8 @@ def main() -> int:
         raw["num_hidden_layers"] = args.layers
     cfg = config_from_dict(raw)
     elem = 2 if args.dtype == "bf16" else 4
+    if args.ragged:
+        return ragged(args, cfg, full_layers, elem)
     batches = [args.batch] + [int(b) for b in args.points.split(",") if b.strip()]
     most = max(batches)
     per_seq = PROMPT + args.warmup + max(args.steps, args.point_steps) + 64
