@@ -264,9 +264,10 @@ def attention_rows(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, 
 def attention_fuses_rotation(dtype: torch.dtype, head_dim: int, group: int, max_q_len: int, rot_width: int,
                              n_seq: int = 1) -> bool:
     """True if attention() should rotate the queries and take in the new keys and values itself for such a step:
-    one row per sequence, bfloat16, a rotated width that is a multiple of 16 or no rotation at all, and few enough
-    sequences that a kernel launch costs more than the rotation repeated in every wave."""
-    return (dtype == torch.bfloat16 and head_dim <= 256 and group <= 128 and max_q_len == 1 and rot_width % 16 == 0
+    one row per sequence, bfloat16, a rotated width that is a multiple of 16 or no rotation at all, few enough
+    sequences that a kernel launch costs more than the rotation repeated in every wave, and heads small enough that
+    the kernel keeps eight waves to a block (measured: at a head size of 128 the kernel of its own is faster)."""
+    return (dtype == torch.bfloat16 and head_dim <= 64 and group <= 128 and max_q_len == 1 and rot_width % 16 == 0
             and n_seq <= 32)
 
 
