@@ -279,40 +279,47 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
           s[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(*(const uint4*)(pk + ks * 32)), as_bf16x8(qf[ks]), s[kt], 0, 0, 0);
       }
       // lane: row = lane%32; element v of tile kt is key  key0 + 32 kt + 8 (v/4) + 4 half + v%4
+      // m is the running maximum of the raw scores; the scale (times log2 e) enters with the exponent, one fused
+      // multiply-add a score
       const bool need_mask = key0 + PAGE - 1 > w_pos_min || key0 < w_lo_max;
       float mx = -INFINITY;
+      if (need_mask) {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int key = key0 + kt * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
+            s[kt][v] = (key <= pos && key >= lo) ? s[kt][v] : -INFINITY;
+          }
+      }
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          float sv = s[kt][v] * scale_log2e;
-          if (need_mask) {
-            const int key = key0 + kt * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
-            sv = (key <= pos && key >= lo) ? sv : -INFINITY;
-          }
-          s[kt][v] = sv;
-          mx = fmaxf(mx, sv);
-        }
+        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s[kt][v]);
       mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
       const float m_new = fmaxf(m, mx);
       const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = fast_exp2(m - m_use);
+      const float off = -m_use * scale_log2e;
       float rs = 0.f;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const float p = fast_exp2(s[kt][v] - m_use);
+          const float p = fast_exp2(fmaf(s[kt][v], scale_log2e, off));
           s[kt][v] = p;
           rs += p;
         }
       rs += __shfl_xor(rs, 32, WAVE);
-      l = l * alpha + rs;
+      if (__any(m_new != m)) {               // the sums so far are rescaled only when some row's maximum moved
+        const float alpha = fast_exp2(fmaf(m, scale_log2e, off));
+        l *= alpha;
+#pragma unroll
+        for (int d = 0; d < DT; ++d)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) o[d][v] *= alpha;
+      }
+      l += rs;
       m = m_new;
-#pragma unroll
-      for (int d = 0; d < DT; ++d)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) o[d][v] *= alpha;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -698,6 +705,7 @@ extern "C" const char* dlgo_attention_prefill(const void* q, int ldq, void* out,
   DLGO_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)out & 7) == 0 && ((uintptr_t)cache & 15) == 0 && page_stride % 8 == 0 && v_off % 8 == 0,
                "attention: operands must be 16-byte aligned");
   DLGO_REQUIRE(window >= 0 && max_pages > 0, "attention: bad window or page table width");
+  DLGO_REQUIRE(scale > 0.f, "attention: the tiled kernel takes a positive scale, got %g", (double)scale);
   if (n_seq == 0 || max_q_len == 0) return nullptr;
   const int bq = PF_ROWS / group;
   dim3 grid((max_q_len + bq - 1) / bq, n_seq, n_kv);
