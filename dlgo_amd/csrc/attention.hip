@@ -154,11 +154,16 @@ __device__ __forceinline__ bf16x8_t join_bf16x8(const uint2& lo, const uint2& hi
 }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-#define PF_THREADS 256
-#define PF_ROWS 128   // query rows (token x head of the group) per block
+#define PF_THREADS 256   // threads of a team
+#define PF_ROWS 128      // query rows (token x head of the group) per block
+// two teams for head sizes up to 64: there a wave gets by with the 128 registers that 16 waves on a compute unit leave it
+#define PF_TEAMS (HEAD_DIM <= 64 ? 2 : 1)
 
 // Prefill.  grid (q tiles, sequences, kv heads).  bq = tokens per block (bq * group <= 128).
-__global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
+// (At least two waves on a SIMD leave a wave at most 256 registers, all of them ordinary ones: the compiler then keeps
+// the MFMA results where the vector unit can reach them, instead of copying scores and sums in and out of the
+// accumulation registers in every turn.)
+__global__ __launch_bounds__(PF_THREADS* PF_TEAMS) __attribute__((amdgpu_waves_per_eu(PF_TEAMS == 2 ? 4 : 2))) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, const int32_t* __restrict__ cu_q,
     const int32_t* __restrict__ start_pos, const int32_t* __restrict__ slots, const int32_t* __restrict__ page_table,
     int max_pages, const bf16_t* __restrict__ cache, long long page_stride, long long v_off, int group, int bq, int window,
@@ -167,13 +172,20 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
   constexpr int KS = HD / 16;               // k steps of K Q^T (32x32x16)
   constexpr int DT = (HD + 31) / 32;        // 32-row tiles of the output's head dimension
   constexpr int KROW = HD * 2 + 16;         // bytes of a key row in LDS (padded)
-  constexpr int VROW = PAGE * 2 + 16;       // bytes of a row of transposed values in LDS
+  constexpr int VROW = PAGE * 2 + 8;        // bytes of a row of transposed values in LDS: 34 words, so that the 32 rows
+                                            // that half a wave reads 8 bytes of at a time fall on different banks
   constexpr int KCH = PAGE * HD / 8;        // 16-byte chunks of a key tile
   constexpr int VCH = HD * PAGE / 8;
   constexpr int NKC = (KCH + PF_THREADS - 1) / PF_THREADS;
   constexpr int NVC = (VCH + PF_THREADS - 1) / PF_THREADS;
-  __shared__ __attribute__((aligned(16))) char ldsK[PAGE * KROW];
-  __shared__ __attribute__((aligned(16))) char ldsV[DT * 32 * VROW];
+  constexpr int KBYTES = PAGE * KROW, VBYTES = DT * 32 * VROW;
+  constexpr int TEAMS = PF_TEAMS;
+  // Each team of four waves has a page of its own in LDS.  With two teams the block's pages go to them in turn, both
+  // teams work on the same 128 query rows, and team 1 hands its sums to team 0 through LDS at the end.
+  __shared__ __attribute__((aligned(16))) char lds_all[TEAMS * (KBYTES + VBYTES)];
+  static_assert(TEAMS == 1 || TEAMS * (KBYTES + VBYTES) >= PF_ROWS * (HD + 4) * 4, "the teams' merge must fit their pages");
+  char* ldsK = lds_all + (threadIdx.x / PF_THREADS) * (KBYTES + VBYTES);
+  char* ldsV = ldsK + KBYTES;
 
   const int seq = blockIdx.y, kvh = blockIdx.z;
   const int q0 = cu_q[seq], qn = cu_q[seq + 1] - q0;
@@ -188,7 +200,8 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
   const int start = start_pos[seq];
   const int slot = slots[seq];
   const int kv_len = start + qn;                          // keys the cache holds for this sequence now
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5;
+  const int team = threadIdx.x / PF_THREADS;
+  const int tid = threadIdx.x % PF_THREADS, lane = tid & 63, wave = tid >> 6, half = lane >> 5;     // within the team
 
   // this lane's query row
   const int r = wave * 32 + (lane & 31);
@@ -257,17 +270,24 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
 #pragma unroll
     for (int i = 0; i < NVC; ++i) {
       const int c = tid + i * PF_THREADS;
-      if (c < VCH) *(uint4*)(ldsV + (c >> 3) * VROW + (c & 7) * 16) = rv[i];
+      if (c < VCH) {                          // rows are 8-byte aligned only
+        *(uint2*)(ldsV + (c >> 3) * VROW + (c & 7) * 16) = make_uint2(rv[i].x, rv[i].y);
+        *(uint2*)(ldsV + (c >> 3) * VROW + (c & 7) * 16 + 8) = make_uint2(rv[i].z, rv[i].w);
+      }
     }
   };
 
-  fetch(pg_lo);
-  for (int pg = pg_lo; pg <= pg_hi; ++pg) {
-    stash();
+  // turn n: team t takes page pg_lo + n * TEAMS + t, if the block has that many
+  const int turns = (pg_hi - pg_lo + TEAMS) / TEAMS;
+  if (pg_lo + team <= pg_hi) fetch(pg_lo + team);
+  for (int turn = 0; turn < turns; ++turn) {
+    const int pg = pg_lo + turn * TEAMS + team;
+    const bool mine = pg <= pg_hi;
+    if (mine) stash();
     __syncthreads();
-    if (pg < pg_hi) fetch(pg + 1);
+    if (pg + TEAMS <= pg_hi) fetch(pg + TEAMS);
     const int key0 = pg * PAGE;
-    if (wave_ok && key0 <= w_pos_max && key0 + PAGE - 1 >= w_lo_min) {
+    if (mine && wave_ok && key0 <= w_pos_max && key0 + PAGE - 1 >= w_lo_min) {
       f32x16_t s[2];
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt) {
@@ -338,6 +358,43 @@ __global__ __launch_bounds__(PF_THREADS) void attn_prefill_kernel(
         }
     }
     __syncthreads();
+  }
+  if (TEAMS == 2) {
+    // team 1 leaves, for each of its rows, the weighted values, the maximum and the sum; team 0 adds them to its own
+    float* mrg = (float*)lds_all + (size_t)r * (HD + 4);      // rows of 16-byte pieces
+    if (team == 1) {
+#pragma unroll
+      for (int d = 0; d < DT; ++d)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+          const int dd = d * 32 + 8 * qd + 4 * half;
+          if (dd < HD) *(float4*)(mrg + dd) = make_float4(o[d][4 * qd], o[d][4 * qd + 1], o[d][4 * qd + 2], o[d][4 * qd + 3]);
+        }
+      if (half == 0) {
+        mrg[HD] = m;
+        mrg[HD + 1] = l;
+      }
+    }
+    __syncthreads();
+    if (team == 1) return;
+    const float m2 = mrg[HD], l2 = mrg[HD + 1];
+    const float mm = fmaxf(m, m2);
+    const float m_use = mm == -INFINITY ? 0.f : mm;
+    const float a1 = fast_exp2((m - m_use) * scale_log2e), a2 = fast_exp2((m2 - m_use) * scale_log2e);
+    l = l * a1 + l2 * a2;
+#pragma unroll
+    for (int d = 0; d < DT; ++d)
+#pragma unroll
+      for (int qd = 0; qd < 4; ++qd) {
+        const int dd = d * 32 + 8 * qd + 4 * half;
+        if (dd < HD) {
+          const float4 o2 = *(const float4*)(mrg + dd);
+          o[d][4 * qd] = o[d][4 * qd] * a1 + o2.x * a2;
+          o[d][4 * qd + 1] = o[d][4 * qd + 1] * a1 + o2.y * a2;
+          o[d][4 * qd + 2] = o[d][4 * qd + 2] * a1 + o2.z * a2;
+          o[d][4 * qd + 3] = o[d][4 * qd + 3] * a1 + o2.w * a2;
+        }
+      }
   }
   if (!row_ok) return;
   const float inv = 1.0f / l;
@@ -709,7 +766,7 @@ extern "C" const char* dlgo_attention_prefill(const void* q, int ldq, void* out,
   if (n_seq == 0 || max_q_len == 0) return nullptr;
   const int bq = PF_ROWS / group;
   dim3 grid((max_q_len + bq - 1) / bq, n_seq, n_kv);
-  hipLaunchKernelGGL(attn_prefill_kernel, grid, dim3(PF_THREADS), 0, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo, cu_q,
+  hipLaunchKernelGGL(attn_prefill_kernel, grid, dim3(PF_THREADS * PF_TEAMS), 0, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo, cu_q,
                      start_pos, slots, page_table, max_pages, (const bf16_t*)cache, page_stride, v_off, group, bq, window,
                      scale * LOG2E);
   DLGO_LAUNCH_CHECK("attention_prefill");
