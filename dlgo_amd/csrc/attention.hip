@@ -680,40 +680,61 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_kernel(
   }
 }
 
-// grid (sequences, heads); merges the partials of the splits that hold keys of the token, in page order.
+// grid (sequences, heads); merges the partials of the splits that hold keys of the token, in page order.  A lane takes
+// one element of the head (and every lane the same maxima and sums).  Eight splits at a time, their loads issued before
+// the token's position is known: which of them count is decided afterwards, so that the position and the partials
+// cost one trip to memory, not three.
 __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, int ldo,
                                                             const int32_t* __restrict__ positions, int n_heads,
                                                             int n_splits, int window) {
   constexpr int HD = HEAD_DIM;
   constexpr int PS = HD + 4;
+  constexpr int ND = (HD + WAVE - 1) / WAVE;           // elements of the head per lane
   const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
-  const int pos = positions[seq];
-  const int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
-  const int n_pages = pos / PAGE - lo / PAGE + 1;
-  const int span = (n_pages - 1 + n_splits) / n_splits;
-  const int s0 = 0, s1 = (n_pages - 1) / span;         // the splits that were given pages
   const float* base = part + (size_t)(seq * n_heads + head) * n_splits * PS;
-  float M = -INFINITY, L = 0.f;
-  for (int c0 = s0; c0 <= s1; c0 += WAVE) {            // weights of up to 64 splits at a time, one per lane
-    const int sl = c0 + lane;
-    const float ms = sl <= s1 ? base[(size_t)sl * PS + HD] : -INFINITY;
-    const float ls = sl <= s1 ? base[(size_t)sl * PS + HD + 1] : 0.f;
-    const float M_new = fmaxf(M, wave_max(ms));
-    L = L * fast_exp2(M - M_new) + wave_sum(fast_exp2(ms - M_new) * ls);
+  const int pos = positions[seq];
+  float M = -INFINITY, L = 0.f, acc[ND];
+#pragma unroll
+  for (int i = 0; i < ND; ++i) acc[i] = 0.f;
+  int s1 = 0;
+  for (int c0 = 0; c0 < n_splits && c0 <= s1; c0 += 8) {
+    float ms[8], ls[8], v[8][ND];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int sl = c0 + i < n_splits ? c0 + i : n_splits - 1;
+      ms[i] = base[(size_t)sl * PS + HD];
+      ls[i] = base[(size_t)sl * PS + HD + 1];
+#pragma unroll
+      for (int e = 0; e < ND; ++e) v[i][e] = base[(size_t)sl * PS + (e * WAVE + lane < HD ? e * WAVE + lane : HD - 1)];
+    }
+    if (c0 == 0) {
+      const int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+      const int n_pages = pos / PAGE - lo / PAGE + 1;
+      const int span = (n_pages - 1 + n_splits) / n_splits;
+      s1 = (n_pages - 1) / span;                     // the last split that was given pages
+    }
+    float M_new = M;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (c0 + i <= s1) M_new = fmaxf(M_new, ms[i]);
+    const float keep = fast_exp2(M - M_new);       // 0 at the first round (M = -inf, M_new finite: every split given pages holds a key)
+    L *= keep;
+#pragma unroll
+    for (int e = 0; e < ND; ++e) acc[e] *= keep;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      if (c0 + i <= s1) {
+        const float w = fast_exp2(ms[i] - M_new);
+        L = fmaf(w, ls[i], L);
+#pragma unroll
+        for (int e = 0; e < ND; ++e) acc[e] = fmaf(w, v[i][e], acc[e]);
+      }
     M = M_new;
   }
   const float inv = 1.0f / L;
-  for (int d0 = 0; d0 < HD; d0 += WAVE) {              // every lane stays in the loop: the shuffles need them all
-    const int d = d0 + lane < HD ? d0 + lane : HD - 1;
-    float acc = 0.f;
-    for (int c0 = s0; c0 <= s1; c0 += WAVE) {
-      const int sl = c0 + lane;
-      const float w = sl <= s1 ? fast_exp2(base[(size_t)sl * PS + HD] - M) : 0.f;
-      const int n = s1 - c0 + 1 < WAVE ? s1 - c0 + 1 : WAVE;
-      for (int i = 0; i < n; ++i) acc = fmaf(__shfl(w, i, WAVE), base[(size_t)(c0 + i) * PS + d], acc);
-    }
-    if (d0 + lane < HD) out[(size_t)seq * ldo + (size_t)head * HD + d] = f32_to_bf16(acc * inv);
-  }
+#pragma unroll
+  for (int e = 0; e < ND; ++e)
+    if (e * WAVE + lane < HD) out[(size_t)seq * ldo + (size_t)head * HD + e * WAVE + lane] = f32_to_bf16(acc[e] * inv);
 }
 
 extern "C" int dlgo_attention_head_dim() { return HEAD_DIM; }

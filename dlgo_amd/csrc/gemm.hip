@@ -343,12 +343,20 @@ __global__ __launch_bounds__(256) void split_sum_kernel(const float* __restrict_
   const float* p = part + (size_t)t * N + n;
   float v[4] = {0.f, 0.f, 0.f, 0.f};
   if ((N & 3) == 0) {
-    for (int r = 0; r < runs; ++r) {
-      const float4 x = *(const float4*)(p + (size_t)r * run_stride);
-      v[0] += x.x;
-      v[1] += x.y;
-      v[2] += x.z;
-      v[3] += x.w;
+    // eight runs at a time, all loads of a round on their way before the first sum (the last run stands in for those
+    // beyond it, and is not added twice)
+    for (int r0 = 0; r0 < runs; r0 += 8) {
+      float4 x[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = *(const float4*)(p + (size_t)(r0 + i < runs ? r0 + i : runs - 1) * run_stride);
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (r0 + i < runs) {
+          v[0] += x[i].x;
+          v[1] += x[i].y;
+          v[2] += x[i].z;
+          v[3] += x[i].w;
+        }
     }
   } else {
     for (int r = 0; r < runs; ++r)
