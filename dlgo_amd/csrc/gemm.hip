@@ -406,9 +406,9 @@ static const char* launch_tiled(const void* W, const void* X, void* Y, int N, in
 template <typename T, int EPI>
 static const char* dispatch(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy, int force,
                             int splits, float* part, long long part_elems, hipStream_t stream) {
-  // force: 0 = choose, 2 = 128x128 tiles, 3 = 64x64, 4 = 32x32, 10 = 256x128, 11 = 256x256, 12 = 256x256 with 8 waves,
-  // 13 = 128x64, 14 = 64x128; direct loads into LDS: 20 = 256x256 with 16 waves, 21 = 128x128 with 8 waves and two
-  // blocks on a compute unit, 22 = 128x128 with 8 waves and three stages, 23 = 64x64 with four stages.
+  // force: 0 = choose, 2 = 128x128 tiles, 3 = 64x64, 4 = 32x32, 12 = 256x256 with 8 waves, 14 = 64x128; direct loads
+  // into LDS: 20 = 256x256 with 16 waves, 21 = 128x128 with 8 waves and two blocks on a compute unit, 22 = 128x128
+  // with 8 waves and three stages, 23 = 64x64 with four stages.
   // splits: 0 = choose, 1 = every block sums the whole of k, more = k in that many runs (64x64 tiles; needs part)
   int kind = force;
   const bool direct = direct_takes(K, ldw, ldx, sizeof(T));
@@ -451,11 +451,8 @@ static const char* dispatch(const void* W, const void* X, void* Y, int N, int Tn
     // the largest tile that still gives every compute unit a block, and two where one block would leave a SIMD one wave
     kind = b256 >= 256 ? 12 : (big >= 512 ? 2 : (tall >= 256 ? 14 : (big >= 256 ? 2 : (mid >= 256 ? 3 : 4))));
   }
-  if (kind == 13) return launch_tiled<T, 128, 64, 2, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 14) return launch_tiled<T, 64, 128, 2, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 12) return launch_tiled<T, 256, 256, 2, 4, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
-  if (kind == 11) return launch_tiled<T, 256, 256, 2, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
-  if (kind == 10) return launch_tiled<T, 256, 128, 2, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 2) return launch_tiled<T, 128, 128, 2, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 3) return launch_tiled<T, 64, 64, 2, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   return launch_tiled<T, 32, 32, 1, 1, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
@@ -488,7 +485,7 @@ extern "C" const char* dlgo_gemm(const void* W, const void* X, void* Y, int dtyp
   DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm: SwiGLU epilogue needs an even N and ldy >= N/2");
   DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm: ldy %d shorter than N %d", ldy, N);
   DLGO_REQUIRE(splits >= 0 && part_elems >= 0, "gemm: bad split %d", splits);
-  DLGO_REQUIRE(force_kind == 0 || (force_kind >= 2 && force_kind <= 4) || (force_kind >= 10 && force_kind <= 14) ||
+  DLGO_REQUIRE(force_kind == 0 || (force_kind >= 2 && force_kind <= 4) || force_kind == 12 || force_kind == 14 ||
                    (force_kind >= 20 && force_kind <= 23),
                "gemm: unknown kernel choice %d", force_kind);
   if (Tn == 0) return nullptr;
