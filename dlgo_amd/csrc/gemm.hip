@@ -365,6 +365,67 @@ __global__ __launch_bounds__(256) void split_sum_kernel(const float* __restrict_
   epilogue4<T, EPI>(Y, ldy, N, t, n, v[0], v[1], v[2], v[3]);
 }
 
+// The same sum for a product that adds into the float32 residual stream, one block per token, which then also leaves
+// rmsnorm(new row) * norm_w in `normed` (run dtype): the norm that the next part would otherwise run as a kernel of
+// its own (out = x * (1 / sqrt(sum(x^2)/N + eps)) * w, as rmsnorm.hip).  N is a multiple of 4, at most 1024 * NCH.
+template <typename T, int NCH>
+__global__ __launch_bounds__(256) void split_sum_norm_kernel(const float* __restrict__ part, int runs, long long run_stride,
+                                                             float* __restrict__ Y, int ldy, int N,
+                                                             const float* __restrict__ norm_w, float eps, T* __restrict__ normed,
+                                                             int ldn) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const float* p = part + (size_t)t * N;
+  float* y = Y + (size_t)t * ldy;
+  float4 row[NCH];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int n = (c * 256 + threadIdx.x) * 4;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (n < N) {
+      const float4 old = *(const float4*)(y + n);
+      for (int r0 = 0; r0 < runs; r0 += 8) {
+        float4 x[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = *(const float4*)(p + n + (size_t)(r0 + i < runs ? r0 + i : runs - 1) * run_stride);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          if (r0 + i < runs) {
+            v.x += x[i].x;
+            v.y += x[i].y;
+            v.z += x[i].z;
+            v.w += x[i].w;
+          }
+      }
+      v.x += old.x;
+      v.y += old.y;
+      v.z += old.z;
+      v.w += old.w;
+      *(float4*)(y + n) = v;
+      ss += v.x * v.x;
+      ss += v.y * v.y;
+      ss += v.z * v.z;
+      ss += v.w * v.w;
+    }
+    row[c] = v;
+  }
+  ss = block_sum<4>(ss, red);
+  const float scale = 1.0f / sqrtf(ss / (float)N + eps);
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int n = (c * 256 + threadIdx.x) * 4;
+    if (n < N) {
+      const float4 w = *(const float4*)(norm_w + n);
+      T* o = normed + (size_t)t * ldn + n;
+      Elem<T>::store(o, row[c].x * scale * w.x);
+      Elem<T>::store(o + 1, row[c].y * scale * w.y);
+      Elem<T>::store(o + 2, row[c].z * scale * w.z);
+      Elem<T>::store(o + 3, row[c].w * scale * w.w);
+    }
+  }
+}
+
 // Few rows of X and few rows of W leave a chip of 256 compute units idle unless k is shared out as well: the runs of
 // k go to blocks of their own (64x64 tiles), and split_sum_kernel adds their sums in a fixed order.
 template <typename T, int EPI, int BN = 64, int BT = 64, int WN = 2, int WT = 2, int NS = 4>
@@ -403,26 +464,28 @@ static const char* launch_tiled(const void* W, const void* X, void* Y, int N, in
   return nullptr;
 }
 
+// In how many runs a product shares its k tiles out when the choice is the kernel's: few rows of X, few tiles of output.
+static int auto_splits(int N, int Tn, int nk_all, long long part_elems) {
+  const long small = (long)((N + 63) / 64) * ((Tn + 63) / 64);
+  if (!(Tn <= 128 && small <= 64 && nk_all >= 32)) return 1;
+  int splits = (int)(256 / small);                          // a block for every compute unit ...
+  if (splits > nk_all / 8) splits = nk_all / 8;             // ... of at least eight k tiles
+  if ((long long)splits * Tn * N > part_elems) splits = 1;
+  return splits;
+}
+
 template <typename T, int EPI>
 static const char* dispatch(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy, int force,
                             int splits, float* part, long long part_elems, hipStream_t stream) {
   // force: 0 = choose, 2 = 128x128 tiles, 3 = 64x64, 4 = 32x32, 12 = 256x256 with 8 waves, 14 = 64x128; direct loads
   // into LDS: 20 = 256x256 with 16 waves, 21 = 128x128 with 8 waves and two blocks on a compute unit, 22 = 128x128
-  // with 8 waves and three stages, 23 = 64x64 with four stages.
+  // with 16 waves and three stages, 23 = 64x64 with four stages.
   // splits: 0 = choose, 1 = every block sums the whole of k, more = k in that many runs (64x64 tiles; needs part)
   int kind = force;
   const bool direct = direct_takes(K, ldw, ldx, sizeof(T));
   if ((kind >= 20 || splits > 1) && !direct) DLGO_FAIL("gemm: kernel %d needs K %% %d == 0, got K=%d", kind, (int)(128 / sizeof(T)), K);
   const int nk_all = K / (int)(128 / sizeof(T));
-  if (splits == 0) {
-    splits = 1;
-    const long small = (long)((N + 63) / 64) * ((Tn + 63) / 64);
-    if (kind == 0 && direct && part && Tn <= 128 && small <= 64 && nk_all >= 32) {
-      splits = (int)(256 / small);                          // a block for every compute unit ...
-      if (splits > nk_all / 8) splits = nk_all / 8;         // ... of at least eight k tiles
-      if ((long long)splits * Tn * N > part_elems) splits = 1;
-    }
-  }
+  if (splits == 0) splits = kind == 0 && direct && part ? auto_splits(N, Tn, nk_all, part_elems) : 1;
   if (splits > 1) {
     DLGO_REQUIRE(kind == 0 || kind == 23, "gemm: k is split for the 64x64 tiles only, not kernel %d", kind);
     DLGO_REQUIRE(part && (long long)splits * Tn * N <= part_elems && ((uintptr_t)part & 15) == 0,
@@ -442,7 +505,7 @@ static const char* dispatch(const void* W, const void* X, void* Y, int N, int Tn
   if (kind == 23) return launch_direct<T, 64, 64, 2, 2, 4, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 20) return launch_direct<T, 256, 256, 4, 4, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 21) return launch_direct<T, 128, 128, 2, 4, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
-  if (kind == 22) return launch_direct<T, 128, 128, 4, 2, 3, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  if (kind == 22) return launch_direct<T, 128, 128, 4, 4, 3, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 0) {
     const long b256 = (long)((N + 255) / 256) * ((Tn + 255) / 256);
     const long big = (long)((N + 127) / 128) * ((Tn + 127) / 128);
@@ -492,5 +555,46 @@ extern "C" const char* dlgo_gemm(const void* W, const void* X, void* Y, int dtyp
   const char* err = by_epilogue<elem_t>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, force_kind, splits, part, part_elems, stream);
   if (err) return err;
   DLGO_LAUNCH_CHECK("gemm");
+  return nullptr;
+}
+
+// The number of runs dlgo_gemm would share k out in for this product, left to choose (1: it would not split).
+extern "C" int dlgo_gemm_auto_splits(int dtype, int N, int Tn, int K, int ldw, int ldx, long long part_elems) {
+  const size_t elem = dtype == DLGO_DTYPE_F32 ? 4 : 2;
+  if (N <= 0 || Tn <= 0 || K <= 0 || !direct_takes(K, ldw, ldx, elem)) return 1;
+  return auto_splits(N, Tn, K / (int)(128 / elem), part_elems);
+}
+
+// Y += X W^T with k shared out in `splits` runs (> 1), and normed = rmsnorm(Y) * norm_w of the new rows beside it.
+extern "C" const char* dlgo_gemm_accum_norm(const void* W, const void* X, float* Y, int dtype, int N, int Tn, int K, int ldw, int ldx,
+                                            int ldy, int splits, float* part, long long part_elems, const float* norm_w, float eps,
+                                            void* normed, int ldn, hipStream_t stream) {
+  DLGO_REQUIRE(N > 0 && Tn >= 0 && K > 0, "gemm: bad sizes N=%d T=%d K=%d", N, Tn, K);
+  DLGO_REQUIRE(dtype == DLGO_ELEM, "gemm: this library is built for dtype code %d, got %d", DLGO_ELEM, dtype);
+  const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
+  DLGO_REQUIRE(direct_takes(K, ldw, ldx, sizeof(elem_t)), "gemm: a split product needs K %% %d == 0, got K=%d", 8 * epc, K);
+  DLGO_REQUIRE(ldw % epc == 0 && ldx % epc == 0 && ldw >= K && ldx >= K, "gemm: row strides (%d, %d) must be multiples of %d and at least K", ldw, ldx, epc);
+  DLGO_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0, "gemm: W and X must be 16-byte aligned");
+  DLGO_REQUIRE(N % 4 == 0 && N <= 8192 && ldy % 4 == 0 && ldy >= N && ldn >= N, "gemm: the sum with a norm takes N %% 4 == 0 up to 8192, got %d", N);
+  DLGO_REQUIRE(((uintptr_t)Y & 15) == 0 && ((uintptr_t)norm_w & 15) == 0 && ((uintptr_t)part & 15) == 0, "gemm: Y, the norm weight and the scratch must be 16-byte aligned");
+  DLGO_REQUIRE(eps > 0.f, "gemm: eps must be positive");
+  const int nk_all = K / (int)(128 / sizeof(elem_t));
+  DLGO_REQUIRE(splits > 1 && splits <= nk_all, "gemm: %d runs of k with %d tiles", splits, nk_all);
+  DLGO_REQUIRE(part && (long long)splits * Tn * N <= part_elems, "gemm: %d runs of k need %lld floats of scratch, got %lld", splits,
+               (long long)splits * Tn * N, part_elems);
+  if (Tn == 0) return nullptr;
+  const long long plane = (long long)Tn * N;
+  const char* err = launch_direct<elem_t, 64, 64, 2, 2, 4, EPI_STORE_F32>(W, X, part, N, Tn, K, ldw, ldx, N, stream, splits, plane);
+  if (err) return err;
+  const int nk_split = (nk_all + splits - 1) / splits, runs = (nk_all + nk_split - 1) / nk_split;
+#define SUM_NORM(C_)                                                                                                              \
+  hipLaunchKernelGGL((split_sum_norm_kernel<elem_t, C_>), dim3((unsigned)Tn), dim3(256), 0, stream, part, runs, plane, Y, ldy, N, \
+                     norm_w, eps, (elem_t*)normed, ldn)
+  if (N <= 1024) SUM_NORM(1);
+  else if (N <= 2048) SUM_NORM(2);
+  else if (N <= 4096) SUM_NORM(4);
+  else SUM_NORM(8);
+#undef SUM_NORM
+  DLGO_LAUNCH_CHECK("gemm_accum_norm");
   return nullptr;
 }

@@ -79,7 +79,7 @@ def _lib(module: str, defines=()):
     lib = _libs.get(key)
     if lib is None:
         lib = build.load(module, defines)
-        for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_attention_rows",
+        for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_accum_norm", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_attention_rows",
                      "dlgo_attention_prefill", "dlgo_attention_decode", "dlgo_argmax", "dlgo_sample"):
             if hasattr(lib, name):
                 getattr(lib, name).restype = ctypes.c_char_p
@@ -121,6 +121,51 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
     return out
 
 
+def _streams_rows(weight: torch.Tensor, t: int, kind: int, has_scratch: bool, splits: int) -> bool:
+    """Whether a product of t rows with this weight goes to the weight-streaming kernels (else to the tiled ones)."""
+    n, k = weight.shape
+    # k in 128-byte pieces, if it is a whole number of them (what the kernels that load tiles straight into LDS take)
+    piece = 128 // weight.element_size()
+    nk = k // piece if k % piece == 0 else 0
+    can_split = has_scratch and splits != 1 and nk >= 32 and n <= 4096
+    if kind != GEMM_AUTO or splits > 1:
+        return kind in (GEMM_STREAM, 5, 6, 7, 8, 9)
+    if t <= GEMM_FEW_ROWS_WIDE:         # measured on the shapes of a 1B Llama: a long inner size is better split,
+        return not (can_split and nk >= 64) and not (n >= GEMM_VERY_WIDE and nk > 0)   # a vocabulary better tiled
+    if t <= GEMM_FEW_ROWS:
+        return n < 16384 and not (can_split and (nk >= 64 or t >= 24)) and (t <= 40 or nk == 0)
+    return False
+
+
+def gemm_accum_then_norm(weight: torch.Tensor, x: torch.Tensor, residual: torch.Tensor, scratch: Optional[torch.Tensor],
+                         norm_weight: torch.Tensor, eps: float, normed: torch.Tensor) -> bool:
+    """residual += x @ weight.T and, beside it, normed = rmsnorm(residual) * norm_weight of the new rows, if this
+    product is one whose inner size gemm() would share out over blocks (then the sum of the runs gives the norm for
+    nothing).  Returns False, having done nothing, if it is not: the caller then runs gemm() and the norm."""
+    _need(weight, "gemm weight", dims=2)
+    _need(x, "gemm input", weight.dtype, 2)
+    n, k = weight.shape
+    t = x.shape[0]
+    if scratch is None or t == 0 or n % 4 or n > 8192 or _streams_rows(weight, t, GEMM_AUTO, True, 0):
+        return False
+    _need(scratch, "gemm scratch", torch.float32, 1)
+    lib = _lib("gemm", (("DLGO_ELEM", dtype_code(weight.dtype)),))
+    ldw, ldx = _rows(weight, "gemm weight"), _rows(x, "gemm input")
+    splits = lib.dlgo_gemm_auto_splits(dtype_code(weight.dtype), n, t, k, ldw, ldx, ctypes.c_longlong(scratch.numel()))
+    if splits <= 1:
+        return False
+    _need(residual, "residual rows", torch.float32, 2)
+    _need(norm_weight, "norm weight", torch.float32, 1)
+    _need(normed, "normed rows", weight.dtype, 2)
+    if x.shape[1] != k or tuple(residual.shape) != (t, n) or tuple(normed.shape) != (t, n) or norm_weight.shape[0] != n:
+        raise KernelError(f"gemm_accum_then_norm: x {tuple(x.shape)}, residual {tuple(residual.shape)}, normed {tuple(normed.shape)} "
+                          f"and norm weight {tuple(norm_weight.shape)} do not fit weight {tuple(weight.shape)}")
+    _check(lib.dlgo_gemm_accum_norm(_ptr(weight), _ptr(x), _ptr(residual), dtype_code(weight.dtype), n, t, k, ldw, ldx,
+                                    _rows(residual, "residual rows"), splits, _ptr(scratch), ctypes.c_longlong(scratch.numel()),
+                                    _ptr(norm_weight), ctypes.c_float(eps), _ptr(normed), _rows(normed, "normed rows"), _stream()))
+    return True
+
+
 def gemm(weight: torch.Tensor, x: torch.Tensor, out: torch.Tensor, epilogue: int = EPI_STORE,
          kind: int = GEMM_AUTO, scratch: Optional[torch.Tensor] = None, splits: int = 0) -> torch.Tensor:
     """out (epilogue)= x @ weight.T with weight [N, K], x [T, K].
@@ -147,18 +192,7 @@ def gemm(weight: torch.Tensor, x: torch.Tensor, out: torch.Tensor, epilogue: int
         _need(scratch, "gemm scratch", torch.float32, 1)
     elif splits > 1:
         raise KernelError("gemm: a split product needs scratch")
-    # k in 128-byte pieces, if it is a whole number of them (what the kernels that load tiles straight into LDS take)
-    piece = 128 // weight.element_size()
-    nk = k // piece if k % piece == 0 else 0
-    can_split = scratch is not None and splits != 1 and nk >= 32 and n <= 4096
-    if kind != GEMM_AUTO or splits > 1:
-        rows_kernel = kind in (GEMM_STREAM, 5, 6, 7, 8, 9)
-    elif t <= GEMM_FEW_ROWS_WIDE:       # measured on the shapes of a 1B Llama: a long inner size is better split,
-        rows_kernel = not (can_split and nk >= 64) and not (n >= GEMM_VERY_WIDE and nk > 0)   # a vocabulary better tiled
-    elif t <= GEMM_FEW_ROWS:
-        rows_kernel = n < 16384 and not (can_split and (nk >= 64 or t >= 24)) and (t <= 40 or nk == 0)
-    else:
-        rows_kernel = False
+    rows_kernel = _streams_rows(weight, t, kind, scratch is not None, splits)
     args = (_ptr(weight), _ptr(x), _ptr(out), dtype_code(weight.dtype), n, t, k, _rows(weight, "gemm weight"),
             _rows(x, "gemm input"), _rows(out, "gemm output"), epilogue)
     if rows_kernel:

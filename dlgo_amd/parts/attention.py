@@ -33,7 +33,11 @@ class Mixer(Part):
     the result is added into `residual` (float32 [T, width]).  `unit` is the cache unit this run reads;
     `owns_cache` is False when the unit belongs to another run (then nothing is stored).
     A mixer with state must treat the rows of a sequence in order: ctx.cu_q gives each sequence's rows.
+
+    A mixer that sets `leaves_norm` also takes then=(norm part, rows): "if it costs you nothing, leave that norm of
+    the residual rows as they are after you in `rows`", and returns True if it did (the block then skips the norm).
     """
+    leaves_norm = False
 
     def cache_needs(self) -> List[CacheNeed]:
         return []
@@ -52,6 +56,7 @@ class Mixer(Part):
 
 class Attention(Mixer):
     kernel_modules = ("gemm", "gemm_rows", "rope_kv")
+    leaves_norm = True
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PositionEncoding,
                  window: Optional[int] = None, scale: Optional[float] = None):
@@ -97,7 +102,7 @@ class Attention(Mixer):
     def fuses_norm(self, norm, ctx) -> bool:
         return isinstance(norm, RMSNorm) and ops.fused_norm_pays(self.w_qkv, ctx.n_tokens)
 
-    def forward(self, xn, ctx, unit, residual, owns_cache=True, norm=None) -> None:
+    def forward(self, xn, ctx, unit, residual, owns_cache=True, norm=None, then=None) -> bool:
         t = xn.shape[0]
         n_kv = self.n_kv_heads if owns_cache else 0
         cols = self.q_dim + 2 * n_kv * self.head_dim
@@ -119,7 +124,11 @@ class Attention(Mixer):
         out = ctx.buffer("attention.out", (t, self.q_dim), ctx.dtype)
         self.attend(qkv, out, ctx, kv, rotation=(rot.cos, rot.sin, rot.width, rot.interleaved) if fused and rot else None,
                     new_kv=fused and owns_cache)
+        if then is not None and isinstance(then[0], RMSNorm) and ops.gemm_accum_then_norm(
+                self.w_o, out, residual, split, then[0].weight, then[0].eps, then[1]):
+            return True
         ops.gemm(self.w_o, out, residual, ops.EPI_ACCUM_F32, scratch=split)
+        return False
 
     def attend(self, q, out, ctx, kv, rotation=None, new_kv=False) -> None:
         """Attention of the step's (rotated) query rows over the cache; the kernel is chosen by the

@@ -14,7 +14,12 @@ from .feed_forward import FeedForward
 
 class Block(Part):
     """Interface: parts() names the sub-parts (the names become tensor-name prefixes);
-    forward(x, ctx, unit, owns_cache) updates the float32 residual rows x in place."""
+    forward(x, ctx, unit, owns_cache) updates the float32 residual rows x in place.
+
+    A block that sets `takes_normed` has an `entry_norm` (the norm it applies to x first) and a forward that also takes
+    normed= (rows that already hold entry_norm(x), left by the block before) and then=(the next block's entry norm,
+    rows), and returns True if it left that norm of its result in `rows`."""
+    takes_normed = False
 
     def parts(self) -> List[Tuple[str, Part]]:
         raise NotImplementedError
@@ -40,18 +45,36 @@ class PreNormBlock(Block):
     def mixer(self) -> Mixer:
         return self._mixer
 
-    def forward(self, x, ctx, unit, owns_cache=True) -> None:
+    takes_normed = True
+
+    @property
+    def entry_norm(self) -> Part:
+        return self.mixer_norm
+
+    def forward(self, x, ctx, unit, owns_cache=True, normed=None, then=None) -> bool:
         xn = ctx.buffer("block.normed", tuple(x.shape), ctx.dtype)
-        if self._mixer.fuses_norm(self.mixer_norm, ctx):
-            self._mixer.forward(x, ctx, unit, x, owns_cache, norm=self.mixer_norm)
+        # the mixer may leave the feed-forward's norm of its result, the feed-forward the next block's entry norm
+        after = (self.ffn_norm, xn) if self._mixer.leaves_norm else None
+        if normed is not None:
+            left = self._mixer.forward(normed, ctx, unit, x, owns_cache, **({"then": after} if after else {}))
+        elif self._mixer.fuses_norm(self.mixer_norm, ctx):
+            left = self._mixer.forward(x, ctx, unit, x, owns_cache, norm=self.mixer_norm, **({"then": after} if after else {}))
         else:
             self.mixer_norm(x, xn)
-            self._mixer.forward(xn, ctx, unit, x, owns_cache)
+            # the mixer reads xn until its last product, whose sum is what writes the norm: a buffer of its own
+            mid = ctx.buffer("block.normed_mid", tuple(x.shape), ctx.dtype) if after else None
+            if after:
+                after = (self.ffn_norm, mid)
+            left = self._mixer.forward(xn, ctx, unit, x, owns_cache, **({"then": after} if after else {}))
+            if left:
+                xn = mid
+        onward = {"then": then} if then is not None and self.ffn.leaves_norm else {}
+        if left:
+            return bool(self.ffn.forward(xn, ctx, x, **onward))
         if self.ffn.fuses_norm(self.ffn_norm, ctx):
-            self.ffn.forward(x, ctx, x, norm=self.ffn_norm)
-        else:
-            self.ffn_norm(x, xn)
-            self.ffn.forward(xn, ctx, x)
+            return bool(self.ffn.forward(x, ctx, x, norm=self.ffn_norm, **onward))
+        self.ffn_norm(x, xn)
+        return bool(self.ffn.forward(xn, ctx, x, **onward))
 
 
 BLOCKS = {"pre_norm": PreNormBlock}

@@ -15,7 +15,10 @@ from .norm import RMSNorm
 
 
 class FeedForward(Part):
-    """Interface: forward(xn, ctx, residual) adds the result for the step's rows into `residual`."""
+    """Interface: forward(xn, ctx, residual) adds the result for the step's rows into `residual`.  One that sets
+    `leaves_norm` also takes then=(norm part, rows) and returns True if it left that norm of the new residual rows
+    in `rows` (see Mixer)."""
+    leaves_norm = False
 
     def fuses_norm(self, norm, ctx) -> bool:
         """True if, for this step, it would rather be given the float32 residual rows and the norm part."""
@@ -27,6 +30,7 @@ class FeedForward(Part):
 
 class GatedFeedForward(FeedForward):
     kernel_modules = ("gemm", "gemm_rows")
+    leaves_norm = True
 
     def __init__(self, width: int, inner: int, activation: str = "silu"):
         if activation != "silu":
@@ -55,10 +59,15 @@ class GatedFeedForward(FeedForward):
     def fuses_norm(self, norm, ctx) -> bool:
         return isinstance(norm, RMSNorm) and ops.fused_norm_pays(self.w_gate_up, ctx.n_tokens)
 
-    def forward(self, xn, ctx, residual, norm=None) -> None:
+    def forward(self, xn, ctx, residual, norm=None, then=None) -> bool:
         hid = ctx.buffer("feed_forward.hidden", (xn.shape[0], self.inner), ctx.dtype)
         if norm is not None:      # xn are the float32 residual rows: the norm rides in the product
             ops.gemm_rmsnorm(self.w_gate_up, xn, norm.weight, norm.eps, hid, ops.EPI_SWIGLU)
         else:
             ops.gemm(self.w_gate_up, xn, hid, ops.EPI_SWIGLU)
-        ops.gemm(self.w_down, hid, residual, ops.EPI_ACCUM_F32, scratch=ctx.scratch("gemm.split", ops.GEMM_SPLIT_FLOATS, torch.float32))
+        split = ctx.scratch("gemm.split", ops.GEMM_SPLIT_FLOATS, torch.float32)
+        if then is not None and isinstance(then[0], RMSNorm) and ops.gemm_accum_then_norm(
+                self.w_down, hid, residual, split, then[0].weight, then[0].eps, then[1]):
+            return True
+        ops.gemm(self.w_down, hid, residual, ops.EPI_ACCUM_F32, scratch=split)
+        return False

@@ -99,8 +99,20 @@ class DecoderModel:
         self.embedding(token_ids, x)
         if self.position is not None:
             self.position.on_embedding(x, ctx)
+        # A block may leave the next block's entry norm of its result beside the result (two sets of rows in turn).
+        normed = None
         for i, run in enumerate(self.order):
-            self.layers[run.layer][1].forward(x, ctx, self.run_unit[i], self.run_owns[i])
+            block = self.layers[run.layer][1]
+            if not block.takes_normed:
+                block.forward(x, ctx, self.run_unit[i], self.run_owns[i])
+                normed = None
+                continue
+            nxt = self.layers[self.order[i + 1].layer][1] if i + 1 < len(self.order) else None
+            then = None
+            if nxt is not None and nxt.takes_normed:
+                then = (nxt.entry_norm, ctx.buffer(f"model.normed.{i & 1}", tuple(x.shape), ctx.dtype))
+            left = block.forward(x, ctx, self.run_unit[i], self.run_owns[i], normed=normed, then=then)
+            normed = then[1] if left else None
         return x
 
     def logits(self, ctx, x: torch.Tensor, rows: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:

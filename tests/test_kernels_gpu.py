@@ -172,6 +172,42 @@ def test_gemm_with_split_inner_size(dtype, _, rel, n, t, k, splits):
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("n,t,k,fused", [(2048, 8, 8192, True), (1024, 64, 4096, True), (4096, 33, 8192, True), (3072, 30, 2048, True),
+                                         (2052, 8, 8192, True), (2048, 8, 512, False), (2050, 8, 8192, False), (2048, 200, 8192, False)])
+def test_gemm_into_the_residual_that_leaves_the_next_norm(dtype, _, rel, n, t, k, fused):
+    """A product whose inner size is shared out adds into the residual rows and leaves their RMSNorm beside them; where
+    the product would not be split (or N does not suit) it does nothing and says so."""
+    ops = _ops()
+    if dtype == torch.float32:
+        k //= 2
+    g = torch.Generator().manual_seed(n + t)
+    w = (0.05 * torch.randn(n, k, generator=g)).to(dtype).to(DEV)
+    x = torch.randn(t, k, generator=g).to(dtype).to(DEV)
+    res = (torch.randn(t, n, generator=g) * (1 + torch.arange(t)[:, None] % 3)).to(DEV)
+    nw = (1 + 0.3 * torch.randn(n, generator=g)).to(DEV)
+    eps = 1e-3
+    scratch = torch.full((ops.GEMM_SPLIT_FLOATS,), float("nan"), device=DEV)
+    normed = torch.full((t, n), float("nan"), dtype=dtype, device=DEV)
+    res0 = res.clone()
+    did = ops.gemm_accum_then_norm(w, x, res, scratch, nw, eps, normed)
+    assert did == fused
+    if not did:
+        assert torch.equal(res, res0) and torch.isnan(normed.float()).all()
+        return
+    want = res0.double() + x.double() @ w.double().T
+    close(res, want, 1e-5, "residual")
+    rd = res.double()                                  # the norm of the rows as the kernel left them
+    close(normed, rd / torch.sqrt((rd * rd).mean(-1, keepdim=True) + eps) * nw.double(), 1e-5 if dtype == torch.float32 else 8e-3, "norm")
+    # the same bits as the separate way: split product, then the norm kernel
+    res2 = res0.clone()
+    ops.gemm(w, x, res2, ops.EPI_ACCUM_F32, scratch=scratch)
+    assert torch.equal(res2, res)
+    normed2 = torch.empty_like(normed)
+    ops.rmsnorm(res2, nw, eps, normed2)
+    close(normed2, normed.double(), 1e-6 if dtype == torch.float32 else 8e-3, "norm kernel")
+
+
+@pytest.mark.parametrize("dtype,_,rel", DT)
 @pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5])
 @pytest.mark.parametrize("f,t,k", [(160, 5, 64), (352, 70, 128), (9, 2, 16), (1030, 200, 72), (40, 33, 2056), (8200, 64, 256), (16401, 9, 2048)])
 def test_gemm_swiglu(dtype, _, rel, kind, f, t, k):
