@@ -32,12 +32,30 @@ __device__ __forceinline__ BestIdx better(BestIdx a, BestIdx b) {
   return a;
 }
 
-__device__ BestIdx block_argmax(const float* row, int V, BestIdx* red) {
-  BestIdx best = {-INFINITY, -1};
-  for (int i = threadIdx.x; i < V; i += SAMP_THREADS) {
-    const float v = row[i];
-    if (v == v) best = better(best, BestIdx{v, i});
+// f(index, value) for every element of a row, the block's threads striding over it; 16 bytes a thread at a time, and
+// several of them on their way at once, where the row allows (vec).
+template <typename F>
+__device__ __forceinline__ void for_each_element(const float* __restrict__ row, int V, bool vec, F f) {
+  if (vec) {
+    const float4* r4 = (const float4*)row;
+#pragma unroll 4
+    for (int i = threadIdx.x; i < V / 4; i += SAMP_THREADS) {
+      const float4 x = r4[i];
+      f(4 * i, x.x);
+      f(4 * i + 1, x.y);
+      f(4 * i + 2, x.z);
+      f(4 * i + 3, x.w);
+    }
+  } else {
+    for (int i = threadIdx.x; i < V; i += SAMP_THREADS) f(i, row[i]);
   }
+}
+
+__device__ BestIdx block_argmax(const float* row, int V, BestIdx* red, bool vec = false) {
+  BestIdx best = {-INFINITY, -1};
+  for_each_element(row, V, vec, [&](int i, float v) {
+    if (v == v) best = better(best, BestIdx{v, i});
+  });
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
     BestIdx other;
@@ -111,17 +129,105 @@ __global__ __launch_bounds__(WAVE) void argmax_final_kernel(const BestIdx* __res
 // Largest key tau with measure({i : key_i >= tau}) >= need, by bisection on the key's bits.
 // COUNT: the measure counts elements (top-k); else it sums e_i (top-p).
 template <bool COUNT>
-__device__ uint32_t bisect_threshold(const float* work, const float* e, int V, float need, float* red) {
+__device__ uint32_t bisect_threshold(const float* work, const float* e, int V, float need, float* red, bool vec = false) {
   uint32_t prefix = 0;
   for (int bit = 31; bit >= 0; --bit) {
     const uint32_t cand = prefix | (1u << bit);
     float part = 0.f;
-    for (int i = threadIdx.x; i < V; i += SAMP_THREADS)
-      if (order_key(work[i]) >= cand) part += COUNT ? 1.0f : e[i];
+    if (vec) {
+#pragma unroll 4
+      for (int i = threadIdx.x; i < V / 4; i += SAMP_THREADS) {
+        const float4 w4 = ((const float4*)work)[i];
+        const float4 e4 = COUNT ? make_float4(1.f, 1.f, 1.f, 1.f) : ((const float4*)e)[i];
+        if (order_key(w4.x) >= cand) part += e4.x;
+        if (order_key(w4.y) >= cand) part += e4.y;
+        if (order_key(w4.z) >= cand) part += e4.z;
+        if (order_key(w4.w) >= cand) part += e4.w;
+      }
+    } else {
+      for (int i = threadIdx.x; i < V; i += SAMP_THREADS)
+        if (order_key(work[i]) >= cand) part += COUNT ? 1.0f : e[i];
+    }
     const float total = block_sum_f(part, red);
     if (total >= need) prefix = cand;
   }
   return prefix;
+}
+
+// The candidates of a row after top-k, when they are few enough to sit in LDS one to a thread: the exact top-k cut, top-p,
+// min-p and the draw, all in index order.  cv/ci hold n candidates in any order; every element outside them is masked.
+#define SAMP_CAND SAMP_THREADS
+struct SampleSmall {
+  float cv[SAMP_CAND];
+  int ci[SAMP_CAND];
+  float sv[SAMP_CAND];
+  int si[SAMP_CAND];
+  float se[SAMP_CAND];
+  uint32_t skey[SAMP_CAND];
+  float scan[SAMP_THREADS];
+  int n, first, last;
+  uint32_t tau;
+};
+
+__device__ int sample_small(SampleSmall& S, int n, int k, BestIdx top, float tp, float mp, float u) {
+  const int j = threadIdx.x;
+  const bool have = j < n;
+  // into index order
+  const int my_i0 = have ? S.ci[j] : 0x7fffffff;
+  const float my_v0 = have ? S.cv[j] : -INFINITY;
+  int pos = 0;
+  for (int i = 0; i < n; ++i) pos += S.ci[i] < my_i0;
+  if (have) {
+    S.sv[pos] = my_v0;
+    S.si[pos] = my_i0;
+  }
+  if (j == 0) {
+    S.first = 0x7fffffff;
+    S.last = -1;
+    S.tau = 0;
+  }
+  __syncthreads();
+  const float v = have ? S.sv[j] : -INFINITY;
+  const uint32_t key = order_key(v);
+  S.skey[j] = have ? key : 0u;
+  __syncthreads();
+  // top-k: an element stays if fewer than k are strictly larger (ties at the cut all stay)
+  int rank = 0;
+  for (int i = 0; i < n; ++i) rank += S.skey[i] > key;
+  bool keep = have && rank < k;
+  float e = keep ? expf(v - top.v) : 0.f;
+  if (tp < 1.0f) {      // top-p: the largest cut whose elements at or above it hold p of the mass
+    S.se[j] = e;
+    __syncthreads();
+    float Z = 0.f, mass = 0.f;
+    for (int i = 0; i < n; ++i) {
+      const float ei = S.se[i];
+      Z += ei;
+      if (S.skey[i] >= key) mass += ei;
+    }
+    if (keep && mass >= tp * Z) atomicMax(&S.tau, key);
+    __syncthreads();
+    keep = keep && key >= S.tau;
+  }
+  if (mp > 0.f) keep = keep && !(v < top.v + logf(mp));
+  e = keep ? e : 0.f;
+  // inverse-CDF draw over the cumulative sums in index order
+  S.scan[j] = e;
+  __syncthreads();
+  for (int o = 1; o < SAMP_THREADS; o <<= 1) {
+    const float add = j >= o ? S.scan[j - o] : 0.f;
+    __syncthreads();
+    S.scan[j] += add;
+    __syncthreads();
+  }
+  const float target = u * S.scan[SAMP_THREADS - 1];
+  if (e > 0.f) {
+    if (S.scan[j] >= target) atomicMin(&S.first, j);
+    atomicMax(&S.last, j);
+  }
+  __syncthreads();
+  const int pick = S.first != 0x7fffffff ? S.first : S.last;
+  return pick >= 0 ? S.si[pick] : (top.i < 0 ? 0 : top.i);
 }
 
 __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __restrict__ logits, int ld, int V,
@@ -129,12 +235,15 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
                                                               const float* __restrict__ temperature,
                                                               const int32_t* __restrict__ top_k, const float* __restrict__ top_p,
                                                               const float* __restrict__ min_p, const float* __restrict__ penalty,
-                                                              const int32_t* __restrict__ recent, int n_recent,
+                                                              int32_t* __restrict__ recent, int n_recent,
+                                                              const int32_t* __restrict__ recent_rows, int32_t* __restrict__ counts,
                                                               const float* __restrict__ uniform, int32_t* __restrict__ out) {
   __shared__ BestIdx redb[SAMP_WAVES];
   __shared__ float red[SAMP_WAVES];
-  __shared__ float scan[SAMP_THREADS];
-  __shared__ int chosen;
+  __shared__ SampleSmall S;
+  __shared__ int hist[256];
+  __shared__ int chosen, bstar;
+  float* scan = S.scan;
   const int row = blockIdx.x;
   const float* lg = logits + (size_t)row * ld;
   const float temp = temperature[row];
@@ -146,32 +255,100 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
   float* work = work_all + (size_t)row * V;
   float* e = e_all + (size_t)row * V;
   const float inv_temp = temp == 1.0f ? 1.0f : 1.0f / temp;
-  for (int i = threadIdx.x; i < V; i += SAMP_THREADS) work[i] = lg[i];
+  // temperature for all, then the repetition penalty (which comes first in the pipeline) redone for the few it touches
+  const bool vec = (V & 3) == 0 && (ld & 3) == 0 && ((uintptr_t)logits & 15) == 0 && ((uintptr_t)work_all & 15) == 0;
+  if (vec) {
+#pragma unroll 4
+    for (int i = threadIdx.x; i < V / 4; i += SAMP_THREADS) {
+      float4 x = ((const float4*)lg)[i];
+      if (inv_temp != 1.0f) {
+        x.x *= inv_temp;
+        x.y *= inv_temp;
+        x.z *= inv_temp;
+        x.w *= inv_temp;
+      }
+      ((float4*)work)[i] = x;
+    }
+  } else {
+    for (int i = threadIdx.x; i < V; i += SAMP_THREADS) work[i] = inv_temp != 1.0f ? lg[i] * inv_temp : lg[i];
+  }
   __syncthreads();
   // repetition penalty: each distinct recent token once
+  // The recent tokens of this row: row `rr` of the table, all n_recent entries (-1 where empty), or with `counts` a
+  // ring that holds the last min(counts[rr], n_recent) tokens, to which the token chosen here is added at the end.
   const float pen = penalty[row];
-  if (pen > 1.0f && n_recent > 0 && (int)threadIdx.x < n_recent) {
-    const int32_t* rc = recent + (size_t)row * n_recent;
+  const int rr = recent_rows ? recent_rows[row] : row;
+  const int held = counts ? (counts[rr] < n_recent ? counts[rr] : n_recent) : n_recent;
+  auto finish = [&](int tok) {           // thread 0
+    out[row] = tok;
+    if (counts && n_recent > 0) {
+      recent[(size_t)rr * n_recent + counts[rr] % n_recent] = tok;
+      counts[rr] += 1;
+    }
+  };
+  if (pen > 1.0f && n_recent > 0 && (int)threadIdx.x < held) {
+    const int32_t* rc = recent + (size_t)rr * n_recent;
     const int tok = rc[threadIdx.x];
     bool first = tok >= 0 && tok < V;
     for (int j = 0; first && j < (int)threadIdx.x; ++j) first = rc[j] != tok;
-    if (first) work[tok] = work[tok] > 0.f ? work[tok] / pen : work[tok] * pen;
+    if (first) {
+      const float x = lg[tok] > 0.f ? lg[tok] / pen : lg[tok] * pen;
+      work[tok] = inv_temp != 1.0f ? x * inv_temp : x;
+    }
   }
   __syncthreads();
-  if (inv_temp != 1.0f)
-    for (int i = threadIdx.x; i < V; i += SAMP_THREADS) work[i] *= inv_temp;
-  __syncthreads();
-  // top-k: everything below the k-th largest value is masked; ties at it stay
+  BestIdx top = block_argmax(work, V, redb, vec);
   const int k = top_k[row];
+  const float tp = top_p[row], mp = min_p[row];
+  // top-k: everything below the k-th largest value is masked; ties at it stay
   if (k > 0 && k < V) {
-    const uint32_t tau = bisect_threshold<true>(work, nullptr, V, (float)k, red);
+    // Quick way: count the elements by their distance below the maximum (in steps of 2^16 of the ordered bit
+    // pattern: a sixteenth of a unit around 10), find the distance within which k of them lie, and if those are few,
+    // carry on with them alone.
+    const uint32_t kmax = order_key(top.v);
+    if (threadIdx.x < 256) hist[threadIdx.x] = 0;
+    if (threadIdx.x == 0) {
+      bstar = -1;
+      S.n = 0;
+    }
+    __syncthreads();
+    for_each_element(work, V, vec, [&](int, float x) {
+      const uint32_t bin = (kmax - order_key(x)) >> 16;
+      if (bin < 255u) atomicAdd(&hist[bin], 1);
+    });
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int cum = 0;
+      for (int b = 0; b < 255; ++b) {
+        cum += hist[b];
+        if (cum >= k) {
+          if (cum <= SAMP_CAND) bstar = b;
+          break;
+        }
+      }
+    }
+    __syncthreads();
+    if (bstar >= 0) {
+      const uint32_t lim = (uint32_t)bstar;
+      for_each_element(work, V, vec, [&](int i, float x) {
+        if (((kmax - order_key(x)) >> 16) <= lim) {
+          const int slot = atomicAdd(&S.n, 1);
+          S.cv[slot] = x;
+          S.ci[slot] = i;
+        }
+      });
+      __syncthreads();
+      const int pick = sample_small(S, S.n, k, top, tp, mp, uniform[row]);
+      if (threadIdx.x == 0) finish(pick);
+      return;
+    }
+    // many equal values at the cut, or the k-th value far below the maximum: the cut by bisection over the whole row
+    const uint32_t tau = bisect_threshold<true>(work, nullptr, V, (float)k, red, vec);
     for (int i = threadIdx.x; i < V; i += SAMP_THREADS)
       if (order_key(work[i]) < tau) work[i] = -INFINITY;
     __syncthreads();
   }
-  BestIdx top = block_argmax(work, V, redb);
   // top-p: smallest set, by falling probability, whose mass reaches p
-  const float tp = top_p[row];
   if (tp < 1.0f) {
     float part = 0.f;
     for (int i = threadIdx.x; i < V; i += SAMP_THREADS) {
@@ -181,57 +358,106 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
     }
     __syncthreads();
     const float Z = block_sum_f(part, red);
-    const uint32_t tau = bisect_threshold<false>(work, e, V, tp * Z, red);
+    const uint32_t tau = bisect_threshold<false>(work, e, V, tp * Z, red, vec && ((uintptr_t)e_all & 15) == 0);
     for (int i = threadIdx.x; i < V; i += SAMP_THREADS)
       if (order_key(work[i]) < tau) work[i] = -INFINITY;
     __syncthreads();
   }
   // min-p: probability below min_p * (largest probability) is masked
-  const float mp = min_p[row];
   if (mp > 0.f) {
     const float cut = top.v + logf(mp);
     for (int i = threadIdx.x; i < V; i += SAMP_THREADS)
       if (work[i] < cut) work[i] = -INFINITY;
     __syncthreads();
   }
-  // softmax and inverse-CDF draw, cumulative sums in index order
-  const int chunk = (V + SAMP_THREADS - 1) / SAMP_THREADS;
-  const int b0 = threadIdx.x * chunk, b1 = b0 + chunk < V ? b0 + chunk : V;
-  float mine = 0.f;
-  for (int i = b0; i < b1; ++i) {
-    const float v = expf(work[i] - top.v);
-    e[i] = v;
-    mine += v;
+  // softmax and inverse-CDF draw, cumulative sums in index order.  Each wave owns a run of the row and walks it 256
+  // elements at a time (four to a lane), adding them up within the lane and then by a scan over the lanes; the waves'
+  // totals, added in wave order, tell which wave holds the target, and that wave walks its run once more, with the
+  // same sums, to the element.
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int seg = ((V + SAMP_WAVES - 1) / SAMP_WAVES + 255) / 256 * 256;
+  const int w0 = wave * seg < V ? wave * seg : V, w1 = w0 + seg < V ? w0 + seg : V;
+  auto scan64 = [&](float x) {          // inclusive, lanes in order
+#pragma unroll
+    for (int o = 1; o < WAVE; o <<= 1) {
+      const float y = __shfl_up(x, o, WAVE);
+      if (lane >= o) x += y;
+    }
+    return x;
+  };
+  auto four = [&](int i, float* ev) {   // exp(work - top) of elements i..i+3 of the wave's run, 0 beyond it
+    float x[4];
+    if (vec && i + 3 < w1) {
+      const float4 v4 = *(const float4*)(work + i);
+      x[0] = v4.x; x[1] = v4.y; x[2] = v4.z; x[3] = v4.w;
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) x[c] = i + c < w1 ? work[i + c] : -INFINITY;
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) ev[c] = expf(x[c] - top.v);
+  };
+  float running = 0.f;
+#pragma unroll 2
+  for (int b = w0; b < w1; b += 4 * WAVE) {
+    float ev[4];
+    four(b + 4 * lane, ev);
+    const float mine = ((ev[0] + ev[1]) + ev[2]) + ev[3];
+    running += __shfl(scan64(mine), WAVE - 1, WAVE);
   }
-  scan[threadIdx.x] = mine;
+  if (lane == 0) scan[wave] = running;
   if (threadIdx.x == 0) chosen = -1;
   __syncthreads();
-  for (int o = 1; o < SAMP_THREADS; o <<= 1) {   // inclusive scan
-    const float add = (int)threadIdx.x >= o ? scan[threadIdx.x - o] : 0.f;
-    __syncthreads();
-    scan[threadIdx.x] += add;
-    __syncthreads();
+  float before = 0.f, Z = 0.f;
+  for (int w = 0; w < SAMP_WAVES; ++w) {
+    if (w < wave) before += scan[w];
+    Z += scan[w];
   }
-  const float Z = scan[SAMP_THREADS - 1];
   const float target = uniform[row] * Z;
-  const float incl = scan[threadIdx.x], excl = threadIdx.x ? scan[threadIdx.x - 1] : 0.f;
-  if (mine > 0.f && (excl < target || (threadIdx.x == 0 && target <= 0.f)) && target <= incl) {
-    float cum = excl;
-    int pick = -1, last = -1;
-    for (int i = b0; i < b1; ++i) {
-      if (e[i] > 0.f) {
-        cum += e[i];
-        last = i;
-        if (cum >= target) {
-          pick = i;
-          break;
-        }
+  // the first wave whose total reaches the target (the last one with anything in it, if rounding leaves none)
+  int holder = -1, last_full = -1;
+  {
+    float cum = 0.f;
+    for (int w = 0; w < SAMP_WAVES; ++w) {
+      cum += scan[w];
+      if (scan[w] > 0.f) {
+        last_full = w;
+        if (holder < 0 && cum >= target) holder = w;
       }
     }
-    chosen = pick >= 0 ? pick : last;
+    if (holder < 0) holder = last_full;
+  }
+  if (wave == holder) {
+    float cum = before;
+    int pick = -1, last = -1;
+    for (int b = w0; b < w1 && pick < 0; b += 4 * WAVE) {
+      float ev[4];
+      const int i0 = b + 4 * lane;
+      four(i0, ev);
+      const float s1 = ev[0], s2 = s1 + ev[1], s3 = s2 + ev[2], s4 = s3 + ev[3];
+      const float incl = scan64(s4);
+      float excl = __shfl_up(incl, 1, WAVE);
+      if (lane == 0) excl = 0.f;
+      const float base = cum + excl;
+      // this lane's first element that reaches the target, and its last one with any weight
+      int mine_pick = -1, mine_last = -1;
+      const float sums[4] = {s1, s2, s3, s4};
+#pragma unroll
+      for (int c = 3; c >= 0; --c)
+        if (ev[c] > 0.f) {
+          if (mine_last < 0) mine_last = i0 + c;
+          if (base + sums[c] >= target) mine_pick = i0 + c;
+        }
+      const unsigned long long hit = __ballot(mine_pick >= 0);
+      const unsigned long long any = __ballot(mine_last >= 0);
+      if (any) last = __shfl(mine_last, 63 - __clzll(any), WAVE);
+      if (hit) pick = __shfl(mine_pick, __ffsll((long long)hit) - 1, WAVE);
+      cum += __shfl(incl, WAVE - 1, WAVE);
+    }
+    if (lane == 0) chosen = pick >= 0 ? pick : last;
   }
   __syncthreads();
-  if (threadIdx.x == 0) out[row] = chosen >= 0 ? chosen : (top.i < 0 ? 0 : top.i);
+  if (threadIdx.x == 0) finish(chosen >= 0 ? chosen : (top.i < 0 ? 0 : top.i));
 }
 
 // partial: scratch of n_rows * 64 pairs (float, int32), 8 bytes each.
@@ -249,18 +475,21 @@ extern "C" const char* dlgo_argmax(const float* logits, int ld, int n_rows, int 
   return nullptr;
 }
 
-// work and e: [n_rows, V] float32 scratch.  recent: [n_rows, n_recent] token ids, -1 where empty.
+// work and e: [n_rows, V] float32 scratch.  recent: a table of token ids with n_recent columns.  Without counts, row r of
+// it holds row r's recent tokens, -1 where empty.  With recent_rows and counts, row recent_rows[r] of it is a ring of the
+// last tokens chosen for that key, counts[key] the number chosen so far; the kernel adds the token it chooses.
 extern "C" const char* dlgo_sample(const float* logits, int ld, int n_rows, int V, float* work, float* e,
                                    const float* temperature, const int32_t* top_k, const float* top_p, const float* min_p,
-                                   const float* penalty, const int32_t* recent, int n_recent, const float* uniform,
-                                   int32_t* out, hipStream_t stream) {
+                                   const float* penalty, int32_t* recent, int n_recent, const int32_t* recent_rows,
+                                   int32_t* counts, const float* uniform, int32_t* out, hipStream_t stream) {
   DLGO_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "sample: bad sizes rows=%d V=%d ld=%d", n_rows, V, ld);
   DLGO_REQUIRE(n_recent >= 0 && n_recent <= SAMP_THREADS, "sample: at most %d recent tokens, got %d", SAMP_THREADS, n_recent);
   DLGO_REQUIRE(work && e && temperature && top_k && top_p && min_p && penalty && uniform && out, "sample: missing argument");
   DLGO_REQUIRE(n_recent == 0 || recent, "sample: recent tokens missing");
+  DLGO_REQUIRE((recent_rows == nullptr) == (counts == nullptr), "sample: a ring of recent tokens needs both its rows and its counts");
   if (n_rows == 0) return nullptr;
   hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMP_THREADS), 0, stream, logits, ld, V, work, e, temperature, top_k, top_p,
-                     min_p, penalty, recent, n_recent, uniform, out);
+                     min_p, penalty, recent, n_recent, recent_rows, counts, uniform, out);
   DLGO_LAUNCH_CHECK("sample");
   return nullptr;
 }

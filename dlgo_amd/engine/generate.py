@@ -110,8 +110,9 @@ def _decode_ahead(engine, sampler, live, logits, prompts, results, stats, on_tok
         if len(keep) != len(live):
             logits = logits[keep]
             live = [live[r] for r in keep]
+        keyed = {"keys": [l.slot for l in live]} if getattr(sampler, "keeps_recent", False) else {}
         tok_dev, wait = sampler.choose_async(logits, [l.config.sampler for l in live],
-                                             [uniform(l.seed, l.index, len(l.tokens)) for l in live], None)
+                                             [uniform(l.seed, l.index, len(l.tokens)) for l in live], None, **keyed)
         # queue the next step for every sequence that wants another token after this one, before knowing the ids
         fed = [row for row, l in enumerate(live) if len(l.tokens) + 1 < l.config.max_tokens]
         next_logits = None
@@ -186,8 +187,11 @@ def generate(engine, sampler, prompts: Sequence[Sequence[int]], configs: Sequenc
             stats.prefill_ms += (t1 - t0) * 1000.0
             stats.prompt_tokens += sum(len(prompts[l.index]) for l in live)
             stats.steps += 1
+            keeps = getattr(sampler, "keeps_recent", False)      # then the penalty's tokens need not come back first
             ahead = (hasattr(engine, "decode") and hasattr(sampler, "choose_async")
-                     and not sampler.needs_recent([l.config.sampler for l in live]))
+                     and (keeps or not sampler.needs_recent([l.config.sampler for l in live])))
+            if ahead and keeps:
+                sampler.start([l.slot for l in live])
             if ahead:
                 _decode_ahead(engine, sampler, live, logits, prompts, results, stats, on_token)
                 live = []

@@ -416,7 +416,11 @@ def argmax(logits: torch.Tensor, out: torch.Tensor, scratch: Optional[torch.Tens
 
 def sample(logits: torch.Tensor, work: torch.Tensor, e: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
            top_p: torch.Tensor, min_p: torch.Tensor, penalty: torch.Tensor, recent: Optional[torch.Tensor],
-           uniform: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+           uniform: torch.Tensor, out: torch.Tensor, recent_rows: Optional[torch.Tensor] = None,
+           counts: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token per row of float32 logits, each row with its own options.  recent [rows, w]: the row's recent tokens
+    (-1 where empty) for the repetition penalty.  With recent_rows [rows] and counts: recent is a table of rings, row
+    recent_rows[r] of it belongs to row r and holds its last min(counts, w) tokens; the chosen token is added to it."""
     _need(logits, "logits", torch.float32, 2)
     n, v = logits.shape
     for name, t, dt in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
@@ -431,12 +435,19 @@ def sample(logits: torch.Tensor, work: torch.Tensor, e: torch.Tensor, temperatur
         if t.shape[0] < n or t.shape[1] != v or not t.is_contiguous():
             raise KernelError(f"sample: scratch {name} {tuple(t.shape)} too small for {(n, v)}")
     n_recent = 0
+    if (recent_rows is None) != (counts is None):
+        raise KernelError("sample: a table of rings needs both recent_rows and counts")
     if recent is not None:
         _need(recent, "recent tokens", torch.int32, 2)
-        if recent.shape[0] != n or not recent.is_contiguous():
+        if not recent.is_contiguous() or (counts is None and recent.shape[0] != n):
             raise KernelError("sample: one row of recent tokens per row of logits")
         n_recent = recent.shape[1]
+    if counts is not None:
+        _need(recent_rows, "rows of the recent tokens", torch.int32, 1)
+        _need(counts, "counts of recent tokens", torch.int32, 1)
+        if recent is None or recent_rows.shape[0] != n or counts.shape[0] != recent.shape[0]:
+            raise KernelError("sample: recent_rows has one entry per row of logits, counts one per row of the table")
     _check(_lib("sampling").dlgo_sample(_ptr(logits), _rows(logits, "logits"), n, v, _ptr(work), _ptr(e), _ptr(temperature),
                                         _ptr(top_k), _ptr(top_p), _ptr(min_p), _ptr(penalty), _ptr(recent), n_recent,
-                                        _ptr(uniform), _ptr(out), _stream()))
+                                        _ptr(recent_rows), _ptr(counts), _ptr(uniform), _ptr(out), _stream()))
     return out

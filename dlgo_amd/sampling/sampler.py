@@ -14,6 +14,10 @@ RECENT = 64   # tokens the repetition penalty looks back on (models/llm/generate
 
 
 class Sampler:
+    #: the tokens a request has been given are also kept on the device (start(), and keys= of the choose calls), so
+    #: that the repetition penalty does not need them back from the host before the next choice
+    keeps_recent = True
+
     def __init__(self, vocab: int, device, max_rows: int = 256):
         self.vocab = vocab
         self.device = torch.device(device)
@@ -23,6 +27,23 @@ class Sampler:
         self._pin_next = 0
         self._work: Optional[torch.Tensor] = None
         self._e: Optional[torch.Tensor] = None
+        self._rings: Optional[torch.Tensor] = None      # [keys, RECENT] last tokens chosen per key
+        self._counts: Optional[torch.Tensor] = None     # [keys] tokens chosen so far per key
+
+    def start(self, keys: Sequence[int]) -> None:
+        """Requests begin under these keys (any small integers that stay with a request, such as its slot): what the
+        device remembers of earlier requests under them is forgotten."""
+        need = max(keys) + 1 if len(keys) else 0
+        if self._counts is None or self._counts.shape[0] < need:
+            size = max(need, 2 * (self._counts.shape[0] if self._counts is not None else 0), self.max_rows)
+            counts = torch.zeros(size, dtype=torch.int32, device=self.device)
+            rings = torch.full((size, RECENT), -1, dtype=torch.int32, device=self.device)
+            if self._counts is not None:
+                counts[:self._counts.shape[0]] = self._counts
+                rings[:self._rings.shape[0]] = self._rings
+            self._counts, self._rings = counts, rings
+        if len(keys):
+            self._counts[torch.as_tensor(list(keys), dtype=torch.long)] = 0
 
     def _grow(self, rows: int) -> None:
         if rows > self._out.shape[0]:
@@ -35,10 +56,11 @@ class Sampler:
         return self.choose_device(logits, configs, uniforms, recent).tolist()
 
     def choose_async(self, logits: torch.Tensor, configs: Sequence[SamplerConfig], uniforms: Sequence[float],
-                     recent: Optional[Sequence[Sequence[int]]] = None):
+                     recent: Optional[Sequence[Sequence[int]]] = None, keys: Optional[Sequence[int]] = None):
         """The ids as a device tensor (valid until the next call) and a function that waits for them and
-        returns them as a host list; work can be queued behind the choice before the ids are awaited."""
-        out = self.choose_device(logits, configs, uniforms, recent)
+        returns them as a host list; work can be queued behind the choice before the ids are awaited.
+        keys (instead of recent): each row's key as given to start(); the recent tokens are the device's own record."""
+        out = self.choose_device(logits, configs, uniforms, recent, keys)
         n = out.shape[0]
         i = self._pin_next
         self._pin_next = (i + 1) % len(self._pinned)
@@ -59,7 +81,7 @@ class Sampler:
         return any(c.repetition_penalty > 1.0 and not c.greedy for c in configs)
 
     def choose_device(self, logits: torch.Tensor, configs: Sequence[SamplerConfig], uniforms: Sequence[float],
-                      recent: Optional[Sequence[Sequence[int]]] = None) -> torch.Tensor:
+                      recent: Optional[Sequence[Sequence[int]]] = None, keys: Optional[Sequence[int]] = None) -> torch.Tensor:
         """logits [rows, vocab] float32 on the device -> int32 ids on the device (overwritten by the next call)."""
         n = logits.shape[0]
         if n != len(configs) or n != len(uniforms):
@@ -74,18 +96,28 @@ class Sampler:
             self._work = torch.empty((rows, self.vocab), dtype=torch.float32, device=self.device)
             self._e = torch.empty((rows, self.vocab), dtype=torch.float32, device=self.device)
         f = np.zeros((5, n), dtype=np.float32)
-        k = np.zeros(n, dtype=np.int32)
+        k = np.zeros((2, n), dtype=np.int32)        # top-k, and the row's key if the device keeps the recent tokens
         for i, c in enumerate(configs):
             f[0, i], f[1, i], f[2, i], f[3, i], f[4, i] = c.temperature, c.top_p, c.min_p, c.repetition_penalty, uniforms[i]
-            k[i] = c.top_k
+            k[0, i] = c.top_k
+        penalised = any(c.repetition_penalty > 1.0 and not c.greedy for c in configs)
+        rings = keys is not None and recent is None
+        if rings:
+            if self._counts is None or max(keys) >= self._counts.shape[0]:
+                raise ValueError("sampler: keys that start() was never given")
+            k[1] = np.asarray(keys, dtype=np.int32)
         fd = torch.from_numpy(f).to(self.device)
         kd = torch.from_numpy(k).to(self.device)
+        if rings:       # every choice is recorded, penalty or not: a later row of the request may have one
+            ops.sample(logits, self._work, self._e, fd[0], kd[0], fd[1], fd[2], fd[3], self._rings, fd[4], out,
+                       recent_rows=kd[1], counts=self._counts)
+            return out
         rec = None
-        if recent is not None and any(c.repetition_penalty > 1.0 and not c.greedy for c in configs):
+        if recent is not None and penalised:
             r = np.full((n, RECENT), -1, dtype=np.int32)
             for i, toks in enumerate(recent):
                 toks = list(toks)[-RECENT:]
                 r[i, :len(toks)] = toks
             rec = torch.from_numpy(r).to(self.device)
-        ops.sample(logits, self._work, self._e, fd[0], kd, fd[1], fd[2], fd[3], rec, fd[4], out)
+        ops.sample(logits, self._work, self._e, fd[0], kd[0], fd[1], fd[2], fd[3], rec, fd[4], out)
         return out

@@ -90,6 +90,17 @@ def test_temperature_sampling_is_reproducible_and_matches_plain(folder_b):
     d1 = llm.generate(prompts, dlgo_amd.with_seed(5), dlgo_amd.with_max_tokens(12))
     d2 = llm.generate(prompts, dlgo_amd.with_seed(5), dlgo_amd.with_max_tokens(12))
     assert [r.tokens for r in d1] == [r.tokens for r in d2]
+    # ... and draws what the plain pipeline draws, the penalty looking back on the tokens generated so far; two
+    # requests at a time, so that the second pair takes over the first pair's slots and must not inherit their tokens
+    small = dlgo_amd.load_llm(folder_b, dtype="float32", max_tokens=1024, max_batch=2)
+    d3 = small.generate(prompts, dlgo_amd.with_seed(5), dlgo_amd.with_max_tokens(12), dlgo_amd.with_ignore_eos())
+    for i, (p, r) in enumerate(zip(prompts, d3)):
+        seq, want = list(p), []
+        for step in range(12):
+            tok = plain.sample_token(plain.forward(cfg, w, seq)[-1], uniform(5, i, step), 0.7, 40, 0.9, 0.0, 1.1, want[-64:])
+            want.append(tok)
+            seq.append(tok)
+        assert r.tokens == want, i
 
 
 def test_long_decoding_and_context_end(folder_a):

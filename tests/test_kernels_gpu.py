@@ -611,6 +611,34 @@ def test_sample_matches_plain(v):
             assert got[i] == want, (c, i)
 
 
+def test_sample_top_k_in_awkward_rows():
+    """Rows that the quick way of top-k cannot take, or only just: many equal values at the cut, a k-th value far below
+    the maximum, a k beyond what it keeps, a row of negative values: the same token as the plain implementation."""
+    import plain_llama as plain
+    g = torch.Generator().manual_seed(5)
+    v = 6000
+    rows = []
+    r = torch.randn(v, generator=g) * 2
+    r[100:1400] = 9.0                         # 1300 equal values at the top: more than the quick way keeps
+    rows.append((r, dict(temp=1.0, top_k=50)))
+    r = torch.randn(v, generator=g) * 0.01 - 40.0
+    r[7] = 30.0                               # everything else far below the maximum
+    rows.append((r, dict(temp=1.0, top_k=5)))
+    r = torch.randn(v, generator=g) * 3
+    rows.append((r, dict(temp=1.5, top_k=2000, top_p=0.95)))          # k beyond the candidates kept
+    r = -torch.rand(v, generator=g) * 5 - 1                           # all negative
+    rows.append((r, dict(temp=0.6, top_k=40, top_p=0.9, min_p=0.05)))
+    r = torch.randn(v, generator=g)
+    r[5::7] = 2.5                             # ties inside the kept set and at its edge
+    rows.append((r, dict(temp=0.9, top_k=300, top_p=0.8)))
+    for logits, c in rows:
+        for u in (0.00137, 0.2031, 0.5531, 0.8973, 0.99951):       # no multiples of 1/1300: the equal values' edges
+            got = _sample(logits[None], c["temp"], c.get("top_k", 0), c.get("top_p", 1.0), c.get("min_p", 0.0), u=u)[0]
+            want = plain.sample_token(logits.double().numpy(), u, c["temp"], c.get("top_k", 0), c.get("top_p", 1.0),
+                                      c.get("min_p", 0.0), 1.0, [])
+            assert got == want, (c, u)
+
+
 def test_sample_reference_behaviour():
     """ops/sampling_test.go: a dominant logit is always drawn (:18-30); temperature 2 halves the logits (:48-57)."""
     logits = torch.zeros(1, 50)
