@@ -64,13 +64,14 @@ __global__ __launch_bounds__(WAVE) void attn_rows_kernel(const T* __restrict__ q
                                                          const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ slots,
                                                          const int32_t* __restrict__ page_table, int max_pages,
                                                          const T* __restrict__ cache, long long page_stride, long long v_off,
-                                                         int group, int window, float scale) {
+                                                         int group, int window, float scale, int n_splits,
+                                                         float* __restrict__ part) {
   constexpr int HD = HEAD_DIM;
   constexpr int E = Vec16<T>::E;
   constexpr int ND = (HD + WAVE - 1) / WAVE;
   __shared__ float qs[HD];
   __shared__ float ps[PAGE];
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int t = blockIdx.x, h = blockIdx.y, split = blockIdx.z, lane = threadIdx.x;
   const int pos = positions[t];
   const int slot = slots[tok_seq[t]];
   const int kvh = h / group;
@@ -85,7 +86,14 @@ __global__ __launch_bounds__(WAVE) void attn_rows_kernel(const T* __restrict__ q
 #pragma unroll
   for (int i = 0; i < ND; ++i) acc[i] = 0.f;
 
-  for (int pg = lo / PAGE; pg <= pos / PAGE; ++pg) {
+  // with n_splits > 1 the pages of the row are dealt evenly to that many blocks (as attn_decode_kernel deals them), each
+  // of which leaves (values, maximum, sum) in part[((t * heads + h) * n_splits + split) * (HD + 4)], natural exponents
+  const int first_pg = lo / PAGE, last_pg = pos / PAGE;
+  const int span = (last_pg - first_pg + n_splits) / n_splits;
+  const int pg0 = first_pg + split * span;
+  const int pg1 = pg0 + span - 1 < last_pg ? pg0 + span - 1 : last_pg;
+  if (pg0 > pg1) return;
+  for (int pg = pg0; pg <= pg1; ++pg) {
     const int page = page_table[(size_t)slot * max_pages + pg];
     if (page < 0) continue;   // cannot happen for positions the host has reserved
     const T* kpage = cache + (size_t)page * page_stride + (size_t)kvh * PAGE * HD;
@@ -125,6 +133,19 @@ __global__ __launch_bounds__(WAVE) void attn_rows_kernel(const T* __restrict__ q
         acc[i] = a;
       }
     }
+  }
+  if (n_splits > 1) {
+    float* dst = part + ((size_t)(t * gridDim.y + h) * n_splits + split) * (HD + 4);
+#pragma unroll
+    for (int i = 0; i < ND; ++i) {
+      const int d = lane + i * WAVE;
+      if (d < HD) dst[d] = acc[i];
+    }
+    if (lane == 0) {
+      dst[HD] = m;
+      dst[HD + 1] = l;
+    }
+    return;
   }
   T* orow = out + (size_t)t * ldo + (size_t)h * HD;
   const float inv = 1.0f / l;
@@ -413,6 +434,127 @@ __global__ __launch_bounds__(PF_THREADS* PF_TEAMS) __attribute__((amdgpu_waves_p
     }
 }
 
+// Prefill in float32, for head sizes up to 64: a thread owns a query row (token x head of the group, 128 rows a block),
+// a page of keys and of transposed values sits in LDS, and every product is an FMA on float32 with exact expf; the
+// keys are taken 16 at a time so that the scores stay in registers.  grid and bq as attn_prefill_kernel.
+#if HEAD_DIM <= 64
+#define PF32_THREADS 128
+__global__ __launch_bounds__(PF32_THREADS) void attn_prefill_f32_kernel(
+    const float* __restrict__ q, int ldq, float* __restrict__ out, int ldo, const int32_t* __restrict__ cu_q,
+    const int32_t* __restrict__ start_pos, const int32_t* __restrict__ slots, const int32_t* __restrict__ page_table,
+    int max_pages, const float* __restrict__ cache, long long page_stride, long long v_off, int group, int bq, int window,
+    float scale) {
+  constexpr int HD = HEAD_DIM;
+  constexpr int CH = PAGE * HD / 4;                 // 16-byte chunks of a page of keys (and of values)
+  __shared__ __attribute__((aligned(16))) float ldsK[PAGE * HD];
+  __shared__ __attribute__((aligned(16))) float ldsV[HD * PAGE];
+  const int seq = blockIdx.y, kvh = blockIdx.z;
+  const int q0 = cu_q[seq], qn = cu_q[seq + 1] - q0;
+  const int linear = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const int tile = (linear >> 8) & 1 ? blockIdx.x : gridDim.x - 1 - blockIdx.x;     // as attn_prefill_kernel
+  const int t0 = tile * bq;
+  if (t0 >= qn) return;
+  const int t1 = t0 + bq < qn ? t0 + bq : qn;
+  const int start = start_pos[seq], slot = slots[seq];
+  const int kv_len = start + qn;
+  const int tid = threadIdx.x;
+  const int tok = t0 + tid / group, hig = tid % group;
+  const bool row_ok = tid < bq * group && tok < t1;
+  const int pos = row_ok ? start + tok : -1;
+  const int lo = (row_ok && window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+
+  float qr[HD], o[HD];
+  {
+    const float* qrow = q + (size_t)(q0 + (row_ok ? tok : t0)) * ldq + (size_t)(kvh * group + hig) * HD;
+#pragma unroll
+    for (int d = 0; d < HD; d += 4) {
+      const float4 v = *(const float4*)(qrow + d);
+      qr[d] = v.x * scale;
+      qr[d + 1] = v.y * scale;
+      qr[d + 2] = v.z * scale;
+      qr[d + 3] = v.w * scale;
+    }
+  }
+#pragma unroll
+  for (int d = 0; d < HD; ++d) o[d] = 0.f;
+  float m = -INFINITY, l = 0.f;
+
+  const int b_lo = window > 0 && start + t0 - window + 1 > 0 ? start + t0 - window + 1 : 0;
+  const int pg_lo = b_lo / PAGE, pg_hi = (start + t1 - 1) / PAGE;
+  for (int pg = pg_lo; pg <= pg_hi; ++pg) {
+    const int page = page_table[(size_t)slot * max_pages + pg];
+    const float* kpage = cache + (size_t)(page < 0 ? 0 : page) * page_stride + (size_t)kvh * PAGE * HD;
+    const float* vpage = cache + v_off + (size_t)(page < 0 ? 0 : page) * page_stride + (size_t)kvh * HD * PAGE;
+    const int key0 = pg * PAGE;
+    __syncthreads();                                  // the page before is done with
+    for (int c = tid; c < CH; c += PF32_THREADS) {
+      ((float4*)ldsK)[c] = ((const float4*)kpage)[c];
+      float4 v = ((const float4*)vpage)[c];
+      const int k = key0 + (c % (PAGE / 4)) * 4;      // values of keys beyond the sequence must not reach the sums
+      if (k >= kv_len) v.x = 0.f;
+      if (k + 1 >= kv_len) v.y = 0.f;
+      if (k + 2 >= kv_len) v.z = 0.f;
+      if (k + 3 >= kv_len) v.w = 0.f;
+      ((float4*)ldsV)[c] = v;
+    }
+    __syncthreads();
+    if (!row_ok || key0 > pos || key0 + PAGE - 1 < lo) continue;
+    for (int g = 0; g < PAGE / 16; ++g) {
+      const int kbase = key0 + 16 * g;
+      if (kbase > pos || kbase + 15 < lo) continue;
+      float s[16];
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const float* kr = ldsK + (16 * g + k) * HD;
+        float a = 0.f;
+#pragma unroll
+        for (int d = 0; d < HD; d += 4) {
+          const float4 kv = *(const float4*)(kr + d);
+          a = fmaf(qr[d], kv.x, a);
+          a = fmaf(qr[d + 1], kv.y, a);
+          a = fmaf(qr[d + 2], kv.z, a);
+          a = fmaf(qr[d + 3], kv.w, a);
+        }
+        const int key = kbase + k;
+        s[k] = (key <= pos && key >= lo) ? a : -INFINITY;
+      }
+      float mx = s[0];
+#pragma unroll
+      for (int k = 1; k < 16; ++k) mx = fmaxf(mx, s[k]);
+      const float m_new = fmaxf(m, mx);               // finite: the group holds a key this row sees
+      const float alpha = expf(m - m_new);            // 0 the first time (m = -inf)
+      float rs = 0.f;
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        s[k] = expf(s[k] - m_new);
+        rs += s[k];
+      }
+      l = l * alpha + rs;
+      m = m_new;
+#pragma unroll
+      for (int d = 0; d < HD; ++d) {
+        const float* vr = ldsV + d * PAGE + 16 * g;
+        float a = o[d] * alpha;
+#pragma unroll
+        for (int k = 0; k < 16; k += 4) {
+          const float4 vv = *(const float4*)(vr + k);
+          a = fmaf(s[k], vv.x, a);
+          a = fmaf(s[k + 1], vv.y, a);
+          a = fmaf(s[k + 2], vv.z, a);
+          a = fmaf(s[k + 3], vv.w, a);
+        }
+        o[d] = a;
+      }
+    }
+  }
+  if (!row_ok) return;
+  const float inv = 1.0f / l;
+  float* orow = out + (size_t)(q0 + tok) * ldo + (size_t)(kvh * group + hig) * HD;
+#pragma unroll
+  for (int d = 0; d < HD; d += 4) *(float4*)(orow + d) = make_float4(o[d] * inv, o[d + 1] * inv, o[d + 2] * inv, o[d + 3] * inv);
+}
+#endif
+
 // Rotation of 8 consecutive elements d0..d0+7 of one head vector (bfloat16) at a position whose cos/sin rows are
 // given, as rope_kv.hip does it: split-half pairs (d, d + rot/2) or interleaved pairs (2i, 2i+1); elements from
 // `rot` on are copied.  rot is a multiple of 16, so the 8 elements lie in one half.
@@ -684,7 +826,9 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_kernel(
 // one element of the head (and every lane the same maxima and sums).  Eight splits at a time, their loads issued before
 // the token's position is known: which of them count is decided afterwards, so that the position and the partials
 // cost one trip to memory, not three.
-__global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, int ldo,
+// NATURAL: the partials' maxima are natural exponents and expf is used (the float32 kernels'), else base-2 ones.
+template <typename TO, bool NATURAL>
+__global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restrict__ part, TO* __restrict__ out, int ldo,
                                                             const int32_t* __restrict__ positions, int n_heads,
                                                             int n_splits, int window) {
   constexpr int HD = HEAD_DIM;
@@ -717,14 +861,14 @@ __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restr
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       if (c0 + i <= s1) M_new = fmaxf(M_new, ms[i]);
-    const float keep = fast_exp2(M - M_new);       // 0 at the first round (M = -inf, M_new finite: every split given pages holds a key)
+    const float keep = NATURAL ? expf(M - M_new) : fast_exp2(M - M_new);       // 0 at the first round (M = -inf, M_new finite: every split given pages holds a key)
     L *= keep;
 #pragma unroll
     for (int e = 0; e < ND; ++e) acc[e] *= keep;
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       if (c0 + i <= s1) {
-        const float w = fast_exp2(ms[i] - M_new);
+        const float w = NATURAL ? expf(ms[i] - M_new) : fast_exp2(ms[i] - M_new);
         L = fmaf(w, ls[i], L);
 #pragma unroll
         for (int e = 0; e < ND; ++e) acc[e] = fmaf(w, v[i][e], acc[e]);
@@ -734,7 +878,7 @@ __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restr
   const float inv = 1.0f / L;
 #pragma unroll
   for (int e = 0; e < ND; ++e)
-    if (e * WAVE + lane < HD) out[(size_t)seq * ldo + (size_t)head * HD + e * WAVE + lane] = f32_to_bf16(acc[e] * inv);
+    if (e * WAVE + lane < HD) Elem<TO>::store(out + (size_t)seq * ldo + (size_t)head * HD + e * WAVE + lane, acc[e] * inv);
 }
 
 extern "C" int dlgo_attention_head_dim() { return HEAD_DIM; }
@@ -743,26 +887,40 @@ extern "C" int dlgo_attention_head_dim() { return HEAD_DIM; }
 extern "C" const char* dlgo_attention_rows(const void* q, int ldq, void* out, int ldo, int dtype, int n_tokens, int n_heads,
                                            int n_kv, int head_dim, const int32_t* positions, const int32_t* tok_seq,
                                            const int32_t* slots, const int32_t* page_table, int max_pages, const void* cache,
-                                           long long page_stride, long long v_off, int window, float scale,
-                                           hipStream_t stream) {
+                                           long long page_stride, long long v_off, int window, float scale, int n_splits,
+                                           float* part, long long part_elems, hipStream_t stream) {
   DLGO_REQUIRE(head_dim == HEAD_DIM, "attention: this library is built for head size %d, got %d", HEAD_DIM, head_dim);
   DLGO_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention: bad head counts H=%d KV=%d", n_heads, n_kv);
+  DLGO_REQUIRE(n_splits >= 1 && n_splits <= 65535, "attention: bad number of splits %d", n_splits);
+  DLGO_REQUIRE(n_splits == 1 || (part && part_elems >= (long long)n_tokens * n_heads * n_splits * (HEAD_DIM + 4)),
+               "attention: scratch for partial results too small");
   DLGO_REQUIRE(ldq >= n_heads * head_dim && ldo >= n_heads * head_dim, "attention: row strides too short");
   DLGO_REQUIRE(window >= 0 && max_pages > 0, "attention: bad window or page table width");
   const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
   DLGO_REQUIRE(((uintptr_t)cache & 15) == 0 && page_stride % epc == 0 && v_off % epc == 0, "attention: cache pages must be 16-byte aligned");
   if (n_tokens == 0) return nullptr;
-  dim3 grid(n_tokens, n_heads);
+  dim3 grid(n_tokens, n_heads, n_splits);
   const int group = n_heads / n_kv;
   if (dtype == DLGO_DTYPE_F32)
     hipLaunchKernelGGL(attn_rows_kernel<float>, grid, dim3(WAVE), 0, stream, (const float*)q, ldq, (float*)out, ldo, positions,
-                       tok_seq, slots, page_table, max_pages, (const float*)cache, page_stride, v_off, group, window, scale);
+                       tok_seq, slots, page_table, max_pages, (const float*)cache, page_stride, v_off, group, window, scale,
+                       n_splits, part);
   else if (dtype == DLGO_DTYPE_BF16)
     hipLaunchKernelGGL(attn_rows_kernel<bf16_t>, grid, dim3(WAVE), 0, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo, positions,
-                       tok_seq, slots, page_table, max_pages, (const bf16_t*)cache, page_stride, v_off, group, window, scale);
+                       tok_seq, slots, page_table, max_pages, (const bf16_t*)cache, page_stride, v_off, group, window, scale,
+                       n_splits, part);
   else
     DLGO_FAIL("attention: unknown dtype code %d", dtype);
   DLGO_LAUNCH_CHECK("attention_rows");
+  if (n_splits > 1) {     // the rows are the "sequences" of the combine: one position each
+    if (dtype == DLGO_DTYPE_F32)
+      hipLaunchKernelGGL((attn_combine_kernel<float, true>), dim3(n_tokens, n_heads), dim3(WAVE), 0, stream, part, (float*)out, ldo,
+                         positions, n_heads, n_splits, window);
+    else
+      hipLaunchKernelGGL((attn_combine_kernel<bf16_t, true>), dim3(n_tokens, n_heads), dim3(WAVE), 0, stream, part, (bf16_t*)out, ldo,
+                         positions, n_heads, n_splits, window);
+    DLGO_LAUNCH_CHECK("attention_combine");
+  }
   return nullptr;
 }
 
@@ -792,6 +950,33 @@ extern "C" const char* dlgo_attention_prefill(const void* q, int ldq, void* out,
                      scale * LOG2E);
   DLGO_LAUNCH_CHECK("attention_prefill");
   return nullptr;
+}
+
+// float32, every sequence's rows of this step, head sizes up to 64: arguments as dlgo_attention_prefill.
+extern "C" const char* dlgo_attention_prefill_f32(const void* q, int ldq, void* out, int ldo, int n_seq, int max_q_len, int n_heads,
+                                                  int n_kv, int head_dim, const int32_t* cu_q, const int32_t* start_pos,
+                                                  const int32_t* slots, const int32_t* page_table, int max_pages,
+                                                  const void* cache, long long page_stride, long long v_off, int window,
+                                                  float scale, hipStream_t stream) {
+  DLGO_REQUIRE(head_dim == HEAD_DIM, "attention: this library is built for head size %d, got %d", HEAD_DIM, head_dim);
+#if HEAD_DIM <= 64
+  DLGO_REQUIRE(n_seq >= 0 && max_q_len >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention: bad sizes");
+  const int group = n_heads / n_kv;
+  DLGO_REQUIRE(group <= PF32_THREADS, "attention: the float32 tiled kernel takes up to %d query heads per kv head, got %d", PF32_THREADS, group);
+  DLGO_REQUIRE(ldq >= n_heads * head_dim && ldo >= n_heads * head_dim && ldq % 4 == 0 && ldo % 4 == 0, "attention: row strides");
+  DLGO_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)out & 15) == 0 && ((uintptr_t)cache & 15) == 0 && page_stride % 4 == 0 && v_off % 4 == 0,
+               "attention: operands must be 16-byte aligned");
+  DLGO_REQUIRE(window >= 0 && max_pages > 0, "attention: bad window or page table width");
+  if (n_seq == 0 || max_q_len == 0) return nullptr;
+  const int bq = PF32_THREADS / group;
+  dim3 grid((max_q_len + bq - 1) / bq, n_seq, n_kv);
+  hipLaunchKernelGGL(attn_prefill_f32_kernel, grid, dim3(PF32_THREADS), 0, stream, (const float*)q, ldq, (float*)out, ldo, cu_q,
+                     start_pos, slots, page_table, max_pages, (const float*)cache, page_stride, v_off, group, bq, window, scale);
+  DLGO_LAUNCH_CHECK("attention_prefill_f32");
+  return nullptr;
+#else
+  DLGO_FAIL("attention: the float32 tiled kernel takes head sizes up to 64, this library is built for %d", HEAD_DIM);
+#endif
 }
 
 // bfloat16, one row per sequence.  With cos_t/sin_t ([table_rows, rot/2]) the rows q are unrotated and are rotated
@@ -872,8 +1057,8 @@ extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, 
 #undef DECODE_GO
   DLGO_LAUNCH_CHECK("attention_decode");
   if (n_splits > 1) {
-    hipLaunchKernelGGL(attn_combine_kernel, dim3(n_seq, n_heads), dim3(WAVE), 0, stream, part, (bf16_t*)out, ldo, positions, n_heads,
-                       n_splits, window);
+    hipLaunchKernelGGL((attn_combine_kernel<bf16_t, false>), dim3(n_seq, n_heads), dim3(WAVE), 0, stream, part, (bf16_t*)out, ldo,
+                       positions, n_heads, n_splits, window);
     DLGO_LAUNCH_CHECK("attention_combine");
   }
   return nullptr;

@@ -80,7 +80,7 @@ def _lib(module: str, defines=()):
     if lib is None:
         lib = build.load(module, defines)
         for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_accum_norm", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_attention_rows",
-                     "dlgo_attention_prefill", "dlgo_attention_decode", "dlgo_argmax", "dlgo_sample"):
+                     "dlgo_attention_prefill", "dlgo_attention_prefill_f32", "dlgo_attention_decode", "dlgo_argmax", "dlgo_sample"):
             if hasattr(lib, name):
                 getattr(lib, name).restype = ctypes.c_char_p
         _libs[key] = lib
@@ -272,8 +272,9 @@ def rope_kv(qkv: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, rot: int,
 def attention_rows(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,
                    positions: torch.Tensor, tok_seq: torch.Tensor, slots: torch.Tensor, page_table: torch.Tensor,
                    cache: torch.Tensor, page_stride: int, v_off: int, window: int = 0,
-                   scale: Optional[float] = None) -> torch.Tensor:
-    """One wave per (row, head): the general kernel, every dtype, every step shape."""
+                   scale: Optional[float] = None, n_splits: int = 1, scratch=None) -> torch.Tensor:
+    """One wave per (row, head): the general kernel, every dtype, every step shape.  n_splits > 1 deals each row's
+    pages to that many waves, whose partial results (in scratch(n): float32, n elements) a second kernel merges."""
     _need(q, "query rows", dims=2)
     _need(out, "attention output", q.dtype, 2)
     for name, v in (("positions", positions), ("token->sequence", tok_seq), ("slots", slots)):
@@ -286,11 +287,17 @@ def attention_rows(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, 
     if scale is None:
         scale = 1.0 / math.sqrt(head_dim)
     lib = _lib("attention", (("HEAD_DIM", head_dim),))
+    part = None
+    if n_splits > 1:
+        need = t * n_heads * n_splits * (head_dim + 4)
+        part = scratch(need) if scratch is not None else torch.empty(need, dtype=torch.float32, device=q.device)
+        _need(part, "attention scratch", torch.float32, 1)
     _check(lib.dlgo_attention_rows(_ptr(q), _rows(q, "query rows"), _ptr(out), _rows(out, "attention output"),
                                    dtype_code(q.dtype), t, n_heads, n_kv, head_dim, _ptr(positions), _ptr(tok_seq),
                                    _ptr(slots), _ptr(page_table), page_table.shape[1], _ptr(cache),
                                    ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(window),
-                                   ctypes.c_float(scale), _stream()))
+                                   ctypes.c_float(scale), int(n_splits), _ptr(part),
+                                   ctypes.c_longlong(part.numel() if part is not None else 0), _stream()))
     return out
 
 
@@ -325,20 +332,27 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
     max_q = int(max(q_lens)) if n_seq else 0
     group = n_heads // n_kv
     fast_ok = q.dtype == torch.bfloat16 and head_dim <= 256 and group <= 128
+    tiled_f32 = q.dtype == torch.float32 and head_dim <= 64 and group <= 128       # prompts in float32: a kernel of their own
     if kernel == "auto":
-        kernel = "rows" if not fast_ok else ("split" if max_q == 1 else "tiled")
+        kernel = ("tiled" if tiled_f32 and max_q > 1 else "rows") if not fast_ok else ("split" if max_q == 1 else "tiled")
     if (rotation is not None or new_kv) and not (kernel == "split" and fast_ok and max_q == 1):
         raise KernelError("attention: only the split kernel rotates and stores by itself")
     if kernel == "rows" or n_seq == 0:
+        # a few rows with long histories (a decode step off the fast kernels): each row's pages go to several waves
+        n_splits = 1
+        if max_q == 1 and n_seq > 0:
+            pages = max_pages_used if max_pages_used is not None else (int(max(start_pos)) + PAGE) // PAGE
+            n_splits = max(1, min(pages // 2, 2048 // max(1, n_seq * n_heads)))
         return attention_rows(q, out, n_heads, n_kv, head_dim, positions, tok_seq, slots, page_table, cache, page_stride,
-                              v_off, window, scale)
-    if not fast_ok:
-        raise KernelError("attention: the tiled and split kernels take bfloat16, head sizes up to 256 and up to 128 heads per kv head")
-    _need(q, "query rows", torch.bfloat16, 2)
-    _need(out, "attention output", torch.bfloat16, 2)
+                              v_off, window, scale, n_splits, scratch)
+    if not fast_ok and not (tiled_f32 and kernel == "tiled"):
+        raise KernelError("attention: the tiled and split kernels take bfloat16, head sizes up to 256 and up to 128 heads per kv head "
+                          "(the tiled one also float32 with head sizes up to 64)")
+    _need(q, "query rows", q.dtype, 2)
+    _need(out, "attention output", q.dtype, 2)
     _need(slots, "slots", torch.int32, 1)
     _need(page_table, "page table", torch.int32, 2)
-    _need(cache, "cache", torch.bfloat16)
+    _need(cache, "cache", q.dtype)
     if slots.shape[0] != n_seq or out.shape[0] != q.shape[0] or q.shape[0] != int(sum(q_lens)) or not page_table.is_contiguous():
         raise KernelError("attention: rows, sequences and slots do not match")
     if scale is None:
@@ -387,7 +401,8 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
     _need(start_pos_dev, "start positions", torch.int32, 1)
     if cu_q.shape[0] != n_seq + 1 or start_pos_dev.shape[0] != n_seq:
         raise KernelError("attention: row offsets and start positions do not match the sequences")
-    _check(lib.dlgo_attention_prefill(_ptr(q), _rows(q, "query rows"), _ptr(out), _rows(out, "attention output"), n_seq, max_q,
+    entry = lib.dlgo_attention_prefill_f32 if q.dtype == torch.float32 else lib.dlgo_attention_prefill
+    _check(entry(_ptr(q), _rows(q, "query rows"), _ptr(out), _rows(out, "attention output"), n_seq, max_q,
                                       n_heads, n_kv, head_dim, _ptr(cu_q), _ptr(start_pos_dev), _ptr(slots), _ptr(page_table),
                                       page_table.shape[1], _ptr(cache), ctypes.c_longlong(page_stride),
                                       ctypes.c_longlong(v_off), int(window), ctypes.c_float(scale), _stream()))
