@@ -107,10 +107,40 @@ __global__ __launch_bounds__(256) void rope_kv_pieces_kernel(T* __restrict__ qkv
                                                              const int32_t* __restrict__ slots,
                                                              const int32_t* __restrict__ page_table, int max_pages,
                                                              T* __restrict__ cache, long long page_stride, long long v_off,
-                                                             int write_kv) {
+                                                             int write_kv, int piece_blocks) {
   constexpr int E = Piece<T>::E;
+  if ((int)blockIdx.x >= piece_blocks) {
+    // The values.  A page keeps them transposed ([head size][token]), so a thread that stored its own piece would write
+    // single elements a page row apart.  Instead a block takes 64 consecutive rows of the step, one kv head and up to 64
+    // of its dimensions, turns the tile through LDS, and stores with its lanes along the tokens: where the rows are
+    // consecutive tokens of a sequence, a wave writes a run of a page row at a time.
+    __shared__ T tile[64][66];
+    const int per_tok_tile = (hd + 63) / 64;
+    const int b = blockIdx.x - piece_blocks;
+    const int dpart = b % per_tok_tile, kvh = (b / per_tok_tile) % n_kv, t0 = (b / per_tok_tile / n_kv) * 64;
+    const int dbase = dpart * 64, db = hd - dbase < 64 ? hd - dbase : 64;
+    const int ppr = db / E;                                  // pieces per row of the tile
+    for (int c = threadIdx.x; c < 64 * ppr; c += 256) {
+      const int tk = c / ppr, pc = c % ppr;
+      if (t0 + tk < n_tokens) {
+        float x[E];
+        Piece<T>::load(qkv + (size_t)(t0 + tk) * ld + (size_t)(n_heads + n_kv + kvh) * hd + dbase + pc * E, x);
+#pragma unroll
+        for (int e = 0; e < E; ++e) Elem<T>::store(&tile[tk][pc * E + e], x[e]);
+      }
+    }
+    __syncthreads();
+    const int tk = threadIdx.x & 63, w = threadIdx.x >> 6;
+    if (t0 + tk >= n_tokens) return;
+    const int t = t0 + tk, pos = positions[t];
+    const int page = page_table[(size_t)slots[tok_seq[t]] * max_pages + pos / PAGE];
+    if (page < 0) return;
+    T* vcol = cache + v_off + (size_t)page * page_stride + ((size_t)kvh * hd + dbase) * PAGE + pos % PAGE;
+    for (int d = w; d < db; d += 4) vcol[(size_t)d * PAGE] = tile[tk][d];
+    return;
+  }
   const int per_head = hd / E;
-  const int heads = n_heads + (write_kv ? 2 * n_kv : 0);
+  const int heads = n_heads + (write_kv ? n_kv : 0);       // queries and keys; the values have blocks of their own
   const int per_token = heads * per_head;
   const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (long long)n_tokens * per_token) return;
@@ -124,22 +154,14 @@ __global__ __launch_bounds__(256) void rope_kv_pieces_kernel(T* __restrict__ qkv
   if (rotates && !interleaved && d0 >= half) return;   // done by the thread of the partner piece
   // where the (rotated) pieces go
   T* dst = src;            // queries: in place
-  T* vcol = nullptr;       // values: a column of the transposed page
   if (!is_q) {
     const int slot = slots[tok_seq[t]];
     const int page = page_table[(size_t)slot * max_pages + pos / PAGE];
     if (page < 0) return;
-    const int in_page = pos % PAGE;
-    if (is_k) dst = cache + (size_t)page * page_stride + ((size_t)(head - n_heads) * PAGE + in_page) * hd;
-    else vcol = cache + v_off + (size_t)page * page_stride + (size_t)(head - n_heads - n_kv) * hd * PAGE + in_page;
+    dst = cache + (size_t)page * page_stride + ((size_t)(head - n_heads) * PAGE + pos % PAGE) * hd;
   }
   float x[E];
   Piece<T>::load(src + d0, x);
-  if (vcol) {
-#pragma unroll
-    for (int e = 0; e < E; ++e) Elem<T>::store(vcol + (size_t)(d0 + e) * PAGE, x[e]);
-    return;
-  }
   if (!rotates) {
     if (!is_q) Piece<T>::store(dst + d0, x);      // the part of a key beyond the rotated width is copied
     return;
@@ -186,16 +208,19 @@ extern "C" const char* dlgo_rope_kv(void* qkv, int dtype, int n_tokens, int ld, 
   const bool pieces = hd % epc == 0 && rot % (2 * epc) == 0 && ld % epc == 0 && ((uintptr_t)qkv & 15) == 0 &&
                       (!write_kv || (((uintptr_t)cache & 15) == 0 && page_stride % epc == 0 && v_off % epc == 0));
   if (pieces) {
-    const long long items = (long long)n_tokens * (n_heads + (write_kv ? 2 * n_kv : 0)) * (hd / epc);
-    dim3 g((unsigned)((items + 255) / 256));
+    const long long items = (long long)n_tokens * (n_heads + (write_kv ? n_kv : 0)) * (hd / epc);
+    const long long piece_blocks = (items + 255) / 256;
+    const long long value_blocks = write_kv ? (long long)((n_tokens + 63) / 64) * n_kv * ((hd + 63) / 64) : 0;
+    DLGO_REQUIRE(piece_blocks + value_blocks < (1ll << 31), "rope_kv: too many rows at once");
+    dim3 g((unsigned)(piece_blocks + value_blocks));
     if (dtype == DLGO_DTYPE_F32)
       hipLaunchKernelGGL(rope_kv_pieces_kernel<float>, g, dim3(256), 0, stream, (float*)qkv, ld, n_tokens, n_heads, n_kv, hd, rot,
                          interleaved, cos_t, sin_t, positions, tok_seq, slots, page_table, max_pages, (float*)cache, page_stride,
-                         v_off, write_kv);
+                         v_off, write_kv, (int)piece_blocks);
     else if (dtype == DLGO_DTYPE_BF16)
       hipLaunchKernelGGL(rope_kv_pieces_kernel<bf16_t>, g, dim3(256), 0, stream, (bf16_t*)qkv, ld, n_tokens, n_heads, n_kv, hd, rot,
                          interleaved, cos_t, sin_t, positions, tok_seq, slots, page_table, max_pages, (bf16_t*)cache, page_stride,
-                         v_off, write_kv);
+                         v_off, write_kv, (int)piece_blocks);
     else
       DLGO_FAIL("rope_kv: unknown dtype code %d", dtype);
     DLGO_LAUNCH_CHECK("rope_kv");
