@@ -353,7 +353,7 @@ class Engine:
             ctx.is_decode = True
             if self.use_graphs:
                 ctx.max_pages_used = self.cache.max_pages_per_seq     # the recorded launch must cover any later length
-            x = self.model.hidden(ctx, ctx.token_ids)
+            x = self.model.hidden(ctx, ctx.token_ids, all_rows_wanted=True)
             self.model.logits(ctx, x, None, logits)
             # the second time a batch size is seen it is worth capturing
             self._graph_seen[b] = self._graph_seen.get(b, 0) + 1
@@ -376,7 +376,7 @@ class Engine:
         gc.disable()
         try:
             with torch.cuda.graph(graph):
-                x = self.model.hidden(ctx, ctx.token_ids)
+                x = self.model.hidden(ctx, ctx.token_ids, all_rows_wanted=True)
                 self.model.logits(ctx, x, None, logits)
         finally:
             if was_enabled:

@@ -94,7 +94,10 @@ class DecoderModel:
             self.position.prepare(max_positions, device)
 
     # -- the forward pass over the rows of a step -------------------------------
-    def hidden(self, ctx, token_ids: torch.Tensor) -> torch.Tensor:
+    def hidden(self, ctx, token_ids: torch.Tensor, all_rows_wanted: bool = False) -> torch.Tensor:
+        """The residual rows after the last block.  all_rows_wanted: logits() will be asked for every row, so the last
+        block may leave the final norm of its rows too (kept in ctx.final_normed for logits())."""
+        ctx.final_normed = None
         x = ctx.buffer("model.residual", (token_ids.shape[0], self.width), torch.float32)
         self.embedding(token_ids, x)
         if self.position is not None:
@@ -107,16 +110,23 @@ class DecoderModel:
                 block.forward(x, ctx, self.run_unit[i], self.run_owns[i])
                 normed = None
                 continue
-            nxt = self.layers[self.order[i + 1].layer][1] if i + 1 < len(self.order) else None
+            last = i + 1 == len(self.order)
+            nxt = None if last else self.layers[self.order[i + 1].layer][1]
             then = None
             if nxt is not None and nxt.takes_normed:
                 then = (nxt.entry_norm, ctx.buffer(f"model.normed.{i & 1}", tuple(x.shape), ctx.dtype))
+            elif last and all_rows_wanted:
+                then = (self.final_norm, ctx.buffer(f"model.normed.{i & 1}", tuple(x.shape), ctx.dtype))
             left = block.forward(x, ctx, self.run_unit[i], self.run_owns[i], normed=normed, then=then)
             normed = then[1] if left else None
+            if last and left:
+                ctx.final_normed = normed
         return x
 
     def logits(self, ctx, x: torch.Tensor, rows: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
         """Final norm and output head on the wanted rows of x (all rows if `rows` is None)."""
+        if rows is None and getattr(ctx, "final_normed", None) is not None:
+            return self.head(ctx.final_normed, out)         # the last block left the final norm of every row
         if rows is None and self.head.fuses_norm(self.final_norm, ctx):
             return self.head(x, out, norm=self.final_norm)
         xn = ctx.buffer("model.head_in", (out.shape[0], self.width), ctx.dtype)
