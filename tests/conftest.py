@@ -54,6 +54,15 @@ def tiny_a():
 @pytest.fixture
 def tiny_b():
     return copy.deepcopy(TINY_B)
+# a fourth one: a head size of 80 (above 64, no power of two), one kv head for eight query heads, no scaling of the rotation
+TINY_D = {
+    "architectures": ["LlamaForCausalLM"], "model_type": "llama",
+    "vocab_size": 1000, "hidden_size": 200, "num_hidden_layers": 2, "intermediate_size": 264,
+    "num_attention_heads": 8, "num_key_value_heads": 1, "head_dim": 80,
+    "rms_norm_eps": 1e-4, "rope_theta": 1000000.0, "rope_scaling": None,
+    "max_position_embeddings": 1024, "tie_word_embeddings": False, "initializer_range": 0.04,
+    "hidden_act": "silu", "torch_dtype": "bfloat16", "eos_token_id": [3, 4],
+}
 
 
 @pytest.fixture
