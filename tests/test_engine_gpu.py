@@ -196,6 +196,31 @@ def test_thousands_of_tokens(tmp_path, dtype):
     eng.cache.check_consistent()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_more_sequences_than_a_recorded_step_takes(folders, oracle, dtype):
+    """150 sequences that start together and go on one token at a time: more than the largest batch for which single
+    tokens are recorded and replayed, so the steps take the general way; a few of them checked against the plain one."""
+    from dlgo_amd.engine import Entry
+    n = 150
+    eng = engine_for(folders["A", dtype], dtype, max_tokens=n * 64, max_slots=n, graph_max_batch=64)
+    rng = np.random.default_rng(8)
+    seqs = [rng.integers(0, TINY_A["vocab_size"], size=int(rng.integers(1, 6)) + 4).tolist() for _ in range(n)]
+    slots = eng.open(n)
+    got = [[] for _ in range(n)]
+    out = eng.step([Entry(s, t[:-4], [len(t) - 5]) for s, t in zip(slots, seqs)]).cpu().numpy()
+    for i in range(n):
+        got[i].append(out[i])
+    for k in range(4, 0, -1):
+        out = eng.step([Entry(s, [t[-k]], [0]) for s, t in zip(slots, seqs)]).cpu().numpy()
+        for i in range(n):
+            got[i].append(out[i].copy())
+    for i in (0, 1, 63, 64, 65, 127, 128, 149):
+        want = oracle("A", dtype, seqs[i])[len(seqs[i]) - 5:]
+        assert rel_err(np.stack(got[i]), want) <= TOL[dtype], i
+    eng.close(slots)
+    eng.cache.check_consistent()
+
+
 def test_errors_before_anything_runs(folders):
     from dlgo_amd.engine import EngineError, Entry
     eng = engine_for(folders["A", "float32"], "float32", max_tokens=128)
