@@ -379,29 +379,41 @@ __global__ __launch_bounds__(256) void split_sum_norm_kernel(const float* __rest
   float* y = Y + (size_t)t * ldy;
   float4 row[NCH];
   float ss = 0.f;
+  // the first eight runs of every piece of the row and the old values are all asked for before anything is added:
+  // one trip to memory for the whole row (the last run stands in for those beyond it, and is not added twice)
+  float4 old[NCH], x[NCH][8];
+#pragma unroll
+  for (int c = 0; c < NCH; ++c) {
+    const int n = (c * 256 + threadIdx.x) * 4;
+    const int nn = n < N ? n : 0;
+    old[c] = *(const float4*)(y + nn);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[c][i] = *(const float4*)(p + nn + (size_t)(i < runs ? i : runs - 1) * run_stride);
+  }
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
     const int n = (c * 256 + threadIdx.x) * 4;
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (n < N) {
-      const float4 old = *(const float4*)(y + n);
-      for (int r0 = 0; r0 < runs; r0 += 8) {
-        float4 x[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) x[i] = *(const float4*)(p + n + (size_t)(r0 + i < runs ? r0 + i : runs - 1) * run_stride);
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-          if (r0 + i < runs) {
-            v.x += x[i].x;
-            v.y += x[i].y;
-            v.z += x[i].z;
-            v.w += x[i].w;
-          }
+      for (int i = 0; i < 8; ++i)
+        if (i < runs) {
+          v.x += x[c][i].x;
+          v.y += x[c][i].y;
+          v.z += x[c][i].z;
+          v.w += x[c][i].w;
+        }
+      for (int r = 8; r < runs; ++r) {
+        const float4 more = *(const float4*)(p + n + (size_t)r * run_stride);
+        v.x += more.x;
+        v.y += more.y;
+        v.z += more.z;
+        v.w += more.w;
       }
-      v.x += old.x;
-      v.y += old.y;
-      v.z += old.z;
-      v.w += old.w;
+      v.x += old[c].x;
+      v.y += old[c].y;
+      v.z += old[c].z;
+      v.w += old[c].w;
       *(float4*)(y + n) = v;
       ss += v.x * v.x;
       ss += v.y * v.y;
