@@ -280,10 +280,13 @@ __global__ __launch_bounds__(WN* WT* WAVE) void gemm_direct_kernel(const T* __re
 #pragma unroll
         for (int j = 0; j < NJ; ++j) b[nx][j] = *(const uint4*)(pb + j * 32 * 128 + so);
       }
+      // the reads of the next slab stay in front of this slab's products: they arrive while these run
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < NJ; ++j) Mma<T>::run(a[c][i], b[c][j], acc[i][j]);
+      __builtin_amdgcn_sched_barrier(0);
     }
     stage = stage + 1 == NS ? 0 : stage + 1;
   }
