@@ -2,6 +2,7 @@
 
     python -m dlgo_amd.kernels.probe gemm --n 16384 --k 2048 --t 2048 --epilogue swiglu --kind 20
     python -m dlgo_amd.kernels.probe prefill-attention --tokens 2048 --heads 32 --kv-heads 8 --head-dim 64
+    python -m dlgo_amd.kernels.probe mfma-peak         # MFMAs on registers alone: the rate the chip sustains
 
 Prints the mean wall time of a call, the host's share included (for short kernels that share is most of it).  Under
 `rocprofv3 --pmc ...` or `--kernel-trace --stats` the kernel's own counters and durations are what one reads; this
@@ -63,6 +64,25 @@ def prefill_attention(args) -> None:
           f"{flops / sec / 1e12:.0f} TFLOP/s")
 
 
+def mfma_peak(args) -> None:
+    import ctypes
+
+    from . import build
+    lib = build.load("probe")
+    lib.dlgo_probe_mfma.restype = ctypes.c_char_p
+    out = torch.empty(args.blocks * 256, device="cuda")
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def call():
+        err = lib.dlgo_probe_mfma(ctypes.c_void_p(out.data_ptr()), args.blocks, args.iters, stream)
+        if err:
+            raise RuntimeError(err.decode())
+    sec = _timed(call, args.calls)
+    flops = args.blocks * 4 * args.iters * 16 * 32768.0
+    print(f"MFMA 32x32x16 bf16 on registers alone, {args.blocks} blocks of 4 waves: {sec * 1e3:.2f} ms a call, "
+          f"{flops / sec / 1e12:.0f} TFLOP/s")
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="what", required=True)
@@ -84,6 +104,11 @@ def main() -> int:
     b.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     b.add_argument("--calls", type=int, default=3)
     b.set_defaults(run=prefill_attention)
+    c = sub.add_parser("mfma-peak", help="matrix instructions on registers alone")
+    c.add_argument("--blocks", type=int, default=256 * 8, help="blocks of four waves (256 compute units take 8 each at a time)")
+    c.add_argument("--iters", type=int, default=20000)
+    c.add_argument("--calls", type=int, default=3)
+    c.set_defaults(run=mfma_peak)
     args = ap.parse_args()
     args.run(args)
     return 0
