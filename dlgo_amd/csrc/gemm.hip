@@ -290,8 +290,47 @@ __global__ __launch_bounds__(WN* WT* WAVE) void gemm_direct_kernel(const T* __re
     }
     stage = stage + 1 == NS ? 0 : stage + 1;
   }
-  __syncthreads();      // the stages are free: each wave turns its tiles through a piece of them, as in gemm_kernel
+  __syncthreads();      // the stages are free
 
+  // bfloat16 results leave as whole rows: every wave puts its converted tiles into one [BT][OC] tile in the stages,
+  // then the block stores it in pieces of 16 bytes, a row of the tile after the other (256 bytes in one run instead of
+  // the 32 or 64 that a wave's own tile has per token).
+  constexpr int OC = EPI == EPI_SWIGLU ? BN / 2 : BN;      // columns of Y that the block's tile has
+  constexpr int OROW = OC * 2 + 16;                        // bytes of a row of it in LDS
+  if constexpr (sizeof(T) == 2 && (EPI == EPI_STORE || EPI == EPI_SWIGLU) && BT * OROW <= NS * STAGE) {
+    const int n_out = EPI == EPI_SWIGLU ? N >> 1 : N, c0 = EPI == EPI_SWIGLU ? n0 >> 1 : n0;
+    if ((ldy & 7) == 0 && (n_out & 7) == 0 && ((uintptr_t)Y & 15) == 0) {
+#pragma unroll
+      for (int j = 0; j < NJ; ++j)
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int tl = wt * (BT / WT) + j * 32 + (lane & 31);
+            const int nl = wn * (BN / WN) + i * 32 + 8 * q + 4 * (lane >> 5);     // four consecutive n of that token
+            const float v0 = acc[i][j][4 * q], v1 = acc[i][j][4 * q + 1], v2 = acc[i][j][4 * q + 2], v3 = acc[i][j][4 * q + 3];
+            if (EPI == EPI_SWIGLU) {
+              *(uint32_t*)(lds + tl * OROW + nl) =
+                  (uint32_t)f32_to_bf16(silu_f<T>(v0) * v1) | ((uint32_t)f32_to_bf16(silu_f<T>(v2) * v3) << 16);
+            } else {
+              uint2 p;
+              p.x = (uint32_t)f32_to_bf16(v0) | ((uint32_t)f32_to_bf16(v1) << 16);
+              p.y = (uint32_t)f32_to_bf16(v2) | ((uint32_t)f32_to_bf16(v3) << 16);
+              *(uint2*)(lds + tl * OROW + nl * 2) = p;
+            }
+          }
+      __syncthreads();
+      constexpr int CPR = OC / 8;     // pieces of 16 bytes in a row
+      for (int c = tid; c < BT * CPR; c += NW * WAVE) {
+        const int row = c / CPR, piece = c % CPR;
+        const int t = t0 + row, col = c0 + piece * 8;
+        if (t < Tn && col < n_out) *(uint4*)((T*)Y + (size_t)t * ldy + col) = *(const uint4*)(lds + row * OROW + piece * 16);
+      }
+      return;
+    }
+  }
+
+  // otherwise each wave turns its tiles through a piece of the stages, as in gemm_kernel
   float* turn = (float*)(lds + wave * (32 * GEMM_ROWB));
 #pragma unroll
   for (int j = 0; j < NJ; ++j) {
