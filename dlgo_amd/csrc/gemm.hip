@@ -619,6 +619,29 @@ extern "C" int dlgo_gemm_auto_splits(int dtype, int N, int Tn, int K, int ldw, i
   return auto_splits(N, Tn, K / (int)(128 / elem), part_elems);
 }
 
+// The runs alone: part[r][t][n] = sum over run r of k of X[t, k] W[n, k], r < the returned *runs (planes of Tn * N floats, one
+// after the other).  For a caller whose next kernel adds the runs up as it reads them.
+extern "C" const char* dlgo_gemm_parts(const void* W, const void* X, int dtype, int N, int Tn, int K, int ldw, int ldx, int splits,
+                                       float* part, long long part_elems, int* runs, hipStream_t stream) {
+  DLGO_REQUIRE(N > 0 && Tn >= 0 && K > 0 && runs, "gemm: bad sizes N=%d T=%d K=%d", N, Tn, K);
+  DLGO_REQUIRE(dtype == DLGO_ELEM, "gemm: this library is built for dtype code %d, got %d", DLGO_ELEM, dtype);
+  const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
+  DLGO_REQUIRE(direct_takes(K, ldw, ldx, sizeof(elem_t)), "gemm: a split product needs K %% %d == 0, got K=%d", 8 * epc, K);
+  DLGO_REQUIRE(ldw % epc == 0 && ldx % epc == 0 && ldw >= K && ldx >= K, "gemm: row strides (%d, %d) must be multiples of %d and at least K", ldw, ldx, epc);
+  DLGO_REQUIRE(((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0 && ((uintptr_t)part & 15) == 0, "gemm: W, X and the scratch must be 16-byte aligned");
+  const int nk_all = K / (int)(128 / sizeof(elem_t));
+  DLGO_REQUIRE(splits > 1 && splits <= nk_all, "gemm: %d runs of k with %d tiles", splits, nk_all);
+  DLGO_REQUIRE(part && (long long)splits * Tn * N <= part_elems, "gemm: %d runs of k need %lld floats of scratch, got %lld", splits,
+               (long long)splits * Tn * N, part_elems);
+  const int nk_split = (nk_all + splits - 1) / splits;
+  *runs = (nk_all + nk_split - 1) / nk_split;
+  if (Tn == 0) return nullptr;
+  const char* err = launch_direct<elem_t, 64, 64, 2, 2, 4, EPI_STORE_F32>(W, X, part, N, Tn, K, ldw, ldx, N, stream, splits, (long long)Tn * N);
+  if (err) return err;
+  DLGO_LAUNCH_CHECK("gemm_parts");
+  return nullptr;
+}
+
 // Y += X W^T with k shared out in `splits` runs (> 1), and normed = rmsnorm(Y) * norm_w of the new rows beside it.
 extern "C" const char* dlgo_gemm_accum_norm(const void* W, const void* X, float* Y, int dtype, int N, int Tn, int K, int ldw, int ldx,
                                             int ldy, int splits, float* part, long long part_elems, const float* norm_w, float eps,

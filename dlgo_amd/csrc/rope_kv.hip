@@ -98,6 +98,32 @@ template <> struct Piece<bf16_t> {
   }
 };
 
+// The E elements at column `col` of row t: from the rows themselves, or, where the product that made the rows left the
+// runs of its inner sum unsummed (n_parts planes of float32, `plane` apart, rows of part_ld), their sum in run order.
+template <typename T>
+static __device__ __forceinline__ void load_piece(const T* __restrict__ qkv, int ld, const float* __restrict__ part, int n_parts,
+                                                  long long plane, int part_ld, int t, int col, float* x) {
+  constexpr int E = Piece<T>::E;
+  if (!part) {
+    Piece<T>::load(qkv + (size_t)t * ld + col, x);
+    return;
+  }
+  const float* p = part + (size_t)t * part_ld + col;
+#pragma unroll
+  for (int e = 0; e < E; e += 4) *(float4*)(x + e) = *(const float4*)(p + e);
+  for (int r = 1; r < n_parts; ++r) {
+    p += plane;
+#pragma unroll
+    for (int e = 0; e < E; e += 4) {
+      const float4 v = *(const float4*)(p + e);
+      x[e] += v.x;
+      x[e + 1] += v.y;
+      x[e + 2] += v.z;
+      x[e + 3] += v.w;
+    }
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void rope_kv_pieces_kernel(T* __restrict__ qkv, int ld, int n_tokens, int n_heads, int n_kv, int hd,
                                                              int rot, int interleaved, const float* __restrict__ cos_t,
@@ -107,7 +133,9 @@ __global__ __launch_bounds__(256) void rope_kv_pieces_kernel(T* __restrict__ qkv
                                                              const int32_t* __restrict__ slots,
                                                              const int32_t* __restrict__ page_table, int max_pages,
                                                              T* __restrict__ cache, long long page_stride, long long v_off,
-                                                             int write_kv, int piece_blocks) {
+                                                             int write_kv, int piece_blocks,
+                                                             const float* __restrict__ part, int n_parts, long long plane,
+                                                             int part_ld) {
   constexpr int E = Piece<T>::E;
   if ((int)blockIdx.x >= piece_blocks) {
     // The values.  A page keeps them transposed ([head size][token]), so a thread that stored its own piece would write
@@ -124,7 +152,7 @@ __global__ __launch_bounds__(256) void rope_kv_pieces_kernel(T* __restrict__ qkv
       const int tk = c / ppr, pc = c % ppr;
       if (t0 + tk < n_tokens) {
         float x[E];
-        Piece<T>::load(qkv + (size_t)(t0 + tk) * ld + (size_t)(n_heads + n_kv + kvh) * hd + dbase + pc * E, x);
+        load_piece<T>(qkv, ld, part, n_parts, plane, part_ld, t0 + tk, (n_heads + n_kv + kvh) * hd + dbase + pc * E, x);
 #pragma unroll
         for (int e = 0; e < E; ++e) Elem<T>::store(&tile[tk][pc * E + e], x[e]);
       }
@@ -161,9 +189,9 @@ __global__ __launch_bounds__(256) void rope_kv_pieces_kernel(T* __restrict__ qkv
     dst = cache + (size_t)page * page_stride + ((size_t)(head - n_heads) * PAGE + pos % PAGE) * hd;
   }
   float x[E];
-  Piece<T>::load(src + d0, x);
+  load_piece<T>(qkv, ld, part, n_parts, plane, part_ld, t, head * hd + d0, x);
   if (!rotates) {
-    if (!is_q) Piece<T>::store(dst + d0, x);      // the part of a key beyond the rotated width is copied
+    if (!is_q || part) Piece<T>::store(dst + d0, x);      // the part of a key beyond the rotated width is copied
     return;
   }
   const float* cs = cos_t + (size_t)pos * half;
@@ -180,7 +208,7 @@ __global__ __launch_bounds__(256) void rope_kv_pieces_kernel(T* __restrict__ qkv
   } else {
     // this thread owns the pieces at d0 and d0 + half: both are read before either is written
     float p[E], y0[E], y1[E];
-    Piece<T>::load(src + d0 + half, p);
+    load_piece<T>(qkv, ld, part, n_parts, plane, part_ld, t, head * hd + d0 + half, p);
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       const float c_ = cs[d0 + e], s_ = sn[d0 + e];
@@ -196,7 +224,8 @@ extern "C" const char* dlgo_rope_kv(void* qkv, int dtype, int n_tokens, int ld, 
                                     int interleaved, const float* cos_t, const float* sin_t, int table_rows,
                                     const int32_t* positions, const int32_t* tok_seq, const int32_t* slots,
                                     const int32_t* page_table, int max_pages, void* cache, long long page_stride,
-                                    long long v_off, int write_kv, hipStream_t stream) {
+                                    long long v_off, int write_kv, const float* part, int n_parts, long long plane, int part_ld,
+                                    hipStream_t stream) {
   DLGO_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv >= 0 && hd > 0, "rope_kv: bad sizes");
   DLGO_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv: rotated width %d must be even and at most head_dim %d", rot, hd);
   DLGO_REQUIRE(ld >= (n_heads + 2 * n_kv) * hd, "rope_kv: row stride %d shorter than the heads it holds", ld);
@@ -207,6 +236,11 @@ extern "C" const char* dlgo_rope_kv(void* qkv, int dtype, int n_tokens, int ld, 
   const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
   const bool pieces = hd % epc == 0 && rot % (2 * epc) == 0 && ld % epc == 0 && ((uintptr_t)qkv & 15) == 0 &&
                       (!write_kv || (((uintptr_t)cache & 15) == 0 && page_stride % epc == 0 && v_off % epc == 0));
+  // part: the rows are still the n_parts unsummed runs of the product that makes them (float32 planes of rows of part_ld);
+  // the kernel sums them as it reads, and writes the queries into qkv
+  DLGO_REQUIRE(!part || (pieces && n_parts >= 1 && part_ld % 4 == 0 && part_ld >= (n_heads + (write_kv ? 2 * n_kv : 0)) * hd &&
+                         plane >= (long long)n_tokens * part_ld && plane % 4 == 0 && ((uintptr_t)part & 15) == 0),
+               "rope_kv: unsummed rows need whole 16-byte pieces (head size %d, rotated width %d) and aligned planes", hd, rot);
   if (pieces) {
     const long long items = (long long)n_tokens * (n_heads + (write_kv ? n_kv : 0)) * (hd / epc);
     const long long piece_blocks = (items + 255) / 256;
@@ -216,11 +250,11 @@ extern "C" const char* dlgo_rope_kv(void* qkv, int dtype, int n_tokens, int ld, 
     if (dtype == DLGO_DTYPE_F32)
       hipLaunchKernelGGL(rope_kv_pieces_kernel<float>, g, dim3(256), 0, stream, (float*)qkv, ld, n_tokens, n_heads, n_kv, hd, rot,
                          interleaved, cos_t, sin_t, positions, tok_seq, slots, page_table, max_pages, (float*)cache, page_stride,
-                         v_off, write_kv, (int)piece_blocks);
+                         v_off, write_kv, (int)piece_blocks, part, n_parts, plane, part_ld);
     else if (dtype == DLGO_DTYPE_BF16)
       hipLaunchKernelGGL(rope_kv_pieces_kernel<bf16_t>, g, dim3(256), 0, stream, (bf16_t*)qkv, ld, n_tokens, n_heads, n_kv, hd, rot,
                          interleaved, cos_t, sin_t, positions, tok_seq, slots, page_table, max_pages, (bf16_t*)cache, page_stride,
-                         v_off, write_kv, (int)piece_blocks);
+                         v_off, write_kv, (int)piece_blocks, part, n_parts, plane, part_ld);
     else
       DLGO_FAIL("rope_kv: unknown dtype code %d", dtype);
     DLGO_LAUNCH_CHECK("rope_kv");

@@ -79,7 +79,7 @@ def _lib(module: str, defines=()):
     lib = _libs.get(key)
     if lib is None:
         lib = build.load(module, defines)
-        for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_accum_norm", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_attention_rows",
+        for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_accum_norm", "dlgo_gemm_parts", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_attention_rows",
                      "dlgo_attention_prefill", "dlgo_attention_prefill_f32", "dlgo_attention_decode", "dlgo_argmax", "dlgo_sample"):
             if hasattr(lib, name):
                 getattr(lib, name).restype = ctypes.c_char_p
@@ -166,6 +166,39 @@ def gemm_accum_then_norm(weight: torch.Tensor, x: torch.Tensor, residual: torch.
     return True
 
 
+class UnsummedRows:
+    """The rows x @ weight.T as gemm_runs leaves them: `runs` float32 planes [T, N] one after the other in `scratch`, each
+    the sum over one run of k; the rows themselves are the planes added in order.  A kernel that reads the rows once
+    can do that sum as it reads (rope_kv does) and save the pass that would write them out."""
+    __slots__ = ("scratch", "runs", "rows", "cols")
+
+    def __init__(self, scratch, runs, rows, cols):
+        self.scratch, self.runs, self.rows, self.cols = scratch, runs, rows, cols
+
+
+def gemm_runs(weight: torch.Tensor, x: torch.Tensor, scratch: Optional[torch.Tensor]) -> Optional[UnsummedRows]:
+    """x @ weight.T left as unsummed runs of k in `scratch`, if this product is one whose inner size gemm() would share
+    out over blocks; None, having done nothing, if it is not (the caller then runs gemm())."""
+    _need(weight, "gemm weight", dims=2)
+    _need(x, "gemm input", weight.dtype, 2)
+    n, k = weight.shape
+    t = x.shape[0]
+    if scratch is None or t == 0 or n % 4 or _streams_rows(weight, t, GEMM_AUTO, True, 0):
+        return None
+    _need(scratch, "gemm scratch", torch.float32, 1)
+    if x.shape[1] != k:
+        raise KernelError(f"gemm_runs: x {tuple(x.shape)} does not fit weight {tuple(weight.shape)}")
+    lib = _lib("gemm", (("DLGO_ELEM", dtype_code(weight.dtype)),))
+    ldw, ldx = _rows(weight, "gemm weight"), _rows(x, "gemm input")
+    splits = lib.dlgo_gemm_auto_splits(dtype_code(weight.dtype), n, t, k, ldw, ldx, ctypes.c_longlong(scratch.numel()))
+    if splits <= 1:
+        return None
+    runs = ctypes.c_int(0)
+    _check(lib.dlgo_gemm_parts(_ptr(weight), _ptr(x), dtype_code(weight.dtype), n, t, k, ldw, ldx, splits, _ptr(scratch),
+                               ctypes.c_longlong(scratch.numel()), ctypes.byref(runs), _stream()))
+    return UnsummedRows(scratch, runs.value, t, n)
+
+
 def gemm(weight: torch.Tensor, x: torch.Tensor, out: torch.Tensor, epilogue: int = EPI_STORE,
          kind: int = GEMM_AUTO, scratch: Optional[torch.Tensor] = None, splits: int = 0) -> torch.Tensor:
     """out (epilogue)= x @ weight.T with weight [N, K], x [T, K].
@@ -239,9 +272,11 @@ def gemm_rmsnorm(weight: torch.Tensor, x: torch.Tensor, norm_weight: torch.Tenso
 def rope_kv(qkv: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, rot: int, interleaved: bool,
             cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
             tok_seq: Optional[torch.Tensor], slots: Optional[torch.Tensor], page_table: Optional[torch.Tensor],
-            cache: Optional[torch.Tensor], page_stride: int, v_off: int, write_kv: bool = True) -> None:
+            cache: Optional[torch.Tensor], page_stride: int, v_off: int, write_kv: bool = True,
+            unsummed: Optional[UnsummedRows] = None) -> None:
     """Rotate the query heads of qkv [T, (H+2KV)*hd] in place; rotate the key heads and copy the value heads
-    into the cache page of each token (cache: the first element of this layer's pages)."""
+    into the cache page of each token (cache: the first element of this layer's pages).  unsummed: the rows are not
+    in qkv yet but in the runs that gemm_runs left (see rope_takes_unsummed); the rotated queries are written to qkv."""
     _need(qkv, "qkv rows", dims=2)
     _need(positions, "positions", torch.int32, 1)
     t = qkv.shape[0]
@@ -263,10 +298,21 @@ def rope_kv(qkv: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, rot: int,
         if tok_seq.shape[0] != t or not page_table.is_contiguous():
             raise KernelError("rope_kv: one sequence index per row and a contiguous page table")
         max_pages = page_table.shape[1]
+    part = (_ptr(None), 0, ctypes.c_longlong(0), 0)
+    if unsummed is not None:
+        if unsummed.rows != t or unsummed.cols < (n_heads + (2 * n_kv if write_kv else 0)) * head_dim:
+            raise KernelError(f"rope_kv: unsummed rows [{unsummed.rows}, {unsummed.cols}] do not fit {t} rows of qkv")
+        part = (_ptr(unsummed.scratch), unsummed.runs, ctypes.c_longlong(unsummed.rows * unsummed.cols), unsummed.cols)
     _check(_lib("rope_kv").dlgo_rope_kv(_ptr(qkv), dtype_code(qkv.dtype), t, _rows(qkv, "qkv rows"), n_heads, n_kv, head_dim,
                                         rot, int(interleaved), _ptr(cos), _ptr(sin), table_rows, _ptr(positions),
                                         _ptr(tok_seq), _ptr(slots), _ptr(page_table), max_pages, _ptr(cache),
-                                        ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(write_kv), _stream()))
+                                        ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(write_kv), *part, _stream()))
+
+
+def rope_takes_unsummed(dtype: torch.dtype, head_dim: int, rot: int) -> bool:
+    """Whether rope_kv can read rows that gemm_runs left unsummed: it does so in whole 16-byte pieces."""
+    epc = 4 if dtype == torch.float32 else 8
+    return head_dim % epc == 0 and rot % (2 * epc) == 0
 
 
 def attention_rows(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_dim: int,

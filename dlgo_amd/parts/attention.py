@@ -108,19 +108,25 @@ class Attention(Mixer):
         cols = self.q_dim + 2 * n_kv * self.head_dim
         qkv = ctx.buffer("attention.qkv", (t, self.q_dim + 2 * self.kv_dim), ctx.dtype)
         split = ctx.scratch("gemm.split", ops.GEMM_SPLIT_FLOATS, torch.float32)
-        if norm is not None:      # xn are the float32 residual rows: the norm rides in the product
-            ops.gemm_rmsnorm(self.w_qkv[:cols], xn, norm.weight, norm.eps, qkv[:, :cols])
-        else:
-            ops.gemm(self.w_qkv[:cols], xn, qkv[:, :cols], scratch=split)
         kv = ctx.cache.kv_view(unit)
         rot = self.position.rotation()
         # a step of single tokens: the attention kernel rotates and stores by itself; else a kernel of its own does
         fused = ops.attention_fuses_rotation(ctx.dtype, self.head_dim, self.n_heads // self.n_kv_heads, ctx.max_q_len,
                                              rot.width if rot else 0, ctx.n_seq)
+        unsummed = None
+        if norm is not None:      # xn are the float32 residual rows: the norm rides in the product
+            ops.gemm_rmsnorm(self.w_qkv[:cols], xn, norm.weight, norm.eps, qkv[:, :cols])
+        else:
+            # a product that shares k out over blocks leaves its runs to the rotation kernel, which adds them up as it reads
+            if not fused and ops.rope_takes_unsummed(ctx.dtype, self.head_dim, rot.width if rot else 0):
+                unsummed = ops.gemm_runs(self.w_qkv[:cols], xn, split)
+            if unsummed is None:
+                ops.gemm(self.w_qkv[:cols], xn, qkv[:, :cols], scratch=split)
         if not fused:
             ops.rope_kv(qkv, self.n_heads, n_kv, self.head_dim, rot.width if rot else 0, rot.interleaved if rot else False,
                         rot.cos if rot else None, rot.sin if rot else None, ctx.positions,
-                        ctx.tok_seq, ctx.slots, kv.page_table, kv.cache, kv.page_stride, kv.v_off, write_kv=owns_cache)
+                        ctx.tok_seq, ctx.slots, kv.page_table, kv.cache, kv.page_stride, kv.v_off, write_kv=owns_cache,
+                        unsummed=unsummed)
         out = ctx.buffer("attention.out", (t, self.q_dim), ctx.dtype)
         self.attend(qkv, out, ctx, kv, rotation=(rot.cos, rot.sin, rot.width, rot.interleaved) if fused and rot else None,
                     new_kv=fused and owns_cache)

@@ -359,6 +359,40 @@ def test_rope_kv_write(dtype, _, rel, H, KV, hd, rot, inter):
     assert written == T * 2 * KV * hd
 
 
+@pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("H,KV,hd,rot,inter,write", [(4, 2, 16, 16, False, True), (6, 3, 48, 48, True, True),
+                                                     (8, 1, 128, 64, False, True), (5, 1, 80, 32, False, False)])
+def test_rope_kv_from_unsummed_runs(dtype, _, rel, H, KV, hd, rot, inter, write):
+    """The rows as three unsummed planes (values whose sums are exact in every dtype) give what the summed rows give, bit
+    for bit: rotated queries in qkv, keys and values in the pages."""
+    ops = _ops()
+    from dlgo_amd.parts import rotary_frequencies
+    lens, starts = [70, 3, 129], [5, 0, 64]
+    q_lens = [l - s for l, s in zip(lens, starts)]
+    table, slots, storage, page_stride, unit_off, v_off = _paged_setup(dtype, lens, KV, hd)
+    T = sum(q_lens)
+    cols = (H + (2 * KV if write else 0)) * hd
+    g = torch.Generator().manual_seed(5)
+    planes = torch.randint(-8, 9, (3, T, cols), generator=g).float() / 8      # sums: multiples of 1/8 below 4
+    rows = torch.zeros(T, (H + 2 * KV) * hd)
+    rows[:, :cols] = planes[0] + planes[1] + planes[2]
+    positions = torch.tensor([p for s, n in zip(starts, q_lens) for p in range(s, s + n)], dtype=torch.int32).to(DEV)
+    tok_seq = torch.tensor([i for i, n in enumerate(q_lens) for _ in range(n)], dtype=torch.int32).to(DEV)
+    freqs = rotary_frequencies(rot, 10000.0)
+    ang = np.arange(200)[:, None] * freqs[None]
+    cos, sin = torch.from_numpy(np.cos(ang).astype(np.float32)).to(DEV), torch.from_numpy(np.sin(ang).astype(np.float32)).to(DEV)
+    slot_t = torch.tensor(slots, dtype=torch.int32, device=DEV)
+    got = []
+    for unsummed in (None, ops.UnsummedRows(planes.reshape(-1).to(DEV), 3, T, cols)):
+        dq = rows.to(dtype).to(DEV) if unsummed is None else torch.full_like(rows, float("nan")).to(dtype).to(DEV)
+        store = storage.clone().to(DEV)
+        ops.rope_kv(dq, H, KV if write else 0, hd, rot, inter, cos, sin, positions, tok_seq, slot_t, table.to(DEV),
+                    store[unit_off:], page_stride, v_off, write_kv=write, unsummed=unsummed)
+        got.append((dq[:, :H * hd].cpu(), store.cpu()))
+    assert torch.equal(got[0][0], got[1][0]), "rotated queries"
+    assert torch.equal(torch.nan_to_num(got[0][1].float(), nan=-77.0), torch.nan_to_num(got[1][1].float(), nan=-77.0)), "pages"
+
+
 def _attention_ref(q, k, v, H, KV, hd, pos_of_q, lo_of_q):
     """q [n, H*hd]; k, v [len, KV*hd] for one sequence; row i attends keys lo..pos."""
     g = H // KV
