@@ -569,8 +569,8 @@ __device__ __forceinline__ uint4 rotated8(const bf16_t* __restrict__ vec, int d0
     const float c[4] = {c4.x, c4.y, c4.z, c4.w}, sv[4] = {s4.x, s4.y, s4.z, s4.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      y[2 * i] = x[2 * i] * c[i] - x[2 * i + 1] * sv[i];
-      y[2 * i + 1] = x[2 * i] * sv[i] + x[2 * i + 1] * c[i];
+      y[2 * i] = rotated_lo(x[2 * i], x[2 * i + 1], c[i], sv[i]);
+      y[2 * i + 1] = rotated_hi(x[2 * i], x[2 * i + 1], c[i], sv[i]);
     }
   } else {
     const int half = rot / 2;
@@ -583,7 +583,7 @@ __device__ __forceinline__ uint4 rotated8(const bf16_t* __restrict__ vec, int d0
     *(float4*)sv = *(const float4*)(sn + i0);
     *(float4*)(sv + 4) = *(const float4*)(sn + i0 + 4);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) y[e] = low ? x[e] * c[e] - p[e] * sv[e] : p[e] * sv[e] + x[e] * c[e];
+    for (int e = 0; e < 8; ++e) y[e] = low ? rotated_lo(x[e], p[e], c[e], sv[e]) : rotated_hi(p[e], x[e], c[e], sv[e]);
   }
   union { uint4 u; bf16x8_t v; } o;
 #pragma unroll

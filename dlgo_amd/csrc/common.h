@@ -26,6 +26,11 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
   return __builtin_bit_cast(bf16_t, b);
 }
 
+// One rotation of a pair (x0, x1) by the angle whose cosine and sine are c and s.  Written as a product and one fused
+// multiply-add, so that every kernel that rotates gives the same bits whatever the compiler would otherwise contract.
+__device__ __forceinline__ float rotated_lo(float x0, float x1, float c, float s) { return __builtin_fmaf(-x1, s, x0 * c); }
+__device__ __forceinline__ float rotated_hi(float x0, float x1, float c, float s) { return __builtin_fmaf(x0, s, x1 * c); }
+
 template <typename T> struct Elem;
 template <> struct Elem<float> {
   static constexpr int code = DLGO_DTYPE_F32;

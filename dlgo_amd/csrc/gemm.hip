@@ -518,13 +518,22 @@ static const char* launch_tiled(const void* W, const void* X, void* Y, int N, in
   return nullptr;
 }
 
-// In how many runs a product shares its k tiles out when the choice is the kernel's: few rows of X, few tiles of output.
+// In how many runs a product shares its k tiles out when the choice is the kernel's (64x64 tiles).  Few rows of X and
+// few tiles of output: a block for every compute unit, of at least eight k tiles.  More rows (a short prompt) and a long
+// inner size: about two blocks a unit, at most four runs.  (Measured on the shapes of 1B and 8B Llamas.)
 static int auto_splits(int N, int Tn, int nk_all, long long part_elems) {
   const long small = (long)((N + 63) / 64) * ((Tn + 63) / 64);
-  if (!(Tn <= 128 && small <= 64 && nk_all >= 32)) return 1;
-  int splits = (int)(256 / small);                          // a block for every compute unit ...
-  if (splits > nk_all / 8) splits = nk_all / 8;             // ... of at least eight k tiles
-  if ((long long)splits * Tn * N > part_elems) splits = 1;
+  int splits = 1;
+  if (Tn <= 128) {
+    if (small <= 64 && nk_all >= 32) {
+      splits = (int)(256 / small);
+      if (splits > nk_all / 8) splits = nk_all / 8;
+    }
+  } else if (small <= 256 && nk_all >= 128) {
+    splits = (int)(512 / small);
+    if (splits > 4) splits = 4;
+  }
+  while (splits > 1 && (long long)splits * Tn * N > part_elems) --splits;
   return splits;
 }
 
@@ -550,11 +559,14 @@ static const char* dispatch(const void* W, const void* X, void* Y, int N, int Tn
   if (kind == 0 && direct) {
     const long b256 = (long)((N + 255) / 256) * ((Tn + 255) / 256);
     const long big = (long)((N + 127) / 128) * ((Tn + 127) / 128);
-    // Few rows of X: the weights stream through small tiles.  Else the large tile when it fills the chip; else two blocks
-    // of 128x128 on a unit when there are that many; else one, deeper.  (Measured on the shapes of a 1B Llama.)
+    const long small = (long)((N + 63) / 64) * ((Tn + 63) / 64);
+    // Few rows of X: the weights stream through small tiles, and so does any product of at most two small tiles a compute
+    // unit.  Else the large tile when it fills the chip; else two blocks of 128x128 on a unit when there are that many;
+    // else one, deeper.  (Measured on the shapes of a 1B Llama.)
     if (Tn <= 64) kind = 23;
     else if (Tn <= 128) kind = N >= 32768 ? 21 : 23;
-    else if (big >= 128) kind = b256 >= 256 ? 20 : (big > 256 ? 21 : 22);
+    else if (small <= 512) kind = 23;
+    else if (big >= 128) kind = b256 >= 192 ? 20 : (big > 256 ? 21 : 22);
   }
   if (kind == 23) return launch_direct<T, 64, 64, 2, 2, 4, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 20) return launch_direct<T, 256, 256, 4, 4, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);

@@ -58,8 +58,8 @@ __global__ __launch_bounds__(WAVE) void rope_kv_kernel(T* __restrict__ qkv, int 
     float x0 = Elem<T>::load(src + i0), x1 = Elem<T>::load(src + i1);
     if (c) {
       const float cs = c[i], sn = s[i];
-      const float y0 = x0 * cs - x1 * sn;
-      const float y1 = x0 * sn + x1 * cs;
+      const float y0 = rotated_lo(x0, x1, cs, sn);
+      const float y1 = rotated_hi(x0, x1, cs, sn);
       x0 = y0;
       x1 = y1;
     }
@@ -201,8 +201,8 @@ __global__ __launch_bounds__(256) void rope_kv_pieces_kernel(T* __restrict__ qkv
 #pragma unroll
     for (int i = 0; i < E / 2; ++i) {
       const float c_ = cs[d0 / 2 + i], s_ = sn[d0 / 2 + i];
-      y[2 * i] = x[2 * i] * c_ - x[2 * i + 1] * s_;
-      y[2 * i + 1] = x[2 * i] * s_ + x[2 * i + 1] * c_;
+      y[2 * i] = rotated_lo(x[2 * i], x[2 * i + 1], c_, s_);
+      y[2 * i + 1] = rotated_hi(x[2 * i], x[2 * i + 1], c_, s_);
     }
     Piece<T>::store(dst + d0, y);
   } else {
@@ -212,8 +212,8 @@ __global__ __launch_bounds__(256) void rope_kv_pieces_kernel(T* __restrict__ qkv
 #pragma unroll
     for (int e = 0; e < E; ++e) {
       const float c_ = cs[d0 + e], s_ = sn[d0 + e];
-      y0[e] = x[e] * c_ - p[e] * s_;
-      y1[e] = x[e] * s_ + p[e] * c_;
+      y0[e] = rotated_lo(x[e], p[e], c_, s_);
+      y1[e] = rotated_hi(x[e], p[e], c_, s_);
     }
     Piece<T>::store(dst + d0, y0);
     Piece<T>::store(dst + d0 + half, y1);

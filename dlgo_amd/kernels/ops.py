@@ -18,7 +18,7 @@ PAGE = 64   # tokens per cache page; the kernels are compiled with the same numb
 EPI_STORE, EPI_ACCUM_F32, EPI_SWIGLU, EPI_STORE_F32 = 0, 1, 2, 3
 GEMM_AUTO, GEMM_STREAM, GEMM_TILE128, GEMM_TILE64, GEMM_TILE32, GEMM_ROWS16 = 0, 1, 2, 3, 4, 5
 GEMM_FEW_ROWS = 64      # up to this many rows of x the weight-streaming kernels can be chosen
-GEMM_SPLIT_FLOATS = 1 << 20   # scratch that lets gemm() share the inner size of a product out over blocks
+GEMM_SPLIT_FLOATS = 1 << 22   # scratch that lets gemm() share the inner size of a product out over blocks
 GEMM_VERY_WIDE = 65536   # from this many weight rows on (a vocabulary) the tiled kernel is faster for any number of rows of x
 GEMM_FEW_ROWS_WIDE = 16  # ... and up to this many when the weight has very many rows (there the tiled kernel is faster)
 

@@ -173,7 +173,8 @@ def test_gemm_with_split_inner_size(dtype, _, rel, n, t, k, splits):
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
 @pytest.mark.parametrize("n,t,k,fused", [(2048, 8, 8192, True), (1024, 64, 4096, True), (4096, 33, 8192, True), (3072, 30, 2048, True),
-                                         (2052, 8, 8192, True), (2048, 8, 512, False), (2050, 8, 8192, False), (2048, 200, 8192, False)])
+                                         (2052, 8, 8192, True), (2048, 8, 512, False), (2050, 8, 8192, False), (2048, 200, 8192, True),
+                                         (2048, 200, 2048, False), (2048, 600, 8192, False)])
 def test_gemm_into_the_residual_that_leaves_the_next_norm(dtype, _, rel, n, t, k, fused):
     """A product whose inner size is shared out adds into the residual rows and leaves their RMSNorm beside them; where
     the product would not be split (or N does not suit) it does nothing and says so."""
