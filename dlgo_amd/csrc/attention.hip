@@ -822,6 +822,185 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_kernel(
   }
 }
 
+// float32, one token per sequence, head sizes up to 128: attn_decode_kernel's arrangement (the pages of a split go to the
+// block's waves in turn, all heads of the group are the MFMA's 16 columns, the waves merge through LDS in wave order)
+// with v_mfma_f32_16x16x4_f32, a true float32 product, and expf.  A wave holds the keys and values of KT 16-key tiles
+// at once (64 registers each, whatever the head size) and takes a page in 4 / KT such groups.
+// Scores: MFMA row = key, column = head, and the four elements a lane holds of a 16-element chunk of the head are four
+// k steps (the same elements on the key's and the query's side).  The scores land where the second product wants
+// them: a lane's score of key 16 t + 4 G + v is the operand of k step (t, v), whose value operand is element v of the
+// lane's 16 bytes of a transposed value row.
+#if HEAD_DIM <= 128
+template <int NWV>
+__global__ __launch_bounds__(NWV* WAVE) void attn_decode_f32_kernel(
+    const float* __restrict__ q, int ldq, float* __restrict__ out, int ldo, float* __restrict__ part,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, const int32_t* __restrict__ page_table,
+    int max_pages, const float* __restrict__ cache, long long page_stride, long long v_off, int n_heads, int group,
+    int head_blocks, int n_splits, int window, float scale) {
+  constexpr int HD = HEAD_DIM;
+  constexpr int KC = HD / 16;          // 16-element chunks of the head
+  constexpr int DT = HD / 16;          // 16-row tiles of the output's head dimension
+  constexpr int KT = HD <= 64 ? 4 : 2; // 16-key tiles held at once
+  constexpr int LS = HD + 2;           // floats a wave leaves in LDS per head: values, max, sum
+  extern __shared__ float lds[];
+  const int split = blockIdx.x, seq = blockIdx.z;
+  const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
+  const int pos = positions[seq];
+  const int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+  const int first_pg = lo / PAGE, last_pg = pos / PAGE;
+  const int span = (last_pg - first_pg + n_splits) / n_splits;
+  const int pg0 = first_pg + split * span;
+  const int pg1 = pg0 + span - 1 < last_pg ? pg0 + span - 1 : last_pg;
+  if (pg0 > pg1) return;               // the whole block: fewer pages than splits
+  const int slot = slots[seq];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, j = lane & 15, G = lane >> 4;
+  const int heads_here = group - hb * 16 < 16 ? group - hb * 16 : 16;
+  const bool head_ok = j < heads_here;
+  const int head = kvh * group + hb * 16 + j;
+
+  float4 qf[KC];
+  bool have_q = false;                 // the queries are read behind the first keys' loads
+  f32x4_t o[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d) o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+
+  for (int pg = pg0 + wave; pg <= pg1; pg += NWV) {
+    const int page = page_table[(size_t)slot * max_pages + pg];
+    if (page < 0) continue;
+    const float* kpage = cache + (size_t)page * page_stride + (size_t)kvh * PAGE * HD;
+    const float* vpage = cache + v_off + (size_t)page * page_stride + (size_t)kvh * HD * PAGE;
+#pragma unroll 1
+    for (int kbase = 0; kbase < PAGE; kbase += KT * 16) {
+      const int key0 = pg * PAGE + kbase;
+      if (key0 > pos) break;                       // nothing but keys beyond the token from here on
+      if (key0 + KT * 16 - 1 < lo) continue;       // nothing but keys before the window
+      float4 kf[KT][KC];
+#pragma unroll
+      for (int t = 0; t < KT; ++t) {
+        const float* krow = kpage + (size_t)(kbase + t * 16 + j) * HD + 4 * G;
+#pragma unroll
+        for (int c = 0; c < KC; ++c) kf[t][c] = *(const float4*)(krow + 16 * c);
+      }
+      float4 vf[KT][DT];
+#pragma unroll
+      for (int t = 0; t < KT; ++t)
+#pragma unroll
+        for (int d = 0; d < DT; ++d) vf[t][d] = *(const float4*)(vpage + (size_t)(d * 16 + j) * PAGE + kbase + t * 16 + 4 * G);
+      if (!have_q) {
+        have_q = true;
+        const float* qrow = q + (size_t)seq * ldq + (size_t)(head_ok ? head : kvh * group) * HD + 4 * G;
+#pragma unroll
+        for (int c = 0; c < KC; ++c) qf[c] = head_ok ? *(const float4*)(qrow + 16 * c) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+      f32x4_t s[KT];
+#pragma unroll
+      for (int t = 0; t < KT; ++t) {
+        s[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+          s[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t][c].x, qf[c].x, s[t], 0, 0, 0);
+          s[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t][c].y, qf[c].y, s[t], 0, 0, 0);
+          s[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t][c].z, qf[c].z, s[t], 0, 0, 0);
+          s[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(kf[t][c].w, qf[c].w, s[t], 0, 0, 0);
+        }
+      }
+      // lane: head = lane%16; element v of tile t is key  key0 + 16 t + 4 G + v.  At least one key of the group counts.
+      const bool need_mask = key0 + KT * 16 - 1 > pos || key0 < lo;
+      float mx = -INFINITY;
+#pragma unroll
+      for (int t = 0; t < KT; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          float sv = s[t][v] * scale;
+          if (need_mask) {
+            const int key = key0 + 16 * t + 4 * G + v;
+            sv = (key <= pos && key >= lo) ? sv : -INFINITY;
+          }
+          s[t][v] = sv;
+          mx = fmaxf(mx, sv);
+        }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+      const float m_new = fmaxf(m, mx);
+      const float alpha = expf(m - m_new);
+      float rs = 0.f;
+#pragma unroll
+      for (int t = 0; t < KT; ++t)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+          const float p = expf(s[t][v] - m_new);
+          s[t][v] = p;
+          rs += p;
+        }
+      rs += __shfl_xor(rs, 16, WAVE);
+      rs += __shfl_xor(rs, 32, WAVE);
+      l = l * alpha + rs;
+      m = m_new;
+#pragma unroll
+      for (int d = 0; d < DT; ++d) o[d] *= alpha;
+      const bool tail = key0 + KT * 16 - 1 > pos;    // keys beyond the sequence: their values must not reach the product
+#pragma unroll
+      for (int t = 0; t < KT; ++t) {
+        const int ka = key0 + 16 * t + 4 * G;
+#pragma unroll
+        for (int d = 0; d < DT; ++d) {
+          float4 a = vf[t][d];
+          if (tail) {
+            a.x = ka <= pos ? a.x : 0.f;
+            a.y = ka + 1 <= pos ? a.y : 0.f;
+            a.z = ka + 2 <= pos ? a.z : 0.f;
+            a.w = ka + 3 <= pos ? a.w : 0.f;
+          }
+          o[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, s[t][0], o[d], 0, 0, 0);
+          o[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, s[t][1], o[d], 0, 0, 0);
+          o[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, s[t][2], o[d], 0, 0, 0);
+          o[d] = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, s[t][3], o[d], 0, 0, 0);
+        }
+      }
+    }
+  }
+  // each wave leaves (values, max, sum) per head in LDS; a wave that saw no key leaves (0, -inf, 0)
+  if (head_ok) {
+    float* dst = lds + (size_t)(wave * heads_here + j) * LS;
+#pragma unroll
+    for (int d = 0; d < DT; ++d)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) dst[d * 16 + 4 * G + v] = o[d][v];
+    if (G == 0) {
+      dst[HD] = m;
+      dst[HD + 1] = l;
+    }
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < heads_here * HD; idx += NWV * WAVE) {
+    const int hh = idx / HD, d = idx - hh * HD;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NWV; ++w) M = fmaxf(M, lds[(size_t)(w * heads_here + hh) * LS + HD]);
+    float L = 0.f, acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < NWV; ++w) {
+      const float* src = lds + (size_t)(w * heads_here + hh) * LS;
+      const float wt = expf(src[HD] - M);          // the block holds a key, so M is finite; a wave without one weighs 0
+      L = fmaf(wt, src[HD + 1], L);
+      acc = fmaf(wt, src[d], acc);
+    }
+    const int hd_ = kvh * group + hb * 16 + hh;
+    if (n_splits == 1) {
+      out[(size_t)seq * ldo + (size_t)hd_ * HD + d] = acc / L;
+    } else {
+      float* dst = part + ((size_t)(seq * n_heads + hd_) * n_splits + split) * (HD + 4);
+      dst[d] = acc;
+      if (d == 0) {
+        dst[HD] = M;
+        dst[HD + 1] = L;
+      }
+    }
+  }
+}
+#endif
+
 // grid (sequences, heads); merges the partials of the splits that hold keys of the token, in page order.  A lane takes
 // one element of the head (and every lane the same maxima and sums).  Eight splits at a time, their loads issued before
 // the token's position is known: which of them count is decided afterwards, so that the position and the partials
@@ -1062,4 +1241,52 @@ extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, 
     DLGO_LAUNCH_CHECK("attention_combine");
   }
   return nullptr;
+}
+
+// float32, one row per sequence, head sizes up to 128: arguments as dlgo_attention_decode without the rotation; the
+// scratch is sized by dlgo_attention_decode_splits(..., fused = 0).
+extern "C" const char* dlgo_attention_decode_f32(const void* q, int ldq, void* out, int ldo, float* part, long long part_elems,
+                                                 int n_seq, int n_heads, int n_kv, int head_dim, const int32_t* positions,
+                                                 const int32_t* slots, const int32_t* page_table, int max_pages,
+                                                 int max_pages_used, const void* cache, long long page_stride, long long v_off,
+                                                 int window, float scale, hipStream_t stream) {
+  DLGO_REQUIRE(head_dim == HEAD_DIM, "attention: this library is built for head size %d, got %d", HEAD_DIM, head_dim);
+#if HEAD_DIM <= 128
+  DLGO_REQUIRE(n_seq >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention: bad sizes");
+  DLGO_REQUIRE(max_pages_used >= 1 && max_pages_used <= max_pages, "attention: bad bound on the pages of a sequence");
+  DLGO_REQUIRE(ldq >= n_heads * head_dim && ldo >= n_heads * head_dim && ldq % 4 == 0, "attention: row strides");
+  DLGO_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)cache & 15) == 0 && page_stride % 4 == 0 && v_off % 4 == 0,
+               "attention: operands must be 16-byte aligned");
+  DLGO_REQUIRE(window >= 0, "attention: bad window");
+  const int group = n_heads / n_kv;
+  const int head_blocks = (group + 15) / 16;
+  int nwv, n_splits;
+  decode_plan(n_seq * n_kv * head_blocks, group, max_pages_used, false, &nwv, &n_splits);
+  if (nwv > 8) nwv = 8;                // a wave holds 128 registers of keys and values: two waves to a SIMD
+  DLGO_REQUIRE(n_splits == 1 || (part && part_elems >= (long long)n_seq * n_heads * n_splits * (HEAD_DIM + 4)),
+               "attention: scratch for partial results too small");
+  DLGO_REQUIRE((long long)n_kv * head_blocks <= 65535 && n_seq <= 65535 && n_heads <= 65535, "attention: grid too large");
+  if (n_seq == 0) return nullptr;
+  const int heads_here = group < 16 ? group : 16;
+  const size_t smem = (size_t)nwv * heads_here * (HEAD_DIM + 2) * 4;
+  dim3 grid(n_splits, n_kv * head_blocks, n_seq);
+#define DECODE_GO(W_)                                                                                                         \
+  hipLaunchKernelGGL((attn_decode_f32_kernel<W_>), grid, dim3(W_ * WAVE), smem, stream, (const float*)q, ldq, (float*)out, ldo, \
+                     part, positions, slots, page_table, max_pages, (const float*)cache, page_stride, v_off, n_heads, group,  \
+                     head_blocks, n_splits, window, scale)
+  if (nwv == 8) DECODE_GO(8);
+  else if (nwv == 4) DECODE_GO(4);
+  else if (nwv == 2) DECODE_GO(2);
+  else DECODE_GO(1);
+#undef DECODE_GO
+  DLGO_LAUNCH_CHECK("attention_decode_f32");
+  if (n_splits > 1) {
+    hipLaunchKernelGGL((attn_combine_kernel<float, true>), dim3(n_seq, n_heads), dim3(WAVE), 0, stream, part, (float*)out, ldo,
+                       positions, n_heads, n_splits, window);
+    DLGO_LAUNCH_CHECK("attention_combine");
+  }
+  return nullptr;
+#else
+  DLGO_FAIL("attention: the float32 split kernel takes head sizes up to 128, this library is built for %d", HEAD_DIM);
+#endif
 }

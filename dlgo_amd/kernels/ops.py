@@ -80,7 +80,7 @@ def _lib(module: str, defines=()):
     if lib is None:
         lib = build.load(module, defines)
         for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_accum_norm", "dlgo_gemm_parts", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_attention_rows",
-                     "dlgo_attention_prefill", "dlgo_attention_prefill_f32", "dlgo_attention_decode", "dlgo_argmax", "dlgo_sample"):
+                     "dlgo_attention_prefill", "dlgo_attention_prefill_f32", "dlgo_attention_decode", "dlgo_attention_decode_f32", "dlgo_argmax", "dlgo_sample"):
             if hasattr(lib, name):
                 getattr(lib, name).restype = ctypes.c_char_p
         _libs[key] = lib
@@ -379,10 +379,14 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
     group = n_heads // n_kv
     fast_ok = q.dtype == torch.bfloat16 and head_dim <= 256 and group <= 128
     tiled_f32 = q.dtype == torch.float32 and head_dim <= 64 and group <= 128       # prompts in float32: a kernel of their own
+    split_f32 = q.dtype == torch.float32 and head_dim <= 128 and group <= 128      # and so have steps of single tokens
     if kernel == "auto":
-        kernel = ("tiled" if tiled_f32 and max_q > 1 else "rows") if not fast_ok else ("split" if max_q == 1 else "tiled")
+        if fast_ok:
+            kernel = "split" if max_q == 1 else "tiled"
+        else:
+            kernel = "split" if split_f32 and max_q == 1 else ("tiled" if tiled_f32 and max_q > 1 else "rows")
     if (rotation is not None or new_kv) and not (kernel == "split" and fast_ok and max_q == 1):
-        raise KernelError("attention: only the split kernel rotates and stores by itself")
+        raise KernelError("attention: only the bfloat16 split kernel rotates and stores by itself")
     if kernel == "rows" or n_seq == 0:
         # a few rows with long histories (a decode step off the fast kernels): each row's pages go to several waves
         n_splits = 1
@@ -391,9 +395,9 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
             n_splits = max(1, min(pages // 2, 2048 // max(1, n_seq * n_heads)))
         return attention_rows(q, out, n_heads, n_kv, head_dim, positions, tok_seq, slots, page_table, cache, page_stride,
                               v_off, window, scale, n_splits, scratch)
-    if not fast_ok and not (tiled_f32 and kernel == "tiled"):
+    if not fast_ok and not (tiled_f32 and kernel == "tiled") and not (split_f32 and kernel == "split"):
         raise KernelError("attention: the tiled and split kernels take bfloat16, head sizes up to 256 and up to 128 heads per kv head "
-                          "(the tiled one also float32 with head sizes up to 64)")
+                          "(and float32 with head sizes up to 64 and 128)")
     _need(q, "query rows", q.dtype, 2)
     _need(out, "attention output", q.dtype, 2)
     _need(slots, "slots", torch.int32, 1)
@@ -429,6 +433,13 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
             need = n_seq * n_heads * n_splits * (head_dim + 4)
             part = scratch(need) if scratch is not None else torch.empty(need, dtype=torch.float32, device=q.device)
             _need(part, "attention scratch", torch.float32, 1)
+        if q.dtype == torch.float32:
+            _check(lib.dlgo_attention_decode_f32(_ptr(q), _rows(q, "query rows"), _ptr(out), _rows(out, "attention output"), _ptr(part),
+                                                 ctypes.c_longlong(part.numel() if part is not None else 0), n_seq, n_heads, n_kv,
+                                                 head_dim, _ptr(positions), _ptr(slots), _ptr(page_table), max_pages, max_pages_used,
+                                                 _ptr(cache), ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(window),
+                                                 ctypes.c_float(scale), _stream()))
+            return out
         _check(lib.dlgo_attention_decode(_ptr(q), _rows(q, "query rows"), _ptr(out), _rows(out, "attention output"), _ptr(part),
                                          ctypes.c_longlong(part.numel() if part is not None else 0), n_seq, n_heads, n_kv,
                                          head_dim, _ptr(positions), _ptr(slots), _ptr(page_table), max_pages, max_pages_used,
