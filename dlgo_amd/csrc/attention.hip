@@ -434,10 +434,10 @@ __global__ __launch_bounds__(PF_THREADS* PF_TEAMS) __attribute__((amdgpu_waves_p
     }
 }
 
-// Prefill in float32, for head sizes up to 64: a thread owns a query row (token x head of the group, 128 rows a block),
+// Prefill in float32, for head sizes up to 128: a thread owns a query row (token x head of the group, 128 rows a block),
 // a page of keys and of transposed values sits in LDS, and every product is an FMA on float32 with exact expf; the
 // keys are taken 16 at a time so that the scores stay in registers.  grid and bq as attn_prefill_kernel.
-#if HEAD_DIM <= 64
+#if HEAD_DIM <= 128
 #define PF32_THREADS 128
 __global__ __launch_bounds__(PF32_THREADS) void attn_prefill_f32_kernel(
     const float* __restrict__ q, int ldq, float* __restrict__ out, int ldo, const int32_t* __restrict__ cu_q,
@@ -1131,14 +1131,14 @@ extern "C" const char* dlgo_attention_prefill(const void* q, int ldq, void* out,
   return nullptr;
 }
 
-// float32, every sequence's rows of this step, head sizes up to 64: arguments as dlgo_attention_prefill.
+// float32, every sequence's rows of this step, head sizes up to 128: arguments as dlgo_attention_prefill.
 extern "C" const char* dlgo_attention_prefill_f32(const void* q, int ldq, void* out, int ldo, int n_seq, int max_q_len, int n_heads,
                                                   int n_kv, int head_dim, const int32_t* cu_q, const int32_t* start_pos,
                                                   const int32_t* slots, const int32_t* page_table, int max_pages,
                                                   const void* cache, long long page_stride, long long v_off, int window,
                                                   float scale, hipStream_t stream) {
   DLGO_REQUIRE(head_dim == HEAD_DIM, "attention: this library is built for head size %d, got %d", HEAD_DIM, head_dim);
-#if HEAD_DIM <= 64
+#if HEAD_DIM <= 128
   DLGO_REQUIRE(n_seq >= 0 && max_q_len >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention: bad sizes");
   const int group = n_heads / n_kv;
   DLGO_REQUIRE(group <= PF32_THREADS, "attention: the float32 tiled kernel takes up to %d query heads per kv head, got %d", PF32_THREADS, group);
@@ -1154,7 +1154,7 @@ extern "C" const char* dlgo_attention_prefill_f32(const void* q, int ldq, void* 
   DLGO_LAUNCH_CHECK("attention_prefill_f32");
   return nullptr;
 #else
-  DLGO_FAIL("attention: the float32 tiled kernel takes head sizes up to 64, this library is built for %d", HEAD_DIM);
+  DLGO_FAIL("attention: the float32 tiled kernel takes head sizes up to 128, this library is built for %d", HEAD_DIM);
 #endif
 }
 

@@ -378,7 +378,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
     max_q = int(max(q_lens)) if n_seq else 0
     group = n_heads // n_kv
     fast_ok = q.dtype == torch.bfloat16 and head_dim <= 256 and group <= 128
-    tiled_f32 = q.dtype == torch.float32 and head_dim <= 64 and group <= 128       # prompts in float32: a kernel of their own
+    tiled_f32 = q.dtype == torch.float32 and head_dim <= 128 and group <= 128       # prompts in float32: a kernel of their own
     split_f32 = q.dtype == torch.float32 and head_dim <= 128 and group <= 128      # and so have steps of single tokens
     if kernel == "auto":
         if fast_ok:
@@ -397,7 +397,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
                               v_off, window, scale, n_splits, scratch)
     if not fast_ok and not (tiled_f32 and kernel == "tiled") and not (split_f32 and kernel == "split"):
         raise KernelError("attention: the tiled and split kernels take bfloat16, head sizes up to 256 and up to 128 heads per kv head "
-                          "(and float32 with head sizes up to 64 and 128)")
+                          "(and float32 with head sizes up to 128)")
     _need(q, "query rows", q.dtype, 2)
     _need(out, "attention output", q.dtype, 2)
     _need(slots, "slots", torch.int32, 1)
