@@ -212,9 +212,10 @@ __global__ __launch_bounds__(PF_THREADS* PF_TEAMS) __attribute__((amdgpu_waves_p
   const int q0 = cu_q[seq], qn = cu_q[seq + 1] - q0;
   // Late tiles see more keys than early ones.  Blocks are handed to the compute units in the order of their linear
   // index, 256 at a time: odd rounds walk the tiles forwards and even rounds backwards, so that the blocks that share
-  // a unit add up to about the same number of pages.
-  const int linear = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-  const int tile = (linear >> 8) & 1 ? blockIdx.x : gridDim.x - 1 - blockIdx.x;
+  // a unit add up to about the same number of pages.  The direction is that of the round in which the row of tiles
+  // (one sequence, one kv head) starts: the same for all its blocks, so that every tile is taken exactly once.
+  const int linear0 = gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const int tile = (linear0 >> 8) & 1 ? blockIdx.x : gridDim.x - 1 - blockIdx.x;
   const int t0 = tile * bq;
   if (t0 >= qn) return;
   const int t1 = t0 + bq < qn ? t0 + bq : qn;           // tokens [t0, t1) of the sequence's rows
@@ -450,8 +451,8 @@ __global__ __launch_bounds__(PF32_THREADS) void attn_prefill_f32_kernel(
   __shared__ __attribute__((aligned(16))) float ldsV[HD * PAGE];
   const int seq = blockIdx.y, kvh = blockIdx.z;
   const int q0 = cu_q[seq], qn = cu_q[seq + 1] - q0;
-  const int linear = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
-  const int tile = (linear >> 8) & 1 ? blockIdx.x : gridDim.x - 1 - blockIdx.x;     // as attn_prefill_kernel
+  const int linear0 = gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const int tile = (linear0 >> 8) & 1 ? blockIdx.x : gridDim.x - 1 - blockIdx.x;     // as attn_prefill_kernel
   const int t0 = tile * bq;
   if (t0 >= qn) return;
   const int t1 = t0 + bq < qn ? t0 + bq : qn;

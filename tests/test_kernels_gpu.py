@@ -443,6 +443,10 @@ ATT_CASES = [  # H, KV, hd, window, [(cached length, rows of this step)]
     (6, 2, 48, 0, [(100, 100), (31, 7)]),
     (40, 2, 32, 0, [(90, 90)]),
     (4, 4, 80, 0, [(130, 130), (5, 5)]),
+    # rows of tiles (one sequence, one kv head) that do not divide the 256 blocks of a round of the chip
+    (32, 4, 32, 0, [(63, 45), (300, 215), (2, 1), (300, 214), (2, 1)]),
+    (32, 4, 128, 0, [(63, 45), (300, 215), (2, 1), (300, 214), (2, 1)]),
+    (6, 3, 16, 0, [(700, 700), (650, 650), (90, 90), (300, 300), (641, 641), (64, 64), (200, 77), (690, 690)]),
 ]
 
 
