@@ -17,8 +17,8 @@
 #define SAMP_THREADS 1024
 #define SAMP_WAVES (SAMP_THREADS / WAVE)
 
-__device__ __forceinline__ uint32_t order_key(float f) {   // larger float <-> larger key
-  const uint32_t u = __float_as_uint(f);
+__device__ __forceinline__ uint32_t order_key(float f) {   // larger float <-> larger key; -0 and +0 are one value
+  const uint32_t u = __float_as_uint(f + 0.0f);              // -0 + 0 = +0
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 

@@ -670,6 +670,9 @@ def test_sample_top_k_in_awkward_rows():
     r = torch.randn(v, generator=g)
     r[5::7] = 2.5                             # ties inside the kept set and at its edge
     rows.append((r, dict(temp=0.9, top_k=300, top_p=0.8)))
+    r = torch.tensor([-0., -0., 0.1, -0., -0.25, -0.25, -0., 0., -0.25, 0., 0.])     # -0 and +0 are one value, tied at the cut
+    rows.append((r, dict(temp=0.3, top_k=40, top_p=0.5, min_p=0.2)))
+    rows.append((torch.cat([r, torch.full((3000,), -5.0)]), dict(temp=0.3, top_p=0.5)))
     for logits, c in rows:
         for u in (0.00137, 0.2031, 0.5531, 0.8973, 0.99951):       # no multiples of 1/1300: the equal values' edges
             got = _sample(logits[None], c["temp"], c.get("top_k", 0), c.get("top_p", 1.0), c.get("min_p", 0.0), u=u)[0]
