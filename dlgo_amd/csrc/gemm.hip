@@ -528,6 +528,8 @@ static int auto_splits(int N, int Tn, int nk_all, long long part_elems) {
     if (small <= 64 && nk_all >= 32) {
       splits = (int)(256 / small);
       if (splits > nk_all / 8) splits = nk_all / 8;
+    } else if (small <= 128 && nk_all >= 32) {
+      splits = 2;                                             // half the units would idle otherwise
     }
   } else if (small <= 256 && nk_all >= 128) {
     splits = (int)(512 / small);
