@@ -13,6 +13,7 @@
 // cut are all kept (the reference's unstable sort keeps some of them), and a
 // masked token is never drawn, not even for a uniform number of exactly 0.
 #include "common.h"
+#include <stddef.h>
 
 #define SAMP_THREADS 1024
 #define SAMP_WAVES (SAMP_THREADS / WAVE)
@@ -242,7 +243,8 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
   __shared__ float red[SAMP_WAVES];
   __shared__ SampleSmall S;
   __shared__ int hist[256];
-  __shared__ int chosen, bstar;
+  __shared__ int chosen, bstar, cut_bin;
+  __shared__ unsigned long long cut_before;
   float* scan = S.scan;
   const int row = blockIdx.x;
   const float* lg = logits + (size_t)row * ld;
@@ -253,7 +255,7 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
     return;
   }
   float* work = work_all + (size_t)row * V;
-  float* e = e_all + (size_t)row * V;
+  (void)e_all;     // scratch of an earlier way of finding the top-p cut; the argument stays for its callers
   const float inv_temp = temp == 1.0f ? 1.0f : 1.0f / temp;
   // temperature for all, then the repetition penalty (which comes first in the pipeline) redone for the few it touches
   const bool vec = (V & 3) == 0 && (ld & 3) == 0 && ((uintptr_t)logits & 15) == 0 && ((uintptr_t)work_all & 15) == 0;
@@ -350,15 +352,61 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
   }
   // top-p: smallest set, by falling probability, whose mass reaches p
   if (tp < 1.0f) {
-    float part = 0.f;
-    for (int i = threadIdx.x; i < V; i += SAMP_THREADS) {
-      const float v = expf(work[i] - top.v);
-      e[i] = v;
-      part += v;
+    // The cut is the largest value tau with mass({x >= tau}) >= p * (all the mass).  Masses are exp(x - max) in fixed
+    // point (units of 2^-32) with 64-bit sums: the order of additions does not matter, so atomic additions in LDS give
+    // the same cut every time.  The cut's distance below the maximum, in steps of the ordered bit pattern, is found
+    // 11, 11 and 10 bits at a time, each time from a histogram of masses: three passes over the row.
+    unsigned long long* hist64 = (unsigned long long*)S.sv;     // 2048 bins: sv, si, se and skey, which lie together
+    unsigned long long* tmp64 = (unsigned long long*)S.cv;      // 1024 sums: cv and ci
+    static_assert(offsetof(SampleSmall, skey) - offsetof(SampleSmall, sv) == 3 * SAMP_CAND * 4 && SAMP_CAND * 16 == 2048 * 8 &&
+                      offsetof(SampleSmall, ci) - offsetof(SampleSmall, cv) == SAMP_CAND * 4 && SAMP_THREADS == 1024,
+                  "the histogram borrows the candidates' arrays");
+    const uint32_t kmax = order_key(top.v);
+    uint32_t prefix = 0;            // the distance's upper bits, as far as they are known
+    unsigned long long need = 0;
+    for (int level = 0; level < 3; ++level) {
+      const int shift = level == 0 ? 21 : (level == 1 ? 10 : 0), bits = level == 2 ? 10 : 11;
+      for (int b = threadIdx.x; b < 2048; b += SAMP_THREADS) hist64[b] = 0;
+      __syncthreads();
+      for_each_element(work, V, vec, [&](int, float x) {
+        const uint32_t dist = kmax - order_key(x);
+        if (level == 0 || (dist >> (shift + bits)) == prefix) {
+          const float ev = expf(x - top.v);
+          if (ev > 0.f) {
+            const unsigned long long m = (unsigned long long)(ev * 4294967296.0f);
+            if (m) atomicAdd(&hist64[(dist >> shift) & ((1u << bits) - 1u)], m);
+          }
+        }
+      });
+      __syncthreads();
+      const unsigned long long a = hist64[2 * threadIdx.x], b = hist64[2 * threadIdx.x + 1];
+      tmp64[threadIdx.x] = a + b;
+      __syncthreads();
+      for (int o = 1; o < SAMP_THREADS; o <<= 1) {      // running sums of the pairs of bins, in order
+        const unsigned long long add = (int)threadIdx.x >= o ? tmp64[threadIdx.x - o] : 0ull;
+        __syncthreads();
+        tmp64[threadIdx.x] += add;
+        __syncthreads();
+      }
+      const unsigned long long incl = tmp64[threadIdx.x], excl = incl - (a + b);
+      if (level == 0) {
+        const unsigned long long total = tmp64[SAMP_THREADS - 1];      // at least 2^32: the maximum's own mass
+        need = (unsigned long long)((double)tp * (double)total);
+        need = need < 1ull ? 1ull : (need > total ? total : need);
+      }
+      if (excl < need && need <= excl + a) {
+        cut_bin = 2 * (int)threadIdx.x;
+        cut_before = excl;
+      } else if (excl + a < need && need <= incl) {
+        cut_bin = 2 * (int)threadIdx.x + 1;
+        cut_before = excl + a;
+      }
+      __syncthreads();
+      prefix = (prefix << bits) | (uint32_t)cut_bin;
+      need -= cut_before;
+      __syncthreads();
     }
-    __syncthreads();
-    const float Z = block_sum_f(part, red);
-    const uint32_t tau = bisect_threshold<false>(work, e, V, tp * Z, red, vec && ((uintptr_t)e_all & 15) == 0);
+    const uint32_t tau = kmax - prefix;
     for (int i = threadIdx.x; i < V; i += SAMP_THREADS)
       if (order_key(work[i]) < tau) work[i] = -INFINITY;
     __syncthreads();
