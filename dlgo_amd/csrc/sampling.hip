@@ -13,7 +13,9 @@
 // cut are all kept (the reference's unstable sort keeps some of them), and a
 // masked token is never drawn, not even for a uniform number of exactly 0.
 #include "common.h"
+#include "sampling.h"
 #include <stddef.h>
+#include <mutex>
 
 #define SAMP_THREADS 1024
 #define SAMP_WAVES (SAMP_THREADS / WAVE)
@@ -515,6 +517,41 @@ extern "C" const char* dlgo_argmax(const float* logits, int ld, int n_rows, int 
   DLGO_REQUIRE(n_rows <= 65535, "argmax: at most 65535 rows at a time");
   DLGO_REQUIRE(partial && partial_bytes >= (long long)n_rows * ARGMAX_CHUNKS * (long long)sizeof(BestIdx), "argmax: scratch too small");
   static_assert(ARGMAX_CHUNKS == WAVE, "the final stage reads one candidate per lane");
+  if (n_rows == 0) return nullptr;
+  hipLaunchKernelGGL(argmax_part_kernel, dim3(ARGMAX_CHUNKS, n_rows), dim3(ARGMAX_THREADS), 0, stream, logits, ld, V, (BestIdx*)partial);
+  DLGO_LAUNCH_CHECK("argmax");
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(n_rows), dim3(WAVE), 0, stream, (const BestIdx*)partial, out);
+  DLGO_LAUNCH_CHECK("argmax");
+  return nullptr;
+}
+
+// The first stage's candidates for dlgo_argmax_noalloc.  In host code this name is only a handle: the array's address
+// on a device comes from hipGetSymbolAddress, once per device, and is what the kernels are given.
+static __device__ __align__(256) unsigned char argmax_scratch[DLGO_ARGMAX_NOALLOC_ROWS * ARGMAX_CHUNKS * sizeof(BestIdx)];
+#define DLGO_MAX_DEVICES 64
+static void* argmax_scratch_ptr[DLGO_MAX_DEVICES];
+static std::mutex argmax_scratch_lock;
+
+extern "C" const char* dlgo_argmax_noalloc(const float* logits, int ld, int n_rows, int V, int32_t* out, hipStream_t stream) {
+  DLGO_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "argmax: bad sizes rows=%d V=%d ld=%d", n_rows, V, ld);
+  DLGO_REQUIRE(n_rows <= DLGO_ARGMAX_NOALLOC_ROWS, "argmax without allocation: at most %d rows at a time, got %d",
+               DLGO_ARGMAX_NOALLOC_ROWS, n_rows);
+  DLGO_REQUIRE(logits && out, "argmax: missing argument");
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  DLGO_REQUIRE(e == hipSuccess, "argmax: hipGetDevice failed: %s", hipGetErrorString(e));
+  DLGO_REQUIRE(dev >= 0 && dev < DLGO_MAX_DEVICES, "argmax: device %d is beyond the %d this library keeps scratch for", dev, DLGO_MAX_DEVICES);
+  void* partial;
+  {
+    std::lock_guard<std::mutex> hold(argmax_scratch_lock);
+    if (!argmax_scratch_ptr[dev]) {      // this device's copy of the array, with this device current
+      void* p = nullptr;
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(argmax_scratch));
+      DLGO_REQUIRE(e == hipSuccess && p, "argmax: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+      argmax_scratch_ptr[dev] = p;
+    }
+    partial = argmax_scratch_ptr[dev];
+  }
   if (n_rows == 0) return nullptr;
   hipLaunchKernelGGL(argmax_part_kernel, dim3(ARGMAX_CHUNKS, n_rows), dim3(ARGMAX_THREADS), 0, stream, logits, ld, V, (BestIdx*)partial);
   DLGO_LAUNCH_CHECK("argmax");
