@@ -1,4 +1,5 @@
 import copy
+import math
 import os
 import sys
 
@@ -78,3 +79,24 @@ def make_folder(raw, seed, path, dtype=None, std=None, norm_jitter=0.0):
     from dlgo_amd.weights import write_random_model
     dt = {None: None, "float32": torch.float32, "bfloat16": torch.bfloat16}[dtype]
     return write_random_model(config_from_dict(raw), seed, str(path), dtype=dt, std=std, norm_jitter=norm_jitter)
+
+
+def llama3_blend_cases():
+    """Constructed configurations whose second pair of a head of size 4 has a chosen wavelength, with the frequency the
+    llama3 recipe must give it: (theta, scaling dict, wanted frequency of pair 1, tolerance).  P0 = 64, low 1, high 4:
+    wavelengths between 16 and 64 are blended with s = (P0/wavelength - low)/(high - low).  Pair 1 of a head of size 4
+    has frequency base^(-1/2), so base = (wavelength / 2 pi)^2 places it."""
+    p0, lo, hi, f = 64.0, 1.0, 4.0, 8.0
+    sc = dict(rope_type="llama3", factor=f, low_freq_factor=lo, high_freq_factor=hi, original_max_position_embeddings=int(p0))
+    cases = []
+    for ratio, weight_of_unscaled in ((2.5, 0.5), (1.75, 0.25), (3.25, 0.75)):      # P0/wavelength -> s
+        lam = p0 / ratio
+        th = 2.0 * math.pi / lam
+        cases.append(((lam / (2.0 * math.pi)) ** 2, sc, th * ((1.0 - weight_of_unscaled) / f + weight_of_unscaled), 1e-12))
+    # just inside either edge of the blend: close to the regime next to it
+    for lam, factor in ((p0 / hi * (1 + 1e-7), 1.0), (p0 / lo * (1 - 1e-7), 1.0 / f)):
+        cases.append(((lam / (2.0 * math.pi)) ** 2, sc, 2.0 * math.pi / lam * factor, 1e-5))
+    # just outside: exactly the regime
+    for lam, factor in ((p0 / hi * (1 - 1e-7), 1.0), (p0 / lo * (1 + 1e-7), 1.0 / f)):
+        cases.append(((lam / (2.0 * math.pi)) ** 2, sc, 2.0 * math.pi / lam * factor, 1e-14))
+    return cases

@@ -204,3 +204,20 @@ def test_load_state_checks_too(tiny_a):
         raw = dict(tiny_a)
         del raw["initializer_range"]
         random_tensors(config_from_dict(raw), 0)
+
+
+def test_rotary_frequencies_blend_on_constructed_wavelengths():
+    """The product's llama3 recipe on wavelengths placed at s = 1/2, 1/4, 3/4 and at both edges of the blend (the same
+    cases as the plain implementation's): exchanged weights, a constant half or a geometric blend each fail one of them."""
+    import math
+    from conftest import llama3_blend_cases
+    from dlgo_amd.config import config_from_dict
+    from dlgo_amd.parts import rotary_frequencies
+    for theta, sc, want, tol in llama3_blend_cases():
+        cfg = config_from_dict(dict(TINY_A, head_dim=4, hidden_size=16, rope_theta=theta, rope_scaling=sc, max_position_embeddings=256))
+        got = rotary_frequencies(cfg.head_dim, cfg.rope_theta, cfg.rope_scaling)
+        assert got[0] == 1.0
+        assert math.isclose(got[1], want, rel_tol=tol), (theta, got[1], want)
+    # no scaling block, and a factor of one, leave the plain frequencies
+    cfg = config_from_dict(dict(TINY_A))
+    assert list(rotary_frequencies(16, 10000.0, None)) == [1.0 / math.pow(10000.0, 2.0 * i / 16) for i in range(8)]

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 
 import plain_llama as plain
-from conftest import TINY_A, TINY_B
+from conftest import TINY_A, TINY_B, llama3_blend_cases
 
 
 # -- RMSNorm -------------------------------------------------------------------
@@ -86,13 +86,16 @@ def test_llama3_scaling_invariants():
     b64, s64 = plain.rope_inv_freq(64, 500000.0), plain.rope_inv_freq(64, 500000.0, big)
     assert np.array_equal(s64[:15], b64[:15]) and np.allclose(s64[18:], b64[18:] / 32)
     assert all(b64[i] / 32 < s64[i] < b64[i] for i in (15, 16, 17))
-    # continuity at both edges: a wavelength just inside the blend is close to its neighbour regime
-    p0, lo, hi, f = 8192.0, 1.0, 4.0, 32.0
-    for lam, want_ratio in ((p0 / hi * (1 + 1e-9), 1.0), (p0 / lo * (1 - 1e-9), 1 / f)):
-        th = 2 * math.pi / lam
-        s = (p0 / lam - lo) / (hi - lo)
-        assert math.isclose(((1 - s) * th / f + s * th) / th, want_ratio, rel_tol=1e-6)
 
+
+def test_llama3_blend_on_constructed_wavelengths():
+    """The blend itself, through the implementation: s = 1/2, 1/4, 3/4 exactly and both edges.  A blend with s and 1-s
+    exchanged fails the quarter points and the edges, a constant half fails them too, and a geometric blend
+    (theta * f^-(1-s)) fails the midpoint."""
+    for theta, sc, want, tol in llama3_blend_cases():
+        got = plain.rope_inv_freq(4, theta, sc)
+        assert got[0] == 1.0                                  # wavelength 2 pi: far below P0/high, kept bit for bit
+        assert math.isclose(got[1], want, rel_tol=tol), (theta, got[1], want)
 
 # -- attention -----------------------------------------------------------------
 def test_attention_reference_vectors():
