@@ -39,6 +39,8 @@
 
 static_assert(HEAD_DIM % 16 == 0 && HEAD_DIM >= 16 && HEAD_DIM <= 512, "head sizes come in steps of 16, up to 512");
 
+// true float32 from here (exact_begin.h): the kernel for any dtype and shape, exact in both
+#include "exact_begin.h"
 template <typename T> struct Vec16;   // a 16-byte piece of a row, as floats
 template <> struct Vec16<float> {
   static constexpr int E = 4;
@@ -156,6 +158,11 @@ __global__ __launch_bounds__(WAVE) void attn_rows_kernel(const T* __restrict__ q
   }
 }
 
+#include "exact_end.h"
+
+// How the partial results of several blocks are weighted when they are merged: e^x for the float32 kernels' natural
+// exponents (defined among them), 2^x for the bfloat16 kernels' base-2 ones.
+template <bool NATURAL> __device__ __forceinline__ float merge_weight(float x);
 
 // ----------------------------------------------------------------------------
 // bfloat16 MFMA kernels
@@ -174,6 +181,7 @@ __device__ __forceinline__ bf16x8_t join_bf16x8(const uint2& lo, const uint2& hi
   return x.v;
 }
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+template <> __device__ __forceinline__ float merge_weight<false>(float x) { return fast_exp2(x); }
 
 #define PF_THREADS 256   // threads of a team
 #define PF_ROWS 128      // query rows (token x head of the group) per block
@@ -438,6 +446,8 @@ __global__ __launch_bounds__(PF_THREADS* PF_TEAMS) __attribute__((amdgpu_waves_p
 // Prefill in float32, for head sizes up to 128: a thread owns a query row (token x head of the group, 128 rows a block),
 // a page of keys and of transposed values sits in LDS, and every product is an FMA on float32 with exact expf; the
 // keys are taken 16 at a time so that the scores stay in registers.  grid and bq as attn_prefill_kernel.
+#include "exact_begin.h"      // the float32 prompt kernel: true float32
+template <> __device__ __forceinline__ float merge_weight<true>(float x) { return expf(x); }
 #if HEAD_DIM <= 128
 #define PF32_THREADS 128
 __global__ __launch_bounds__(PF32_THREADS) void attn_prefill_f32_kernel(
@@ -555,6 +565,7 @@ __global__ __launch_bounds__(PF32_THREADS) void attn_prefill_f32_kernel(
   for (int d = 0; d < HD; d += 4) *(float4*)(orow + d) = make_float4(o[d] * inv, o[d + 1] * inv, o[d + 2] * inv, o[d + 3] * inv);
 }
 #endif
+#include "exact_end.h"
 
 // Rotation of 8 consecutive elements d0..d0+7 of one head vector (bfloat16) at a position whose cos/sin rows are
 // given, as rope_kv.hip does it: split-half pairs (d, d + rot/2) or interleaved pairs (2i, 2i+1); elements from
@@ -831,6 +842,7 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_kernel(
 // k steps (the same elements on the key's and the query's side).  The scores land where the second product wants
 // them: a lane's score of key 16 t + 4 G + v is the operand of k step (t, v), whose value operand is element v of the
 // lane's 16 bytes of a transposed value row.
+#include "exact_begin.h"      // the float32 kernel for steps of single tokens, and the merge of partial results
 #if HEAD_DIM <= 128
 template <int NWV>
 __global__ __launch_bounds__(NWV* WAVE) void attn_decode_f32_kernel(
@@ -1041,14 +1053,14 @@ __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restr
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       if (c0 + i <= s1) M_new = fmaxf(M_new, ms[i]);
-    const float keep = NATURAL ? expf(M - M_new) : fast_exp2(M - M_new);       // 0 at the first round (M = -inf, M_new finite: every split given pages holds a key)
+    const float keep = merge_weight<NATURAL>(M - M_new);       // 0 at the first round (M = -inf, M_new finite: every split given pages holds a key)
     L *= keep;
 #pragma unroll
     for (int e = 0; e < ND; ++e) acc[e] *= keep;
 #pragma unroll
     for (int i = 0; i < 8; ++i)
       if (c0 + i <= s1) {
-        const float w = NATURAL ? expf(ms[i] - M_new) : fast_exp2(ms[i] - M_new);
+        const float w = merge_weight<NATURAL>(ms[i] - M_new);
         L = fmaf(w, ls[i], L);
 #pragma unroll
         for (int e = 0; e < ND; ++e) acc[e] = fmaf(w, v[i][e], acc[e]);
@@ -1060,6 +1072,8 @@ __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restr
   for (int e = 0; e < ND; ++e)
     if (e * WAVE + lane < HD) Elem<TO>::store(out + (size_t)seq * ldo + (size_t)head * HD + e * WAVE + lane, acc[e] * inv);
 }
+
+#include "exact_end.h"
 
 extern "C" int dlgo_attention_head_dim() { return HEAD_DIM; }
 

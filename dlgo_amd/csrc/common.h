@@ -36,11 +36,17 @@ template <> struct Elem<float> {
   static constexpr int code = DLGO_DTYPE_F32;
   __device__ static __forceinline__ float load(const float* p) { return *p; }
   __device__ static __forceinline__ void store(float* p, float v) { *p = v; }
+  // two and four consecutive elements at once; p is aligned to what is stored
+  __device__ static __forceinline__ void store2(float* p, float a, float b) { *(float2*)p = make_float2(a, b); }
+  __device__ static __forceinline__ void store4(float* p, float a, float b, float c, float d) { *(float4*)p = make_float4(a, b, c, d); }
 };
 template <> struct Elem<bf16_t> {
   static constexpr int code = DLGO_DTYPE_BF16;
   __device__ static __forceinline__ float load(const bf16_t* p) { return bf16_to_f32(*p); }
   __device__ static __forceinline__ void store(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+  __device__ static __forceinline__ uint32_t pair(float a, float b) { return (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16); }
+  __device__ static __forceinline__ void store2(bf16_t* p, float a, float b) { *(uint32_t*)p = pair(a, b); }
+  __device__ static __forceinline__ void store4(bf16_t* p, float a, float b, float c, float d) { *(uint2*)p = make_uint2(pair(a, b), pair(c, d)); }
 };
 
 __device__ __forceinline__ float wave_sum(float v) {

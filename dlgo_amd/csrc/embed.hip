@@ -4,6 +4,8 @@
 // error of an id out of range (models/llm/forward.go:132-135); here the host
 // rejects such ids before the launch and the kernel clamps so that it cannot fault.
 #include "common.h"
+// everything here is float32 arithmetic whatever the storage type: no approximation can be named (exact_begin.h)
+#include "exact_begin.h"
 
 template <typename T>
 __global__ __launch_bounds__(256) void embed_kernel(const T* __restrict__ table, const int32_t* __restrict__ ids,
@@ -29,3 +31,5 @@ extern "C" const char* dlgo_embed(const void* table, int dtype, const int32_t* i
   DLGO_LAUNCH_CHECK("embed");
   return nullptr;
 }
+
+#include "exact_end.h"

@@ -18,6 +18,7 @@
 #include "gemm_common.h"
 
 template <typename T> struct Mma;
+#if DLGO_ELEM == DLGO_DTYPE_BF16
 template <> struct Mma<bf16_t> {
   // 16 bytes = 8 bfloat16 of k per lane: one 32x32x16 MFMA
   static __device__ __forceinline__ void run(const uint4& a, const uint4& b, f32x16_t& c) {
@@ -27,6 +28,7 @@ template <> struct Mma<bf16_t> {
     c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ua.v, ub.v, c, 0, 0, 0);
   }
 };
+#endif
 template <> struct Mma<float> {
   // 16 bytes = 4 float32 of k per lane: four 32x32x2 MFMAs
   static __device__ __forceinline__ void run(const uint4& a, const uint4& b, f32x16_t& c) {
@@ -310,13 +312,9 @@ __global__ __launch_bounds__(WN* WT* WAVE) void gemm_direct_kernel(const T* __re
             const int nl = wn * (BN / WN) + i * 32 + 8 * q + 4 * (lane >> 5);     // four consecutive n of that token
             const float v0 = acc[i][j][4 * q], v1 = acc[i][j][4 * q + 1], v2 = acc[i][j][4 * q + 2], v3 = acc[i][j][4 * q + 3];
             if (EPI == EPI_SWIGLU) {
-              *(uint32_t*)(lds + tl * OROW + nl) =
-                  (uint32_t)f32_to_bf16(silu_f<T>(v0) * v1) | ((uint32_t)f32_to_bf16(silu_f<T>(v2) * v3) << 16);
+              Elem<T>::store2((T*)(lds + tl * OROW + nl), silu_f<T>(v0) * v1, silu_f<T>(v2) * v3);
             } else {
-              uint2 p;
-              p.x = (uint32_t)f32_to_bf16(v0) | ((uint32_t)f32_to_bf16(v1) << 16);
-              p.y = (uint32_t)f32_to_bf16(v2) | ((uint32_t)f32_to_bf16(v3) << 16);
-              *(uint2*)(lds + tl * OROW + nl * 2) = p;
+              Elem<T>::store4((T*)(lds + tl * OROW + nl * 2), v0, v1, v2, v3);
             }
           }
       __syncthreads();
@@ -689,3 +687,7 @@ extern "C" const char* dlgo_gemm_accum_norm(const void* W, const void* X, float*
   DLGO_LAUNCH_CHECK("gemm_accum_norm");
   return nullptr;
 }
+
+#if DLGO_ELEM == DLGO_DTYPE_F32
+#include "exact_end.h"
+#endif

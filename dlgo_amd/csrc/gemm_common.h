@@ -16,6 +16,13 @@ typedef bf16_t elem_t;
 #error "DLGO_ELEM must be 0 or 1"
 #endif
 
+// The float32 build computes in true float32 from here to the end of the file that includes this: no reduced-precision
+// matrix instruction, no hardware approximation and no bfloat16 type can be named in it (exact_begin.h).
+#if DLGO_ELEM == DLGO_DTYPE_F32
+#define DLGO_EXACT_NO_BF16 1
+#include "exact_begin.h"
+#endif
+
 enum { EPI_STORE = 0, EPI_ACCUM_F32 = 1, EPI_SWIGLU = 2, EPI_STORE_F32 = 3 };
 
 // silu(z) = z / (1 + e^-z).  For a float32 result: the library's exponential and a true division.  For a bfloat16
@@ -23,9 +30,11 @@ enum { EPI_STORE = 0, EPI_ACCUM_F32 = 1, EPI_SWIGLU = 2, EPI_STORE_F32 = 3 };
 // of what bfloat16 keeps; a quarter of the instructions, which a prompt's gate/up product feels.
 template <typename T> __device__ __forceinline__ float silu_f(float z);
 template <> __device__ __forceinline__ float silu_f<float>(float z) { return z / (1.0f + expf(-z)); }
+#if DLGO_ELEM == DLGO_DTYPE_BF16
 template <> __device__ __forceinline__ float silu_f<bf16_t>(float z) {
   return z * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(z * -1.44269504088896341f));
 }
+#endif
 
 // Four consecutive outputs n..n+3 of token t.
 template <typename T, int EPI>
@@ -36,14 +45,7 @@ __device__ __forceinline__ void epilogue4(void* __restrict__ Y, int ldy, int N, 
   if (EPI == EPI_STORE) {
     T* y = (T*)Y + (size_t)t * ldy + n;
     if (full && (ldy & 3) == 0 && ((uintptr_t)y & (4 * sizeof(T) - 1)) == 0) {
-      if (sizeof(T) == 4) {
-        *(float4*)y = make_float4(v0, v1, v2, v3);
-      } else {
-        uint2 p;
-        p.x = (uint32_t)f32_to_bf16(v0) | ((uint32_t)f32_to_bf16(v1) << 16);
-        p.y = (uint32_t)f32_to_bf16(v2) | ((uint32_t)f32_to_bf16(v3) << 16);
-        *(uint2*)y = p;
-      }
+      Elem<T>::store4(y, v0, v1, v2, v3);
     } else {
       const float v[4] = {v0, v1, v2, v3};
       for (int r = 0; r < 4 && n + r < N; ++r) Elem<T>::store(y + r, v[r]);
@@ -67,8 +69,7 @@ __device__ __forceinline__ void epilogue4(void* __restrict__ Y, int ldy, int N, 
   } else {   // EPI_SWIGLU: rows (n, n+1) and (n+2, n+3) are (gate, up) pairs; N is even
     T* y = (T*)Y + (size_t)t * ldy + (n >> 1);
     if (n + 3 < N && (ldy & 1) == 0 && ((uintptr_t)y & (2 * sizeof(T) - 1)) == 0) {     // both halves at once
-      if (sizeof(T) == 4) *(float2*)y = make_float2(silu_f<T>(v0) * v1, silu_f<T>(v2) * v3);
-      else *(uint32_t*)y = (uint32_t)f32_to_bf16(silu_f<T>(v0) * v1) | ((uint32_t)f32_to_bf16(silu_f<T>(v2) * v3) << 16);
+      Elem<T>::store2(y, silu_f<T>(v0) * v1, silu_f<T>(v2) * v3);
     } else {
       Elem<T>::store(y, silu_f<T>(v0) * v1);
       if (n + 3 < N) Elem<T>::store(y + 1, silu_f<T>(v2) * v3);

@@ -15,6 +15,7 @@
 // weight-streaming kernel for up to 8 tokens
 // ----------------------------------------------------------------------------
 template <typename T> struct Chunk;
+#if DLGO_ELEM == DLGO_DTYPE_BF16
 template <> struct Chunk<bf16_t> {
   static constexpr int E = 8;
   static __device__ __forceinline__ void unpack(const uint4& u, float* f) {
@@ -28,6 +29,7 @@ template <> struct Chunk<bf16_t> {
     f[7] = __uint_as_float(u.w & 0xffff0000u);
   }
 };
+#endif
 template <> struct Chunk<float> {
   static constexpr int E = 4;
   static __device__ __forceinline__ void unpack(const uint4& u, float* f) {
@@ -106,6 +108,7 @@ __global__ __launch_bounds__(GEMV_WAVES* WAVE) void gemv_kernel(const T* __restr
 // writing the normed rows: the column operand is X[t,k] * norm_w[k], the sum of squares of each token is
 // gathered on the way, and 1/sqrt(mean + eps) multiplies the finished sums (it is a scalar per token).
 template <typename T> struct Mma16;
+#if DLGO_ELEM == DLGO_DTYPE_BF16
 template <> struct Mma16<bf16_t> {
   static __device__ __forceinline__ void run(const uint4& a, const uint4& b, f32x4_t& c) {
     union { uint4 u; bf16x8_t v; } ua, ub;
@@ -121,6 +124,7 @@ template <> struct Mma16<bf16_t> {
     return x.u;
   }
 };
+#endif
 template <> struct Mma16<float> {
   static __device__ __forceinline__ void run(const uint4& a, const uint4& b, f32x4_t& c) {
     c = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
@@ -363,3 +367,7 @@ extern "C" const char* dlgo_gemm_rmsnorm(const void* W, const float* X, const fl
   DLGO_LAUNCH_CHECK("gemm_rmsnorm");
   return nullptr;
 }
+
+#if DLGO_ELEM == DLGO_DTYPE_F32
+#include "exact_end.h"
+#endif

@@ -6,6 +6,8 @@
 // batch it came in.  An optional row index gathers rows first (the final norm
 // runs on the rows whose logits are wanted only, models/llm/forward_batch.go:222-229).
 #include "common.h"
+// everything here is float32 arithmetic whatever the storage type: no approximation can be named (exact_begin.h)
+#include "exact_begin.h"
 
 // A thread keeps its part of the row (up to HOLD pieces of four floats) in registers between the sum and the write,
 // so that a row is read once; longer rows are read a second time.
@@ -91,3 +93,5 @@ extern "C" const char* dlgo_rmsnorm(const float* x, const int32_t* rows, const f
   DLGO_LAUNCH_CHECK("rmsnorm");
   return nullptr;
 }
+
+#include "exact_end.h"

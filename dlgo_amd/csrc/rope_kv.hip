@@ -12,6 +12,8 @@
 // transposed [kv_head][hd][token], so that both attention products read
 // 16-byte pieces along their reduction axis.
 #include "common.h"
+// everything here is float32 arithmetic whatever the storage type: no approximation can be named (exact_begin.h)
+#include "exact_begin.h"
 
 #define PAGE 64
 
@@ -272,3 +274,5 @@ extern "C" const char* dlgo_rope_kv(void* qkv, int dtype, int n_tokens, int ld, 
   DLGO_LAUNCH_CHECK("rope_kv");
   return nullptr;
 }
+
+#include "exact_end.h"

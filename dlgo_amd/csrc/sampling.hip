@@ -16,6 +16,8 @@
 #include "sampling.h"
 #include <stddef.h>
 #include <mutex>
+// everything here is float32 arithmetic whatever the storage type: no approximation can be named (exact_begin.h)
+#include "exact_begin.h"
 
 #define SAMP_THREADS 1024
 #define SAMP_WAVES (SAMP_THREADS / WAVE)
@@ -578,3 +580,5 @@ extern "C" const char* dlgo_sample(const float* logits, int ld, int n_rows, int 
   DLGO_LAUNCH_CHECK("sample");
   return nullptr;
 }
+
+#include "exact_end.h"

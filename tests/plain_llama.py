@@ -199,10 +199,11 @@ def block(x, positions, w, prefix, cfg, inv_freq, window=None):
     return h + f
 
 
-def forward(cfg, w, tokens, start_pos=0):
+def forward(cfg, w, tokens, start_pos=0, rows=None):
     """Logits [T, V] of one whole sequence (models/llm/forward.go:123-204):
     embedding row, L blocks, final norm, output matrix (the embedding table
-    when tied, models/llm/loader.go:74-76)."""
+    when tied, models/llm/loader.go:74-76).  rows: the positions whose logits
+    are wanted (all of them if None); the blocks always see the whole sequence."""
     H = cfg["num_attention_heads"]
     hd = cfg.get("head_dim", cfg["hidden_size"] // H)
     inv_freq = rope_inv_freq(hd, cfg["rope_theta"], cfg.get("rope_scaling"))
@@ -214,6 +215,8 @@ def forward(cfg, w, tokens, start_pos=0):
     positions = [start_pos + i for i in range(len(tokens))]
     for l in range(cfg["num_hidden_layers"]):
         x = block(x, positions, w, f"model.layers.{l}.", cfg, inv_freq)
+    if rows is not None:
+        x = x[list(rows)]
     x = rmsnorm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
     out_w = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
     return x @ out_w.T
