@@ -6,7 +6,9 @@
 A step is one decode step of the whole batch: greedy choice of the next tokens on
 the device, the step function on those tokens, and the ids' return to the host
 (what the generation loop does per step, in its order).  Random weights, seeded
-uniform-random token ids, no stop tokens.  Prints ONE JSON line.
+uniform-random token ids, no stop tokens.  The K timed steps run as five regions,
+each between two waits for the device; the figures are the median region's.
+Prints ONE JSON line.
 
 Peaks used for the fractions (MI355X, published): HBM 8 TB/s; dense MFMA bf16
 2.5 PFLOP/s, fp32 157.3 TFLOP/s.
@@ -37,6 +39,7 @@ SHAPES = {
 }
 CONTEXT = 4096
 PROMPT = 2048
+REGIONS = 5        # timed regions of a decode measurement; the median one is reported
 HBM_PEAK = 8.0e12
 FLOP_PEAK = {"bf16": 2.5e15, "fp32": 157.3e12}
 
@@ -160,7 +163,7 @@ def main() -> int:
         prompts = [rng.integers(0, cfg.vocab_size, size=PROMPT).tolist() for _ in range(batch)]
         slots = eng.open(batch)
         logits = eng.step([Entry(s, p, [PROMPT - 1]) for s, p in zip(slots, prompts)])
-        # the generation loop's own order (engine/generate.py, _decode_ahead): choose on the device, queue the next
+        # the generation loop's own order (engine/generate.py, _decode_batch): choose on the device, queue the next
         # step with the ids still on the device, then bring the ids of the step before to the host
         state = {"logits": logits}
 
@@ -172,24 +175,30 @@ def main() -> int:
             one()
         torch.cuda.synchronize()
         c0 = eng.length(slots[0])
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            one()
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
+        # exactly `steps` timed steps, in REGIONS regions of (nearly) equal length, each between two waits for the device;
+        # the figure is the median region's time per step
+        n_regions = REGIONS if steps >= REGIONS else 1
+        sizes = [steps // n_regions + (1 if r < steps % n_regions else 0) for r in range(n_regions)]
+        per_step = []
+        for size in sizes:
+            t0 = time.perf_counter()
+            for _ in range(size):
+                one()
+            torch.cuda.synchronize()
+            per_step.append((time.perf_counter() - t0) / size)
         eng.close(slots)
         mean_ctx = c0 + (steps + 1) / 2.0       # keys a step reads per sequence, averaged over the timed steps
-        return dt, mean_ctx
+        return statistics.median(per_step), mean_ctx, per_step
 
-    dt, mean_ctx = decode(args.batch, args.steps, args.warmup)
-    ms_step = dt / args.steps * 1000.0
-    value = args.batch * args.steps / dt
+    step_s, mean_ctx, regions = decode(args.batch, args.steps, args.warmup)
+    ms_step = step_s * 1000.0
+    value = args.batch / step_s
     step_bytes = weight_bytes(cfg, elem) + args.batch * mean_ctx * kv_bytes_per_token(cfg, elem)
-    achieved = step_bytes / (dt / args.steps)
+    achieved = step_bytes / step_s
     points = {}
     for b in batches[1:]:
-        pdt, _ = decode(b, args.point_steps, min(args.warmup, 8))
-        points[f"decode_b{b}"] = round(b * args.point_steps / pdt, 1)
+        p_step, _, _ = decode(b, args.point_steps, min(args.warmup, 8))
+        points[f"decode_b{b}"] = round(b / p_step, 1)
 
     prefill = None
     if not args.no_prefill:
@@ -221,6 +230,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
         "points": points,
+        "regions_ms_per_step": [round(r * 1000.0, 4) for r in regions],
     }
     if prefill is not None:
         line["prefill"] = prefill

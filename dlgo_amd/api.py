@@ -11,8 +11,10 @@ from typing import Callable, List, Optional, Sequence, Union
 
 import torch
 
-from .config import ModelConfig, load_config
-from .engine.engine import Engine
+from .cache import PAGE, tokens_that_fit
+from .config import ModelConfig, build_model, load_config
+from .engine.engine import Engine, EngineError, run_dtype
+from .weights import load_weights
 from .engine.generate import Result, Stats, generate
 from .sampling import GenerateConfig, Option, Sampler, apply_options
 
@@ -33,6 +35,20 @@ class GenerateResult:
     def __str__(self) -> str:
         return (f"{self.tokens_per_sec:.1f} tok/s | prefill: {self.prefill_ms:.0f}ms | gen: {self.generate_ms:.0f}ms | "
                 f"{self.output_tokens} tokens | {self.finish_reason}")
+
+
+@dataclass
+class BenchmarkResult:
+    """dlgo.go:152-168, with the time of every step beside the totals (step_ms[0] is the prompt step)."""
+    tokens: List[int]
+    tokens_per_sec: float
+    prefill_ms: float
+    generate_ms: float
+    total_ms: float
+    prompt_tokens: int
+    output_tokens: int
+    architecture: str
+    step_ms: List[float]
 
 
 class LLM:
@@ -70,9 +86,16 @@ class LLM:
         results, stats = self._run([prompt], opts, on_token=lambda i, t: on_token(t))
         return self._wrap(results[0], stats)
 
-    def benchmark(self, prompt: Prompt, *opts: Option) -> GenerateResult:
-        """A run with separate prefill and generation timings (dlgo.go:93-114)."""
-        return self.generate(prompt, *opts)
+    def benchmark(self, prompt: Prompt, *opts: Option) -> "BenchmarkResult":
+        """A run with separate prefill and generation timings, the whole call's time and the time of every step
+        (dlgo.go:93-114; models/llm/generate.go:227-229,275-282)."""
+        import time
+        t0 = time.perf_counter()
+        results, stats = self._run([prompt], opts)
+        total_ms = (time.perf_counter() - t0) * 1000.0
+        r = results[0]
+        return BenchmarkResult(r.tokens, stats.tokens_per_sec, stats.prefill_ms, stats.generate_ms, total_ms, r.prompt_tokens,
+                               len(r.tokens), self.config.architecture, list(stats.step_ms))
 
     def model_info(self) -> str:
         """dlgo.go:170-185."""
@@ -87,11 +110,21 @@ def load_llm(path: str, max_seq_len: int = 0, dtype: str = "bfloat16", device: s
              max_tokens: Optional[int] = None, **engine_options) -> LLM:
     """Load a model folder (config.json, model.safetensors).  max_seq_len <= 0 or beyond the model's
     context means the model's context (models/llm/generate.go:56-58).  The cache is sized for
-    `max_tokens` tokens over all live sequences (default: max_batch sequences of max_seq_len, at most 2^20)."""
+    `max_tokens` tokens over all live sequences; by default for max_batch sequences of max_seq_len, or for as many
+    tokens as the device's free memory holds once the weights are loaded (a fifth of it stays free), if that is less."""
     config = load_config(path)
     limit = getattr(config, "max_position_embeddings", None)
     ctx = max_seq_len if max_seq_len > 0 and (limit is None or max_seq_len <= limit) else limit
+    if not torch.cuda.is_available():
+        raise EngineError("no HIP device: dlgo_amd runs on an AMD GPU only and has no CPU path")
+    rd = run_dtype(dtype)
+    model = build_model(config)
+    load_weights(model, path, device, rd)
     if max_tokens is None:
-        max_tokens = min(max_batch * ctx, 1 << 20)
-    engine = Engine.from_folder(path, dtype, device, max_tokens=max_tokens, max_ctx=ctx, **engine_options)
+        free, _ = torch.cuda.mem_get_info(torch.device(device))
+        fit = tokens_that_fit(model.unit_needs, rd, free)
+        if fit < PAGE:
+            raise EngineError(f"no device memory left for a cache ({free >> 20} MiB free after the weights)")
+        max_tokens = min(max_batch * ctx, fit)
+    engine = Engine(model, rd, device, max_tokens=max_tokens, max_ctx=ctx, **engine_options)
     return LLM(engine, max_batch)

@@ -1,3 +1,3 @@
-from .cache import PAGE, Cache, CacheError, KVGroup, KVView, OutOfPages, PagePool
+from .cache import PAGE, Cache, CacheError, KVGroup, KVView, OutOfPages, PagePool, kv_bytes_per_token, tokens_that_fit
 
-__all__ = ["PAGE", "Cache", "CacheError", "KVGroup", "KVView", "OutOfPages", "PagePool"]
+__all__ = ["PAGE", "Cache", "CacheError", "KVGroup", "KVView", "OutOfPages", "PagePool", "kv_bytes_per_token", "tokens_that_fit"]

@@ -139,10 +139,13 @@ class Cache:
                     raise CacheError(f"cache unit {u}: unknown need kind {need.kind!r}")
         for spec in specs.values():
             n_pages = self.n_pages
+            per_seq = self.max_pages_per_seq
             if spec.window is not None:
-                per_seq = (spec.window + min(self.max_step_tokens, self.max_ctx) + PAGE - 1) // PAGE + 1
+                per_seq = min(per_seq, (spec.window + min(self.max_step_tokens, self.max_ctx) + PAGE - 1) // PAGE + 1)
                 n_pages = min(n_pages, self.max_slots * per_seq)
-            self.groups.append(KVGroup(spec, n_pages, self.max_slots, self.max_pages_per_seq, dtype, self.device))
+            group = KVGroup(spec, n_pages, self.max_slots, self.max_pages_per_seq, dtype, self.device)
+            group.pages_per_seq = per_seq       # the most pages one sequence holds of this group at any time
+            self.groups.append(group)
 
         self._free_slots = list(range(self.max_slots - 1, -1, -1))
         self._live = np.zeros(self.max_slots, dtype=bool)
@@ -205,12 +208,25 @@ class Cache:
             if new_len > self.max_ctx:
                 return f"slot {slot}: {new_len} tokens exceed the context of {self.max_ctx}"
         for gi, g in enumerate(self.groups):
-            if g.spec.window is not None:
-                continue   # bounded by construction: steps are cut to max_step_tokens
-            need = sum(len(self.pages_wanted(s, n, gi)) for s, n in wants)
+            # a windowed group: a sequence never holds more than its window and the longest piece of a step, because
+            # each piece gives back what no later token sees before the next piece asks for more
+            if g.spec.window is None:
+                need = sum(len(self.pages_wanted(s, n, gi)) for s, n in wants)
+            else:
+                need = sum(min(len(self.pages_wanted(s, n, gi)), max(0, g.pages_per_seq - len(self._held[s][gi]))) for s, n in wants)
             if need > g.pool.n_free:
                 return f"cache full: the step needs {need} more pages of {PAGE} tokens, {g.pool.n_free} of {g.pool.n_pages} are free"
         return None
+
+    def page_demand(self, n_tokens: int) -> Tuple[int, ...]:
+        """Per group: the most pages a sequence that grows to n_tokens holds at any time (a windowed group: its window
+        and the longest step, whatever the length)."""
+        whole = (min(n_tokens, self.max_ctx) + PAGE - 1) // PAGE
+        return tuple(whole if g.spec.window is None else min(whole, g.pages_per_seq) for g in self.groups)
+
+    def free_pages(self) -> Tuple[int, ...]:
+        """Per group: pages that new sequences can still take."""
+        return tuple(g.pool.n_free for g in self.groups)
 
     def reserve(self, wants: Sequence[Tuple[int, int]]) -> None:
         """Make room so that each slot can hold positions below its new length."""
@@ -298,6 +314,23 @@ class Cache:
                 raise CacheError(f"group {gi}: {len(seen)} held + {g.pool.n_free} free != {g.pool.n_pages} pages")
         if len(self._free_slots) + int(self._live.sum()) != self.max_slots or len(set(self._free_slots)) != len(self._free_slots):
             raise CacheError("slot accounting broken")
+
+
+def kv_bytes_per_token(unit_needs: Sequence[Sequence[CacheNeed]], dtype: torch.dtype) -> int:
+    """Bytes of keys and values that one token adds over all cache units (a windowed unit counts like a full one)."""
+    item = torch.empty(0, dtype=dtype).element_size()
+    return sum(2 * need.kv_heads * need.head_dim * item for needs in unit_needs for need in needs if need.kind == "kv")
+
+
+def tokens_that_fit(unit_needs: Sequence[Sequence[CacheNeed]], dtype: torch.dtype, free_bytes: int, keep_free: float = 0.2,
+                    reserve_bytes: int = 2 << 30) -> int:
+    """How many tokens (a whole number of pages) a cache may be sized for when `free_bytes` of device memory are left:
+    a fifth of it and 2 GiB stay free for the step's buffers and the logits."""
+    per_token = kv_bytes_per_token(unit_needs, dtype)
+    budget = int(free_bytes * (1.0 - keep_free)) - reserve_bytes
+    if per_token == 0:
+        return 1 << 20
+    return max(0, budget // (per_token * PAGE)) * PAGE
 
 
 @dataclass

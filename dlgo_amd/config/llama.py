@@ -81,6 +81,7 @@ class LlamaConfig(ModelConfig):
     rope_scaling: Optional[RopeScaling]
     max_position_embeddings: int
     tie_word_embeddings: bool
+    attention_bias: bool
     bos_token_id: Optional[int]
     eos_token_ids: Tuple[int, ...]
     initializer_range: Optional[float]
@@ -130,10 +131,9 @@ class LlamaConfig(ModelConfig):
             else:
                 r.complain(f"eos_token_id: expected a token id or a list of them, found {eos_raw!r}")
 
-        if r.boolean("attention_bias", default=False):
-            r.complain("attention_bias: projections with bias are not part of this architecture here")
+        attention_bias = r.boolean("attention_bias", default=False)
         if r.boolean("mlp_bias", default=False):
-            r.complain("mlp_bias: feed-forward biases are not part of this architecture here")
+            r.complain("mlp_bias: feed-forward biases have no kernel here (the gate/up product ends in SwiGLU directly)")
         act = r.string("hidden_act", default="silu")
         if act is not None and act != "silu":
             r.complain(f"hidden_act: only \"silu\" (SwiGLU) is supported, found {act!r}")
@@ -152,7 +152,7 @@ class LlamaConfig(ModelConfig):
         return cls(architecture=arch, vocab_size=vocab, hidden_size=d, num_hidden_layers=layers,
                    intermediate_size=ffn, num_attention_heads=heads, num_key_value_heads=kv, head_dim=hd,
                    rms_norm_eps=eps, rope_theta=theta, rope_scaling=scaling, max_position_embeddings=max_pos,
-                   tie_word_embeddings=tie, bos_token_id=bos, eos_token_ids=eos,
+                   tie_word_embeddings=tie, attention_bias=bool(attention_bias), bos_token_id=bos, eos_token_ids=eos,
                    initializer_range=init_range, torch_dtype=dtype)
 
     def to_dict(self) -> Dict[str, Any]:
@@ -172,7 +172,7 @@ class LlamaConfig(ModelConfig):
             "rope_scaling": self.rope_scaling.to_dict() if self.rope_scaling else None,
             "max_position_embeddings": self.max_position_embeddings,
             "tie_word_embeddings": self.tie_word_embeddings,
-            "attention_bias": False,
+            "attention_bias": self.attention_bias,
             "mlp_bias": False,
             "torch_dtype": self.torch_dtype,
         }

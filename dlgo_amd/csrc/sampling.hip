@@ -131,10 +131,8 @@ __global__ __launch_bounds__(WAVE) void argmax_final_kernel(const BestIdx* __res
   if (threadIdx.x == 0) out[blockIdx.x] = best.i < 0 ? 0 : best.i;
 }
 
-// Largest key tau with measure({i : key_i >= tau}) >= need, by bisection on the key's bits.
-// COUNT: the measure counts elements (top-k); else it sums e_i (top-p).
-template <bool COUNT>
-__device__ uint32_t bisect_threshold(const float* work, const float* e, int V, float need, float* red, bool vec = false) {
+// Largest key tau with |{i : key_i >= tau}| >= need, by bisection on the key's bits (top-k).
+__device__ uint32_t bisect_threshold(const float* work, int V, float need, float* red, bool vec = false) {
   uint32_t prefix = 0;
   for (int bit = 31; bit >= 0; --bit) {
     const uint32_t cand = prefix | (1u << bit);
@@ -143,15 +141,14 @@ __device__ uint32_t bisect_threshold(const float* work, const float* e, int V, f
 #pragma unroll 4
       for (int i = threadIdx.x; i < V / 4; i += SAMP_THREADS) {
         const float4 w4 = ((const float4*)work)[i];
-        const float4 e4 = COUNT ? make_float4(1.f, 1.f, 1.f, 1.f) : ((const float4*)e)[i];
-        if (order_key(w4.x) >= cand) part += e4.x;
-        if (order_key(w4.y) >= cand) part += e4.y;
-        if (order_key(w4.z) >= cand) part += e4.z;
-        if (order_key(w4.w) >= cand) part += e4.w;
+        if (order_key(w4.x) >= cand) part += 1.0f;
+        if (order_key(w4.y) >= cand) part += 1.0f;
+        if (order_key(w4.z) >= cand) part += 1.0f;
+        if (order_key(w4.w) >= cand) part += 1.0f;
       }
     } else {
       for (int i = threadIdx.x; i < V; i += SAMP_THREADS)
-        if (order_key(work[i]) >= cand) part += COUNT ? 1.0f : e[i];
+        if (order_key(work[i]) >= cand) part += 1.0f;
     }
     const float total = block_sum_f(part, red);
     if (total >= need) prefix = cand;
@@ -236,7 +233,7 @@ __device__ int sample_small(SampleSmall& S, int n, int k, BestIdx top, float tp,
 }
 
 __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __restrict__ logits, int ld, int V,
-                                                              float* __restrict__ work_all, float* __restrict__ e_all,
+                                                              float* __restrict__ work_all,
                                                               const float* __restrict__ temperature,
                                                               const int32_t* __restrict__ top_k, const float* __restrict__ top_p,
                                                               const float* __restrict__ min_p, const float* __restrict__ penalty,
@@ -259,7 +256,6 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
     return;
   }
   float* work = work_all + (size_t)row * V;
-  (void)e_all;     // scratch of an earlier way of finding the top-p cut; the argument stays for its callers
   const float inv_temp = temp == 1.0f ? 1.0f : 1.0f / temp;
   // temperature for all, then the repetition penalty (which comes first in the pipeline) redone for the few it touches
   const bool vec = (V & 3) == 0 && (ld & 3) == 0 && ((uintptr_t)logits & 15) == 0 && ((uintptr_t)work_all & 15) == 0;
@@ -349,7 +345,7 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
       return;
     }
     // many equal values at the cut, or the k-th value far below the maximum: the cut by bisection over the whole row
-    const uint32_t tau = bisect_threshold<true>(work, nullptr, V, (float)k, red, vec);
+    const uint32_t tau = bisect_threshold(work, V, (float)k, red, vec);
     for (int i = threadIdx.x; i < V; i += SAMP_THREADS)
       if (order_key(work[i]) < tau) work[i] = -INFINITY;
     __syncthreads();
@@ -562,20 +558,20 @@ extern "C" const char* dlgo_argmax_noalloc(const float* logits, int ld, int n_ro
   return nullptr;
 }
 
-// work and e: [n_rows, V] float32 scratch.  recent: a table of token ids with n_recent columns.  Without counts, row r of
+// work: [n_rows, V] float32 scratch.  recent: a table of token ids with n_recent columns.  Without counts, row r of
 // it holds row r's recent tokens, -1 where empty.  With recent_rows and counts, row recent_rows[r] of it is a ring of the
 // last tokens chosen for that key, counts[key] the number chosen so far; the kernel adds the token it chooses.
-extern "C" const char* dlgo_sample(const float* logits, int ld, int n_rows, int V, float* work, float* e,
+extern "C" const char* dlgo_sample(const float* logits, int ld, int n_rows, int V, float* work,
                                    const float* temperature, const int32_t* top_k, const float* top_p, const float* min_p,
                                    const float* penalty, int32_t* recent, int n_recent, const int32_t* recent_rows,
                                    int32_t* counts, const float* uniform, int32_t* out, hipStream_t stream) {
   DLGO_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "sample: bad sizes rows=%d V=%d ld=%d", n_rows, V, ld);
   DLGO_REQUIRE(n_recent >= 0 && n_recent <= SAMP_THREADS, "sample: at most %d recent tokens, got %d", SAMP_THREADS, n_recent);
-  DLGO_REQUIRE(work && e && temperature && top_k && top_p && min_p && penalty && uniform && out, "sample: missing argument");
+  DLGO_REQUIRE(work && temperature && top_k && top_p && min_p && penalty && uniform && out, "sample: missing argument");
   DLGO_REQUIRE(n_recent == 0 || recent, "sample: recent tokens missing");
   DLGO_REQUIRE((recent_rows == nullptr) == (counts == nullptr), "sample: a ring of recent tokens needs both its rows and its counts");
   if (n_rows == 0) return nullptr;
-  hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMP_THREADS), 0, stream, logits, ld, V, work, e, temperature, top_k, top_p,
+  hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMP_THREADS), 0, stream, logits, ld, V, work, temperature, top_k, top_p,
                      min_p, penalty, recent, n_recent, recent_rows, counts, uniform, out);
   DLGO_LAUNCH_CHECK("sample");
   return nullptr;

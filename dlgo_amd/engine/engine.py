@@ -96,7 +96,10 @@ class Engine:
         self.workspace = Workspace(self.device, self.max_step_tokens)
         model.prepare(self.max_ctx, self.device)
         self.vocab = model.vocab
-        self.use_graphs = use_graphs
+        # a step is recorded only if every part says its launches depend on nothing but device arrays (Part.graph_safe)
+        unsafe = [name for name, part in model.named_parts() if not getattr(part, "graph_safe", True)]
+        self.use_graphs = use_graphs and not unsafe
+        self.eager_because = unsafe
         self.graph_max_batch = min(graph_max_batch, self.max_step_tokens)
         self._graphs: Dict[int, _Graph] = {}
         self._graph_seen: Dict[int, int] = {}
@@ -146,10 +149,14 @@ class Engine:
     def free_slots(self) -> int:
         return self.cache.n_free_slots
 
-    def free_pages(self) -> int:
-        """Pages (of 64 tokens) that new sequences can still take."""
-        full = [g.pool.n_free for g in self.cache.groups if g.spec.window is None]
-        return min(full) if full else self.cache.n_pages
+    def free_pages(self) -> Tuple[int, ...]:
+        """Pages (of 64 tokens) that new sequences can still take, for each storage group of the cache (a model
+        without keys and values has none)."""
+        return self.cache.free_pages()
+
+    def page_demand(self, n_tokens: int) -> Tuple[int, ...]:
+        """For each storage group: the most pages a sequence that grows to n_tokens holds at any time."""
+        return self.cache.page_demand(n_tokens)
 
     # -- uploads -----------------------------------------------------------------
     def _stage(self, n_ints: int) -> torch.Tensor:
@@ -224,10 +231,11 @@ class Engine:
             raise EngineError(f"step: {why}")
         self.steps_run += 1
 
-        if (sink is None and len(entries) <= self.graph_max_batch
+        if (sink is None
                 and all(n == 1 for n in q_lens) and all(list(e.want) == [0] for e in entries)):
             self.steps_run -= 1
-            return self.decode([e.slot for e in entries], tokens, checked=True)
+            # decode() hands out a view of a buffer that the next step overwrites; a step's result is the caller's to keep
+            return self.decode([e.slot for e in entries], tokens, checked=True).clone()
 
         # wanted rows: (output row, flat row), in output order
         cu = np.concatenate([[0], np.cumsum(q_lens)])
@@ -306,15 +314,22 @@ class Engine:
         }
 
     def decode(self, slots: Sequence[int], tokens, checked: bool = False) -> torch.Tensor:
-        """One token for each of `slots`, logits [len(slots), vocab] for each (a view that the next decode
+        """One token for each of `slots`, logits [len(slots), vocab] for each (a view that the next decode or step
         overwrites).  `tokens` are ids on the host, or an int32 tensor on the device in the order of `slots`
         (the sampler's output: the ids need not come to the host before the next step starts)."""
         b = len(slots)
+        if b > self.graph_max_batch:
+            # more sequences than the fixed arrays of a recorded step hold: in runs of that many, into a buffer of this call
+            out = torch.empty((b, self.vocab), dtype=torch.float32, device=self.device)
+            for c0 in range(0, b, self.graph_max_batch):
+                c1 = min(b, c0 + self.graph_max_batch)
+                out[c0:c1].copy_(self.decode(slots[c0:c1], tokens[c0:c1], checked))
+            return out
         slot_arr = np.asarray(slots, dtype=np.int64)
         on_device = isinstance(tokens, torch.Tensor)
         if not checked:
-            if b < 1 or b > self.graph_max_batch:
-                raise EngineError(f"decode: between 1 and {self.graph_max_batch} sequences, got {b}")
+            if b < 1:
+                raise EngineError("decode: no sequences")
             if len(set(slots)) != b or slot_arr.min() < 0 or slot_arr.max() >= self.cache.max_slots \
                     or not self.cache._live[slot_arr].all():
                 raise EngineError("decode: slots must be distinct and in use")

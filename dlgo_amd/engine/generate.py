@@ -12,17 +12,20 @@ once and gives its slot back; when a batch is done the next one starts, in the
 slots the last one freed.  Results come back in request order.
 
 The loop decides with host data only and talks to the engine and the sampler
-through four calls (open, close, step, choose), so its decisions can be tested
-with stand-ins.
+through a handful of calls, so its decisions can be tested with stand-ins:
 
-When the engine takes token ids from the device (`decode`) and the sampler can
-hand them over without waiting (`choose_async`), the loop runs one step ahead:
-the step that feeds the tokens just chosen is queued before those tokens reach
-the host, so the GPU does not wait for the host's bookkeeping.  Whether a
-sequence goes on after a token is then known one step late: a sequence that
-turns out to have stopped has been given one step too many, whose result is
-dropped and whose slot is given back as before.  Choices that depend on the
-tokens generated so far (the repetition penalty) keep the simple order.
+    engine:  open(n) -> slots, close(slots), step(entries) -> logits rows (the prompts),
+             decode(slots, ids) -> logits rows (one token each; ids as the sampler left them on the device),
+             max_ctx, free_slots(), free_pages() and page_demand(n_tokens) (per storage group of the cache)
+    sampler: start(keys), choose_async(logits, configs, uniforms, keys=) -> (ids on the device, wait() -> ids on the host)
+
+The loop runs one step ahead of the host: the step that feeds the tokens just
+chosen is queued before those tokens reach the host, so the GPU does not wait
+for the host's bookkeeping.  Whether a sequence goes on after a token is then
+known one step late: a sequence that turns out to have stopped has been given
+one step too many, whose result is dropped and whose slot is given back as
+before.  The sampler keeps each request's recent tokens itself (by key: the
+request's slot), so the repetition penalty does not need them back first.
 """
 from __future__ import annotations
 
@@ -32,11 +35,7 @@ from typing import Callable, List, Optional, Sequence
 
 from ..sampling.options import GenerateConfig
 from ..sampling.rng import resolve_seed, uniform
-from ..sampling.sampler import RECENT
 from .engine import Entry
-
-PAGE = 64
-
 
 @dataclass
 class Result:
@@ -47,13 +46,16 @@ class Result:
 
 @dataclass
 class Stats:
-    """What computerex/dlgo reports per call (models/llm/generate.go:192-200,275-282)."""
+    """What computerex/dlgo reports per call (models/llm/generate.go:192-200,227-229,275-282), and the time of every
+    step: step_ms[0] of a batch is its prompt step, the others are the times from one step's tokens reaching the
+    host to the next step's (the loop runs a step ahead, so that is what a step costs)."""
     prefill_ms: float = 0.0
     generate_ms: float = 0.0
     output_tokens: int = 0
     prompt_tokens: int = 0
     batches: int = 0
     steps: int = 0
+    step_ms: List[float] = field(default_factory=list)
 
     @property
     def tokens_per_sec(self) -> float:
@@ -75,26 +77,30 @@ class _Live:
     tokens: List[int] = field(default_factory=list)
 
 
-def plan_batch(prompt_lens: Sequence[int], max_new: Sequence[int], free_slots: int, free_pages: int, max_batch: int,
-               max_ctx: int) -> int:
-    """How many of the waiting requests (in order) start together: each needs a slot and, at worst,
-    pages for min(prompt + max_new, context) tokens."""
-    n, pages = 0, 0
+def plan_batch(prompt_lens: Sequence[int], max_new: Sequence[int], free_slots: int, free_pages: Sequence[int], max_batch: int,
+               max_ctx: int, page_demand: Callable[[int], Sequence[int]]) -> int:
+    """How many of the waiting requests (in order) start together: each needs a slot and, at worst, in every storage
+    group of the cache the pages that page_demand gives for min(prompt + max_new, context) tokens."""
+    n = 0
+    used = [0] * len(free_pages)
     for p, m in zip(prompt_lens, max_new):
-        need = (min(p + m, max_ctx) + PAGE - 1) // PAGE
-        if n >= min(free_slots, max_batch) or pages + need > free_pages:
+        need = page_demand(min(p + m, max_ctx))
+        if n >= min(free_slots, max_batch) or any(u + d > f for u, d, f in zip(used, need, free_pages)):
             break
         n += 1
-        pages += need
+        used = [u + d for u, d in zip(used, need)]
     return n
 
 
-def _decode_ahead(engine, sampler, live, logits, prompts, results, stats, on_token) -> None:
-    """The decode loop of one batch, one step ahead of the host (see the module's text)."""
+def _decode_batch(engine, sampler, live, logits, prompts, results, stats, on_token) -> None:
+    """The decode loop of one batch, one step ahead of the host (see the module's text).  `logits` has one row per
+    entry of `live`, in order."""
     def finish(l, reason):
         results[l.index] = Result(l.tokens, reason, len(prompts[l.index]))
         engine.close([l.slot])
+        l.slot = -1
 
+    last = time.perf_counter()
     while live:
         # before a token is chosen: who may not go on at all
         keep = []
@@ -110,17 +116,18 @@ def _decode_ahead(engine, sampler, live, logits, prompts, results, stats, on_tok
         if len(keep) != len(live):
             logits = logits[keep]
             live = [live[r] for r in keep]
-        keyed = {"keys": [l.slot for l in live]} if getattr(sampler, "keeps_recent", False) else {}
-        tok_dev, wait = sampler.choose_async(logits, [l.config.sampler for l in live],
-                                             [uniform(l.seed, l.index, len(l.tokens)) for l in live], None, **keyed)
+        ids, wait = sampler.choose_async(logits, [l.config.sampler for l in live],
+                                         [uniform(l.seed, l.index, len(l.tokens)) for l in live], keys=[l.slot for l in live])
         # queue the next step for every sequence that wants another token after this one, before knowing the ids
-        fed = [row for row, l in enumerate(live) if len(l.tokens) + 1 < l.config.max_tokens]
+        fed = [row for row, l in enumerate(live) if len(l.tokens) + 1 < l.config.max_tokens and l.pos + 1 < engine.max_ctx - 1]
         next_logits = None
         if fed:
-            ids = tok_dev if len(fed) == len(live) else tok_dev[fed]
-            next_logits = engine.decode([live[r].slot for r in fed], ids)
+            next_logits = engine.decode([live[r].slot for r in fed], ids if len(fed) == len(live) else ids[fed])
             stats.steps += 1
         chosen = wait()
+        now = time.perf_counter()
+        stats.step_ms.append((now - last) * 1000.0)
+        last = now
         still = []
         for row, (l, tok) in enumerate(zip(live, chosen)):
             tok = int(tok)
@@ -128,31 +135,28 @@ def _decode_ahead(engine, sampler, live, logits, prompts, results, stats, on_tok
                 finish(l, "stop")         # if it was fed, that step's row is dropped
                 continue
             l.tokens.append(tok)
+            l.pos += 1
             stats.output_tokens += 1
             if on_token is not None:
                 on_token(l.index, tok)
             if len(l.tokens) >= l.config.max_tokens:
                 finish(l, "length")
-                continue
-            still.append(row)
+            elif l.pos >= engine.max_ctx - 1:
+                finish(l, "context")
+            else:
+                still.append(row)
         if not still:
             return
         rows = [fed.index(r) for r in still]          # every row in `still` was fed
         logits = next_logits if len(rows) == len(fed) else next_logits[rows]
         live = [live[r] for r in still]
-        for l in live:
-            l.pos += 1
 
 
 def generate(engine, sampler, prompts: Sequence[Sequence[int]], configs: Sequence[GenerateConfig],
              default_stop: Sequence[int] = (), on_token: Optional[Callable[[int, int], None]] = None,
              max_batch: int = 64, sync: Optional[Callable[[], None]] = None):
-    """Run every request; returns ([Result] in request order, Stats).
-
-    engine: open(n) -> slots, close(slots), step(entries) -> logits rows, max_ctx, free_pages(), free_slots().
-    sampler: choose(logits, sampler configs, uniforms, recent) -> token ids.
-    on_token(request index, token id) is called once per emitted token.
-    """
+    """Run every request; returns ([Result] in request order, Stats).  on_token(request index, token id) is called once
+    per emitted token; sync() waits for the device (for the timings)."""
     if len(prompts) != len(configs):
         raise GenerationError("one configuration per prompt")
     for i, p in enumerate(prompts):
@@ -167,7 +171,7 @@ def generate(engine, sampler, prompts: Sequence[Sequence[int]], configs: Sequenc
     seeds = [resolve_seed(c.seed) for c in configs]
     while waiting:
         n = plan_batch([len(prompts[i]) for i in waiting], [configs[i].max_tokens for i in waiting],
-                       engine.free_slots(), engine.free_pages(), max_batch, engine.max_ctx)
+                       engine.free_slots(), engine.free_pages(), max_batch, engine.max_ctx, engine.page_demand)
         if n == 0:
             i = waiting[0]
             raise GenerationError(f"request {i}: {len(prompts[i])} prompt tokens plus {configs[i].max_tokens} new ones do not fit the cache")
@@ -185,65 +189,16 @@ def generate(engine, sampler, prompts: Sequence[Sequence[int]], configs: Sequenc
             sync()
             t1 = time.perf_counter()
             stats.prefill_ms += (t1 - t0) * 1000.0
+            stats.step_ms.append((t1 - t0) * 1000.0)
             stats.prompt_tokens += sum(len(prompts[l.index]) for l in live)
             stats.steps += 1
-            keeps = getattr(sampler, "keeps_recent", False)      # then the penalty's tokens need not come back first
-            ahead = (hasattr(engine, "decode") and hasattr(sampler, "choose_async")
-                     and (keeps or not sampler.needs_recent([l.config.sampler for l in live])))
-            if ahead and keeps:
-                sampler.start([l.slot for l in live])
-            if ahead:
-                _decode_ahead(engine, sampler, live, logits, prompts, results, stats, on_token)
-                live = []
-            while live:
-                # sequences that may not go on leave before a token is chosen for them
-                keep_rows = []
-                for row, l in enumerate(live):
-                    if len(l.tokens) >= l.config.max_tokens:
-                        results[l.index] = Result(l.tokens, "length", len(prompts[l.index]))
-                    elif l.pos >= engine.max_ctx - 1:
-                        results[l.index] = Result(l.tokens, "context", len(prompts[l.index]))
-                    else:
-                        keep_rows.append(row)
-                        continue
-                    engine.close([l.slot])
-                if not keep_rows:
-                    live = []
-                    break
-                if len(keep_rows) != len(live):
-                    logits = logits[keep_rows] if hasattr(logits, "__getitem__") else logits
-                    live = [live[r] for r in keep_rows]
-                chosen = sampler.choose(logits, [l.config.sampler for l in live],
-                                        [uniform(l.seed, l.index, len(l.tokens)) for l in live],
-                                        [l.tokens[-RECENT:] for l in live])
-                nxt: List[_Live] = []
-                for l, tok in zip(live, chosen):
-                    tok = int(tok)
-                    if tok in l.stop:
-                        results[l.index] = Result(l.tokens, "stop", len(prompts[l.index]))
-                        engine.close([l.slot])
-                        continue
-                    l.tokens.append(tok)
-                    stats.output_tokens += 1
-                    if on_token is not None:
-                        on_token(l.index, tok)
-                    if len(l.tokens) >= l.config.max_tokens:
-                        results[l.index] = Result(l.tokens, "length", len(prompts[l.index]))
-                        engine.close([l.slot])
-                        continue
-                    nxt.append(l)
-                live = nxt
-                if not live:
-                    break
-                logits = engine.step([Entry(l.slot, [l.tokens[-1]], [0]) for l in live])
-                stats.steps += 1
-                for l in live:
-                    l.pos += 1
+            sampler.start([l.slot for l in live])
+            _decode_batch(engine, sampler, live, logits, prompts, results, stats, on_token)
             sync()
             stats.generate_ms += (time.perf_counter() - t1) * 1000.0
         except BaseException:
             for l in live:
-                if results[l.index] is None:
+                if results[l.index] is None and l.slot >= 0:
                     try:
                         engine.close([l.slot])
                     except Exception:

@@ -223,7 +223,7 @@ DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128)
 
 
 def all_variants(head_dims: Sequence[int] = DEFAULT_HEAD_DIMS) -> list[Variant]:
-    out: list[Variant] = [(m, ()) for m in ("embed", "rmsnorm", "rope_kv", "sampling")]
+    out: list[Variant] = [(m, ()) for m in ("embed", "rmsnorm", "rope_kv", "rowwise", "sampling")]
     out += [(m, (("DLGO_ELEM", code),)) for m in ("gemm", "gemm_rows") for code in (0, 1)]
     out += [("attention", (("HEAD_DIM", hd),)) for hd in head_dims]
     return out

@@ -80,7 +80,7 @@ def _lib(module: str, defines=()):
     if lib is None:
         lib = build.load(module, defines)
         for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_accum_norm", "dlgo_gemm_parts", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_attention_rows",
-                     "dlgo_attention_prefill", "dlgo_attention_prefill_f32", "dlgo_attention_decode", "dlgo_attention_decode_f32", "dlgo_argmax", "dlgo_sample"):
+                     "dlgo_attention_prefill", "dlgo_attention_prefill_f32", "dlgo_attention_decode", "dlgo_attention_decode_f32", "dlgo_argmax", "dlgo_sample", "dlgo_bias_add", "dlgo_head_rmsnorm"):
             if hasattr(lib, name):
                 getattr(lib, name).restype = ctypes.c_char_p
         _libs[key] = lib
@@ -119,6 +119,28 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor
     _check(_lib("rmsnorm").dlgo_rmsnorm(_ptr(x), _ptr(rows), _ptr(weight), _ptr(out), dtype_code(out.dtype), n, d,
                                         ctypes.c_float(eps), _stream()))
     return out
+
+
+def bias_add(y: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """y[t, n] += bias[n]; y rows in float32 or bfloat16 (row stride free), bias float32."""
+    _need(y, "rows", dims=2)
+    _need(bias, "bias", torch.float32, 1)
+    if bias.shape[0] != y.shape[1] or not bias.is_contiguous():
+        raise KernelError(f"bias_add: bias {tuple(bias.shape)} does not fit rows {tuple(y.shape)}")
+    _check(_lib("rowwise").dlgo_bias_add(_ptr(y), dtype_code(y.dtype), y.shape[0], y.shape[1], _rows(y, "rows"), _ptr(bias), _stream()))
+    return y
+
+
+def head_rmsnorm(x: torch.Tensor, first_col: int, n_heads: int, head_dim: int, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """Each of n_heads heads of head_dim consecutive elements, from column first_col on, of every row of x is RMS-normalised
+    in place over its own elements and multiplied by weight [head_dim] (float32)."""
+    _need(x, "rows", dims=2)
+    _need(weight, "head norm weight", torch.float32, 1)
+    if weight.shape[0] != head_dim or not weight.is_contiguous() or first_col < 0 or first_col + n_heads * head_dim > x.shape[1]:
+        raise KernelError(f"head_rmsnorm: {n_heads} heads of {head_dim} from column {first_col} and weight {tuple(weight.shape)} do not fit rows {tuple(x.shape)}")
+    _check(_lib("rowwise").dlgo_head_rmsnorm(_ptr(x), dtype_code(x.dtype), x.shape[0], _rows(x, "rows"), first_col, n_heads, head_dim,
+                                             _ptr(weight), ctypes.c_float(eps), _stream()))
+    return x
 
 
 def _streams_rows(weight: torch.Tensor, t: int, kind: int, has_scratch: bool, splits: int) -> bool:
@@ -486,11 +508,11 @@ def argmax(logits: torch.Tensor, out: torch.Tensor, scratch: Optional[torch.Tens
     return out
 
 
-def sample(logits: torch.Tensor, work: torch.Tensor, e: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
+def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
            top_p: torch.Tensor, min_p: torch.Tensor, penalty: torch.Tensor, recent: Optional[torch.Tensor],
            uniform: torch.Tensor, out: torch.Tensor, recent_rows: Optional[torch.Tensor] = None,
            counts: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """One token per row of float32 logits, each row with its own options.  recent [rows, w]: the row's recent tokens
+    """One token per row of float32 logits, each row with its own options.  work: float32 scratch [rows, vocab].  recent [rows, w]: the row's recent tokens
     (-1 where empty) for the repetition penalty.  With recent_rows [rows] and counts: recent is a table of rings, row
     recent_rows[r] of it belongs to row r and holds its last min(counts, w) tokens; the chosen token is added to it."""
     _need(logits, "logits", torch.float32, 2)
@@ -502,10 +524,9 @@ def sample(logits: torch.Tensor, work: torch.Tensor, e: torch.Tensor, temperatur
         _need(t, name, dt, 1)
         if t.shape[0] != n:
             raise KernelError(f"sample: {name} has {t.shape[0]} entries for {n} rows")
-    for name, t in (("work", work), ("e", e)):
-        _need(t, name, torch.float32, 2)
-        if t.shape[0] < n or t.shape[1] != v or not t.is_contiguous():
-            raise KernelError(f"sample: scratch {name} {tuple(t.shape)} too small for {(n, v)}")
+    _need(work, "work", torch.float32, 2)
+    if work.shape[0] < n or work.shape[1] != v or not work.is_contiguous():
+        raise KernelError(f"sample: scratch {tuple(work.shape)} too small for {(n, v)}")
     n_recent = 0
     if (recent_rows is None) != (counts is None):
         raise KernelError("sample: a table of rings needs both recent_rows and counts")
@@ -519,7 +540,7 @@ def sample(logits: torch.Tensor, work: torch.Tensor, e: torch.Tensor, temperatur
         _need(counts, "counts of recent tokens", torch.int32, 1)
         if recent is None or recent_rows.shape[0] != n or counts.shape[0] != recent.shape[0]:
             raise KernelError("sample: recent_rows has one entry per row of logits, counts one per row of the table")
-    _check(_lib("sampling").dlgo_sample(_ptr(logits), _rows(logits, "logits"), n, v, _ptr(work), _ptr(e), _ptr(temperature),
+    _check(_lib("sampling").dlgo_sample(_ptr(logits), _rows(logits, "logits"), n, v, _ptr(work), _ptr(temperature),
                                         _ptr(top_k), _ptr(top_p), _ptr(min_p), _ptr(penalty), _ptr(recent), n_recent,
                                         _ptr(recent_rows), _ptr(counts), _ptr(uniform), _ptr(out), _stream()))
     return out

@@ -5,7 +5,9 @@ computerex/dlgo resolves a LayerSpec for each layer (models/llm/loader.go:88-125
 which for this architecture is {RMSNorm, attention, standard residual, SwiGLU}
 (models/llm/model.go:12-55).  Tensor names are those of a config.json/safetensors
 folder: model.embed_tokens, model.layers.{i}.{input_layernorm, self_attn.{q,k,v,o}_proj,
-post_attention_layernorm, mlp.{gate,up,down}_proj}, model.norm, lm_head.
+post_attention_layernorm, mlp.{gate,up,down}_proj}, model.norm, lm_head; with
+`attention_bias` the four attention projections also have a `.bias` each (the reference adds
+biases where a layer has them, models/llm/forward.go:227-235).
 Projection rows in such a folder are not permuted, so the rotary pairing is
 split-half (the reference's interleaved pairing for "llama", models/llm/arch.go:18,
 suits the permuted rows of its own file format).
@@ -40,7 +42,7 @@ def build_llama(config: LlamaConfig) -> DecoderModel:
     for i, spec in enumerate(layer_specs(config)):
         position = make_part("position", spec.position, config.head_dim, config.rope_theta, config.rope_scaling)
         mixer = make_part("mixer", spec.mixer, d, config.num_attention_heads, config.num_key_value_heads, config.head_dim,
-                          position, window=spec.window)
+                          position, window=spec.window, bias=config.attention_bias, out_bias=config.attention_bias)
         ffn = make_part("feed_forward", spec.feed_forward, d, config.intermediate_size, "silu")
         block = make_part("block", spec.block,
                           ("input_layernorm", make_part("norm", spec.norm, d, config.rms_norm_eps)),

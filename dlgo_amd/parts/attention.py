@@ -11,6 +11,13 @@ are one kernel, and the output projection adds into the float32 residual stream.
 The mixer's sizes are its parameters; `window` limits each token to the last
 `window` keys (layers/gqa.go:98-132).  A run of the layer that reads another
 run's cache computes queries only and stores nothing.
+
+Two options that the reference applies when a layer has the tensors for them
+(models/llm/forward.go:227-244), both between projection and rotation: biases of
+the projections (`bias`; `out_bias` for the output projection's), and an RMSNorm
+of every q and k head over the head's own elements (`qk_norm_eps`).  A layer
+without them launches nothing for them; a layer with them takes the separate
+rotation kernel, since the fused ones read the product's result as it is.
 """
 from __future__ import annotations
 
@@ -55,11 +62,11 @@ class Mixer(Part):
 
 
 class Attention(Mixer):
-    kernel_modules = ("gemm", "gemm_rows", "rope_kv")
     leaves_norm = True
 
     def __init__(self, width: int, n_heads: int, n_kv_heads: int, head_dim: int, position: PositionEncoding,
-                 window: Optional[int] = None, scale: Optional[float] = None):
+                 window: Optional[int] = None, scale: Optional[float] = None, bias: bool = False, out_bias: bool = False,
+                 qk_norm_eps: Optional[float] = None):
         if n_heads % n_kv_heads:
             raise ValueError(f"attention: {n_heads} heads are not a multiple of {n_kv_heads} kv heads")
         if head_dim % 16:
@@ -69,19 +76,44 @@ class Attention(Mixer):
         self.position = position
         self.window = window
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)
+        self.bias, self.out_bias = bool(bias), bool(out_bias)
+        self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
         self.w_qkv: Optional[torch.Tensor] = None
         self.w_o: Optional[torch.Tensor] = None
+        self.b_qkv: Optional[torch.Tensor] = None
+        self.b_o: Optional[torch.Tensor] = None
+        self.q_norm: Optional[torch.Tensor] = None
+        self.k_norm: Optional[torch.Tensor] = None
+
+    @property
+    def kernel_modules(self):
+        extra = ("rowwise",) if self.bias or self.out_bias or self.qk_norm_eps is not None else ()
+        return ("gemm", "gemm_rows", "rope_kv") + extra
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:
-        return {
+        specs = {
             "q_proj.weight": TensorSpec((self.q_dim, self.width)),
             "k_proj.weight": TensorSpec((self.kv_dim, self.width)),
             "v_proj.weight": TensorSpec((self.kv_dim, self.width)),
             "o_proj.weight": TensorSpec((self.width, self.q_dim)),
         }
+        if self.bias:
+            specs.update({"q_proj.bias": TensorSpec((self.q_dim,), kind="vector", init="normal"),
+                          "k_proj.bias": TensorSpec((self.kv_dim,), kind="vector", init="normal"),
+                          "v_proj.bias": TensorSpec((self.kv_dim,), kind="vector", init="normal")})
+        if self.out_bias:
+            specs["o_proj.bias"] = TensorSpec((self.width,), kind="vector", init="normal")
+        if self.qk_norm_eps is not None:
+            specs.update({"q_norm.weight": TensorSpec((self.head_dim,), kind="vector", init="ones"),
+                          "k_norm.weight": TensorSpec((self.head_dim,), kind="vector", init="ones")})
+        return specs
+
+    MAX_HEAD_DIM = 512       # the attention kernels are compiled per head size, up to this one
 
     def check(self, dtype) -> None:
         check_inner("attention", (("width", self.width), ("heads * head size", self.q_dim)), dtype)
+        if self.head_dim > self.MAX_HEAD_DIM:
+            raise ValueError(f"attention: head size {self.head_dim} is beyond the kernels' largest, {self.MAX_HEAD_DIM}")
 
     def kernel_variants(self, dtype):
         from ..kernels.build import variant
@@ -98,6 +130,19 @@ class Attention(Mixer):
         fused = torch.cat([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], dim=0)
         self.w_qkv = stored(fused, spec["q_proj.weight"], device, dtype)
         self.w_o = stored(tensors["o_proj.weight"], spec["o_proj.weight"], device, dtype)
+        if self.bias:
+            fused_b = torch.cat([tensors["q_proj.bias"].float(), tensors["k_proj.bias"].float(), tensors["v_proj.bias"].float()])
+            self.b_qkv = stored(fused_b, spec["q_proj.bias"], device, dtype)
+        if self.out_bias:
+            self.b_o = stored(tensors["o_proj.bias"], spec["o_proj.bias"], device, dtype)
+        if self.qk_norm_eps is not None:
+            self.q_norm = stored(tensors["q_norm.weight"], spec["q_norm.weight"], device, dtype)
+            self.k_norm = stored(tensors["k_norm.weight"], spec["k_norm.weight"], device, dtype)
+
+    @property
+    def _between(self) -> bool:
+        """Something stands between the projections and the rotation."""
+        return self.bias or self.qk_norm_eps is not None
 
     def fuses_norm(self, norm, ctx) -> bool:
         return isinstance(norm, RMSNorm) and ops.fused_norm_pays(self.w_qkv, ctx.n_tokens)
@@ -111,17 +156,23 @@ class Attention(Mixer):
         kv = ctx.cache.kv_view(unit)
         rot = self.position.rotation()
         # a step of single tokens: the attention kernel rotates and stores by itself; else a kernel of its own does
-        fused = ops.attention_fuses_rotation(ctx.dtype, self.head_dim, self.n_heads // self.n_kv_heads, ctx.max_q_len,
-                                             rot.width if rot else 0, ctx.n_seq)
+        fused = not self._between and ops.attention_fuses_rotation(ctx.dtype, self.head_dim, self.n_heads // self.n_kv_heads,
+                                                                   ctx.max_q_len, rot.width if rot else 0, ctx.n_seq)
         unsummed = None
         if norm is not None:      # xn are the float32 residual rows: the norm rides in the product
             ops.gemm_rmsnorm(self.w_qkv[:cols], xn, norm.weight, norm.eps, qkv[:, :cols])
         else:
             # a product that shares k out over blocks leaves its runs to the rotation kernel, which adds them up as it reads
-            if not fused and ops.rope_takes_unsummed(ctx.dtype, self.head_dim, rot.width if rot else 0):
+            if not fused and not self._between and ops.rope_takes_unsummed(ctx.dtype, self.head_dim, rot.width if rot else 0):
                 unsummed = ops.gemm_runs(self.w_qkv[:cols], xn, split)
             if unsummed is None:
                 ops.gemm(self.w_qkv[:cols], xn, qkv[:, :cols], scratch=split)
+        if self.bias:
+            ops.bias_add(qkv[:, :cols], self.b_qkv[:cols])
+        if self.qk_norm_eps is not None:
+            ops.head_rmsnorm(qkv, 0, self.n_heads, self.head_dim, self.q_norm, self.qk_norm_eps)
+            if n_kv:
+                ops.head_rmsnorm(qkv, self.q_dim, n_kv, self.head_dim, self.k_norm, self.qk_norm_eps)
         if not fused:
             ops.rope_kv(qkv, self.n_heads, n_kv, self.head_dim, rot.width if rot else 0, rot.interleaved if rot else False,
                         rot.cos if rot else None, rot.sin if rot else None, ctx.positions,
@@ -130,6 +181,10 @@ class Attention(Mixer):
         out = ctx.buffer("attention.out", (t, self.q_dim), ctx.dtype)
         self.attend(qkv, out, ctx, kv, rotation=(rot.cos, rot.sin, rot.width, rot.interleaved) if fused and rot else None,
                     new_kv=fused and owns_cache)
+        if self.out_bias:        # the bias goes into the residual after the product: no norm of it can be left on the way
+            ops.gemm(self.w_o, out, residual, ops.EPI_ACCUM_F32, scratch=split)
+            ops.bias_add(residual, self.b_o)
+            return False
         if then is not None and isinstance(then[0], RMSNorm) and ops.gemm_accum_then_norm(
                 self.w_o, out, residual, split, then[0].weight, then[0].eps, then[1]):
             return True

@@ -26,7 +26,6 @@ class Sampler:
         self._pinned = [torch.empty(max_rows, dtype=torch.int32, pin_memory=True) for _ in range(4)]
         self._pin_next = 0
         self._work: Optional[torch.Tensor] = None
-        self._e: Optional[torch.Tensor] = None
         self._rings: Optional[torch.Tensor] = None      # [keys, RECENT] last tokens chosen per key
         self._counts: Optional[torch.Tensor] = None     # [keys] tokens chosen so far per key
 
@@ -48,7 +47,7 @@ class Sampler:
     def _grow(self, rows: int) -> None:
         if rows > self._out.shape[0]:
             self._out = torch.empty(rows, dtype=torch.int32, device=self.device)
-            self._work = self._e = None
+            self._work = None
 
     def choose(self, logits: torch.Tensor, configs: Sequence[SamplerConfig], uniforms: Sequence[float],
                recent: Optional[Sequence[Sequence[int]]] = None) -> List[int]:
@@ -94,7 +93,6 @@ class Sampler:
         if self._work is None:
             rows = self._out.shape[0]
             self._work = torch.empty((rows, self.vocab), dtype=torch.float32, device=self.device)
-            self._e = torch.empty((rows, self.vocab), dtype=torch.float32, device=self.device)
         f = np.zeros((5, n), dtype=np.float32)
         k = np.zeros((2, n), dtype=np.int32)        # top-k, and the row's key if the device keeps the recent tokens
         for i, c in enumerate(configs):
@@ -109,7 +107,7 @@ class Sampler:
         fd = torch.from_numpy(f).to(self.device)
         kd = torch.from_numpy(k).to(self.device)
         if rings:       # every choice is recorded, penalty or not: a later row of the request may have one
-            ops.sample(logits, self._work, self._e, fd[0], kd[0], fd[1], fd[2], fd[3], self._rings, fd[4], out,
+            ops.sample(logits, self._work, fd[0], kd[0], fd[1], fd[2], fd[3], self._rings, fd[4], out,
                        recent_rows=kd[1], counts=self._counts)
             return out
         rec = None
@@ -119,5 +117,5 @@ class Sampler:
                 toks = list(toks)[-RECENT:]
                 r[i, :len(toks)] = toks
             rec = torch.from_numpy(r).to(self.device)
-        ops.sample(logits, self._work, self._e, fd[0], kd[0], fd[1], fd[2], fd[3], rec, fd[4], out)
+        ops.sample(logits, self._work, fd[0], kd[0], fd[1], fd[2], fd[3], rec, fd[4], out)
         return out

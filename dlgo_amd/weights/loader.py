@@ -54,7 +54,11 @@ def open_folder(folder: str) -> Dict[str, SafetensorsFile]:
         files = [single]
     elif os.path.exists(index):
         with open(index) as f:
-            files = sorted({os.path.join(folder, v) for v in json.load(f)["weight_map"].values()})
+            shards = sorted(set(json.load(f)["weight_map"].values()))
+        outside = [v for v in shards if not isinstance(v, str) or os.path.isabs(v) or os.path.basename(v) != v or v in ("", ".", "..")]
+        if outside:
+            raise WeightsError(folder, other=[f"the index names a shard outside the folder: {v!r}" for v in outside])
+        files = [os.path.join(folder, v) for v in shards]
     else:
         raise WeightsError(folder, other=[f"neither model.safetensors nor model.safetensors.index.json found"])
     where: Dict[str, SafetensorsFile] = {}

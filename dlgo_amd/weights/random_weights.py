@@ -11,6 +11,7 @@ as 1 + w, shows).
 from __future__ import annotations
 
 import json
+import math
 import os
 import zlib
 from typing import Dict, Optional
@@ -23,10 +24,20 @@ from .safetensors_io import write_safetensors
 _DTYPES = {"bfloat16": torch.bfloat16, "float32": torch.float32, "float16": torch.float16}
 
 
-def _generator(seed: int, name: str, device) -> torch.Generator:
-    g = torch.Generator(device=device)
+def _generator(seed: int, name: str) -> torch.Generator:
+    """A tensor's own stream, keyed by the seed and the tensor's name.  It always runs on the host, so that a model drawn
+    straight onto a device and a model folder written for the same seed hold the same values."""
+    g = torch.Generator(device="cpu")
     g.manual_seed((int(seed) * 1000003 + zlib.crc32(name.encode())) % (2 ** 63))
     return g
+
+
+def _table(spec, g: torch.Generator) -> torch.Tensor:
+    """An integer table: a random permutation of its last axis in every row (ids that stay inside the table's own range,
+    whatever they index)."""
+    rows = math.prod(spec.shape[:-1])
+    perms = torch.stack([torch.randperm(spec.shape[-1], generator=g) for _ in range(rows)])
+    return perms.reshape(spec.shape).to(torch.int32)
 
 
 def random_tensors(config: ModelConfig, seed: int, dtype: Optional[torch.dtype] = None, std: Optional[float] = None,
@@ -43,18 +54,19 @@ def random_tensors(config: ModelConfig, seed: int, dtype: Optional[torch.dtype] 
             raise ValueError("random weights: the configuration has no initializer_range; pass std")
     out: Dict[str, torch.Tensor] = {}
     for name, spec in model.expected_tensors().items():
-        g = _generator(seed, name, device)
+        g = _generator(seed, name)
         if spec.kind == "table":
-            raise ValueError(f"random weights: no rule for the integer table {name}")
+            out[name] = _table(spec, g).to(device)
+            continue
         if spec.init == "ones":
-            t = torch.ones(spec.shape, dtype=torch.float32, device=device)
+            t = torch.ones(spec.shape, dtype=torch.float32)
             if norm_jitter:
-                t += norm_jitter * torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device)
+                t += norm_jitter * torch.randn(spec.shape, generator=g, dtype=torch.float32)
         elif spec.init == "normal":
-            t = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * std
+            t = torch.randn(spec.shape, generator=g, dtype=torch.float32) * std
         else:
             raise ValueError(f"random weights: unknown init {spec.init!r} of {name}")
-        out[name] = t.to(dtype)
+        out[name] = t.to(dtype).to(device)
     return out
 
 

@@ -41,6 +41,15 @@ class TensorInfo:
 class SafetensorsFile:
     """One open file: `infos` by name, `tensor(name)` as a CPU tensor over the mapping."""
 
+    def names(self):
+        return list(self.infos)
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
     def __init__(self, path: str):
         self.path = path
         try:
@@ -63,10 +72,24 @@ class SafetensorsFile:
         for name, info in header.items():
             if name == "__metadata__":
                 continue
-            b, e = info["data_offsets"]
-            shape = tuple(int(s) for s in info["shape"])
+            try:
+                b, e = (int(v) for v in info["data_offsets"])
+                shape = tuple(int(s) for s in info["shape"])
+                dtype_name = info["dtype"]
+            except (KeyError, TypeError, ValueError):
+                raise SafetensorsError(f"{path}: header entry of tensor {name} is malformed") from None
+            if b < 0 or e < b or any(d < 0 for d in shape):
+                raise SafetensorsError(f"{path}: tensor {name} has offsets [{b}, {e}) and shape {list(shape)}")
             if self.data_start + e > size:
                 raise SafetensorsError(f"{path}: truncated (tensor {name} ends at byte {self.data_start + e} of {size})")
+            if dtype_name in _DTYPES:
+                n = 1
+                for d in shape:
+                    n *= d
+                want = n * torch.empty(0, dtype=_DTYPES[dtype_name]).element_size()
+                if e - b != want:
+                    raise SafetensorsError(f"{path}: tensor {name} of shape {list(shape)} and type {dtype_name} needs {want} bytes, "
+                                           f"its offsets [{b}, {e}) give {e - b}")
             self.infos[name] = TensorInfo(name, info["dtype"], shape, b, e, path)
         self._map = None
 

@@ -187,12 +187,18 @@ def block(x, positions, w, prefix, cfg, inv_freq, window=None):
     q = xn @ w[prefix + "self_attn.q_proj.weight"].T
     k = xn @ w[prefix + "self_attn.k_proj.weight"].T
     v = xn @ w[prefix + "self_attn.v_proj.weight"].T
+    if prefix + "self_attn.q_proj.bias" in w:          # biases where the layer has them (models/llm/forward.go:227-235)
+        q = q + w[prefix + "self_attn.q_proj.bias"]
+        k = k + w[prefix + "self_attn.k_proj.bias"]
+        v = v + w[prefix + "self_attn.v_proj.bias"]
     T = x.shape[0]
     for t in range(T):
         q[t] = rope_apply(q[t].reshape(H, hd), positions[t], inv_freq).reshape(-1)
         k[t] = rope_apply(k[t].reshape(KV, hd), positions[t], inv_freq).reshape(-1)
     a = attention(q, k, v, H, KV, hd, window)
     h = x + a @ w[prefix + "self_attn.o_proj.weight"].T
+    if prefix + "self_attn.o_proj.bias" in w:          # (models/llm/forward.go:286-289)
+        h = h + w[prefix + "self_attn.o_proj.bias"]
     hn = rmsnorm(h, w[prefix + "post_attention_layernorm.weight"], eps)
     f = feed_forward(hn, w[prefix + "mlp.gate_proj.weight"], w[prefix + "mlp.up_proj.weight"],
                      w[prefix + "mlp.down_proj.weight"])

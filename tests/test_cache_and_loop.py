@@ -139,9 +139,51 @@ def test_random_traffic_keeps_the_books():
         assert c.groups[0].pool.n_free == 40 - held
 
 
+def test_a_cache_of_windowed_groups_only_is_counted_too():
+    """No full group to run out first: the windowed pool itself is what a step is checked against, before anything is
+    taken, and what the loop plans with."""
+    need = [CacheNeed(kind="kv", kv_heads=2, head_dim=16, window=100)]
+    c = Cache([need], max_tokens=8 * PAGE, max_ctx=8 * PAGE, dtype=torch.float32, device="cpu", max_slots=3, max_step_tokens=64)
+    assert c.groups[0].pool.n_pages == 8 and c.groups[0].pages_per_seq == 4       # window + a step's piece, in pages, + 1
+    assert c.page_demand(500) == (4,) and c.page_demand(70) == (2,) and c.free_pages() == (8,)
+    assert plan_batch([400, 400, 400], [50, 50, 50], 3, c.free_pages(), 64, c.max_ctx, c.page_demand) == 2
+    slots = [c.alloc_slot() for _ in range(3)]
+
+    def grow(slot, total):                       # a long prompt, in pieces of a step's size
+        while c.length(slot) < total:
+            n = min(64, total - c.length(slot))
+            assert c.can_reserve([(slot, c.length(slot) + n)]) is None
+            c.reserve([(slot, c.length(slot) + n)])
+            c.advance(slot, n)
+            c.check_consistent()
+            assert len(c.held_pages(slot)) <= 4
+    grow(slots[0], 400)
+    grow(slots[1], 400)
+    held = len(c.held_pages(slots[0])) + len(c.held_pages(slots[1]))
+    assert c.free_pages() == (8 - held,)
+    # a whole long prompt is judged by what it holds at worst, not by its length
+    assert c.can_reserve([(slots[0], 512)]) is None
+    # the third sequence does not fit beside them: the check says so, and nothing was taken
+    free = c.free_pages()
+    why = c.can_reserve([(slots[2], 64 * (free[0] + 1))])
+    assert why is not None and "cache full" in why
+    with pytest.raises(OutOfPages):
+        c.reserve([(slots[2], 64 * (free[0] + 1))])
+    assert c.free_pages() == free and not c.held_pages(slots[2])
+    c.check_consistent()
+    c.free_slot(slots[0])
+    grow(slots[2], 200)
+    for s in slots[1:]:
+        c.free_slot(s)
+    assert c.free_pages() == (8,)
+    c.check_consistent()
+
+
 # -- the generation loop -------------------------------------------------------------
 class FakeEngine:
-    """Slots and pages like the real one; 'logits' are the (request, position) pairs the sampler decides on."""
+    """Slots and pages like the real one; 'logits' are rows (slot, tokens held) that the sampler decides on.  Like the
+    real one it takes the prompts through step() and single tokens through decode(), whose ids are whatever the
+    sampler left 'on the device' (here: an array whose values the loop has not looked at yet)."""
 
     def __init__(self, max_ctx=64, slots=3, pages=6):
         self.max_ctx, self._slots, self._pages = max_ctx, slots, pages
@@ -154,7 +196,10 @@ class FakeEngine:
         return len(self.free)
 
     def free_pages(self):
-        return self._pages - sum((n + PAGE - 1) // PAGE for n in self.held.values())
+        return (self._pages - sum((n + PAGE - 1) // PAGE for n in self.held.values()),)
+
+    def page_demand(self, n_tokens):
+        return ((n_tokens + PAGE - 1) // PAGE,)
 
     def open(self, n):
         out = [self.free.pop(0) for _ in range(n)]
@@ -169,36 +214,68 @@ class FakeEngine:
             self.free.append(s)
             self.closed.append(s)
 
+    def _run(self, rows):
+        assert len({slot for slot, _, _ in rows}) == len(rows)
+        for slot, tokens, _ in rows:
+            assert slot in self.held, "a step for a slot that was given back"
+            self.held[slot] += len(tokens)
+            assert self.held[slot] <= self.max_ctx
+        assert self.free_pages()[0] >= 0
+        self.steps.append(rows)
+        return np.array([(slot, self.held[slot]) for slot, _, _ in rows])
+
     def step(self, entries):
-        assert len({e.slot for e in entries}) == len(entries)
-        for e in entries:
-            assert e.slot in self.held
-            self.held[e.slot] += len(e.tokens)
-            assert self.held[e.slot] <= self.max_ctx
-        assert self.free_pages() >= 0
-        self.steps.append([(e.slot, list(e.tokens), list(e.want)) for e in entries])
-        return [(e.slot, self.held[e.slot]) for e in entries]
+        return self._run([(e.slot, list(e.tokens), list(e.want)) for e in entries])
+
+    def decode(self, slots, ids):
+        assert len(slots) == len(ids)
+        return self._run([(int(s), [int(t)], [0]) for s, t in zip(slots, ids)])
 
 
 class ScriptSampler:
-    """Token = 100 + length of the sequence so far, or a scripted stop."""
+    """Token = 100 + length of the sequence so far, or a scripted stop.  It keeps each key's recent tokens itself, as the
+    real one does on the device."""
 
     def __init__(self, stop_at=None):
         self.stop_at = stop_at or {}
         self.calls = []
+        self.recent = {}
+        self.waited = 0
 
-    def choose(self, logits, configs, uniforms, recent):
-        self.calls.append((list(logits), list(uniforms), [list(r) for r in recent]))
-        return [self.stop_at.get((slot, n), 100 + n) for slot, n in logits]
+    def start(self, keys):
+        for k in keys:
+            self.recent[k] = []
+
+    def choose_async(self, logits, configs, uniforms, recent=None, keys=None):
+        assert recent is None and len(keys) == len(logits) == len(configs) == len(uniforms)
+        assert all(int(slot) == k for (slot, _), k in zip(logits, keys)), "rows and keys out of step"
+        self.calls.append(([tuple(r) for r in logits], list(uniforms), [list(self.recent[k]) for k in keys]))
+        ids = np.array([self.stop_at.get((int(slot), int(n)), 100 + int(n)) for slot, n in logits])
+        for k, t in zip(keys, ids):
+            self.recent[k] = (self.recent[k] + [int(t)])[-64:]
+
+        def wait():
+            self.waited += 1
+            return ids.tolist()
+        return ids, wait
+
+
+def one_group(n):
+    return ((n + PAGE - 1) // PAGE,)
 
 
 def test_plan_batch():
-    assert plan_batch([5, 9, 1], [8, 8, 8], free_slots=3, free_pages=6, max_batch=64, max_ctx=4096) == 3
-    assert plan_batch([5, 9, 1], [8, 8, 8], free_slots=2, free_pages=6, max_batch=64, max_ctx=4096) == 2
-    assert plan_batch([60, 60, 60], [8, 8, 8], free_slots=3, free_pages=5, max_batch=64, max_ctx=4096) == 2
-    assert plan_batch([60, 60], [1000, 8], free_slots=3, free_pages=2, max_batch=64, max_ctx=64) == 2      # capped by the context
-    assert plan_batch([200], [8], free_slots=3, free_pages=2, max_batch=64, max_ctx=4096) == 0
-    assert plan_batch([1] * 9, [1] * 9, free_slots=9, free_pages=9, max_batch=4, max_ctx=64) == 4
+    assert plan_batch([5, 9, 1], [8, 8, 8], 3, (6,), max_batch=64, max_ctx=4096, page_demand=one_group) == 3
+    assert plan_batch([5, 9, 1], [8, 8, 8], 2, (6,), max_batch=64, max_ctx=4096, page_demand=one_group) == 2
+    assert plan_batch([60, 60, 60], [8, 8, 8], 3, (5,), max_batch=64, max_ctx=4096, page_demand=one_group) == 2
+    assert plan_batch([60, 60], [1000, 8], 3, (2,), max_batch=64, max_ctx=64, page_demand=one_group) == 2      # capped by the context
+    assert plan_batch([200], [8], 3, (2,), max_batch=64, max_ctx=4096, page_demand=one_group) == 0
+    assert plan_batch([1] * 9, [1] * 9, 9, (9,), max_batch=4, max_ctx=64, page_demand=one_group) == 4
+    # every storage group of the cache counts: a second, windowed group that allows two pages a sequence
+    two = lambda n: ((n + PAGE - 1) // PAGE, min((n + PAGE - 1) // PAGE, 2))
+    assert plan_batch([300, 300, 300], [8, 8, 8], 3, (100, 5), max_batch=64, max_ctx=4096, page_demand=two) == 2
+    # and a model that keeps no keys or values at all is limited by its slots only
+    assert plan_batch([300, 300, 300], [8, 8, 8], 2, (), max_batch=64, max_ctx=4096, page_demand=lambda n: ()) == 2
 
 
 def test_loop_unequal_batch_early_finishers_and_slot_reuse():
@@ -219,18 +296,31 @@ def test_loop_unequal_batch_early_finishers_and_slot_reuse():
     # no step feeds a sequence's last token back; the second batch runs in slots the first gave back
     assert sum(len(s) for s in eng.steps) == 3 + 2 + 2 + 1 + 1 + 2 + 2 + 1 + 1
     assert sorted(eng.closed) == [0, 0, 1, 1, 2] and not eng.held and eng.free_slots() == 3
+    # a time for every step: a prompt step and then one per choice, for each batch
+    assert stats.steps == len(eng.steps) and len(stats.step_ms) == 2 + samp.waited and all(t >= 0 for t in stats.step_ms)
 
 
-def test_loop_stop_tokens_are_not_emitted_nor_fed_back():
+def test_loop_runs_a_step_ahead_and_drops_the_step_of_a_sequence_that_stopped():
+    """The step that feeds a token is queued before the token is known.  A stop token is therefore fed once, in the step
+    that was already on its way; that step's row is dropped, nothing of it is emitted, the slot goes back, and the rows
+    of the sequences that go on are picked out of the result by their place among the sequences that were fed."""
     eng = FakeEngine()
     samp = ScriptSampler(stop_at={(0, 7): 2, (1, 3): 9})      # request 0 stops at its third choice, request 1 at once
     cfg = GenerateConfig(max_tokens=6, sampler=SamplerConfig(temperature=0))
-    results, _ = generate(eng, samp, [[1] * 5, [1] * 3, [1] * 2], [cfg] * 3, default_stop=(2, 9))
+    results, stats = generate(eng, samp, [[1] * 5, [1] * 3, [1] * 2], [cfg] * 3, default_stop=(2, 9))
     assert results[0].tokens == [105, 106] and results[0].finish_reason == "stop"
     assert results[1].tokens == [] and results[1].finish_reason == "stop"             # immediate stop: nothing
-    assert len(results[2].tokens) == 6 and results[2].finish_reason == "length"
-    fed = [t for s in eng.steps[1:] for _, toks, _ in s for t in toks]
-    assert 2 not in fed and 9 not in fed
+    assert results[2].tokens == [102, 103, 104, 105, 106, 107] and results[2].finish_reason == "length"
+    # step 1 was queued for all three before request 1's stop was known; request 1 is not in step 2
+    assert [slot for slot, _, _ in eng.steps[1]] == [0, 1, 2] and eng.steps[1][1][1] == [9]
+    assert [slot for slot, _, _ in eng.steps[2]] == [0, 2]
+    # request 0's stop token (2) went into step 3, the step after it only has request 2
+    assert eng.steps[3] == [(0, [2], [0]), (2, [104], [0])] and [slot for slot, _, _ in eng.steps[4]] == [2]
+    # the sampler never saw a row of a sequence that had stopped, and rows stayed with their sequences
+    for rows, _, _ in samp.calls[1:]:
+        assert all((slot, n) != (1, 4) for slot, n in rows)
+    assert samp.calls[3][0] == [(2, 5)]
+    assert stats.output_tokens == 8 and not eng.held and sorted(eng.closed) == [0, 1, 2]
     # the same script with ignore_eos runs to the length
     cfg2 = GenerateConfig(max_tokens=6, sampler=SamplerConfig(temperature=0), ignore_eos=True)
     r2, _ = generate(FakeEngine(), ScriptSampler(stop_at={(0, 7): 2}), [[1] * 5], [cfg2], default_stop=(2,))
@@ -246,6 +336,7 @@ def test_loop_context_end_and_errors():
     cfg = GenerateConfig(max_tokens=100, sampler=SamplerConfig(temperature=0))
     results, _ = generate(eng, ScriptSampler(), [[1] * 10], [cfg])
     assert results[0].finish_reason == "context" and len(results[0].tokens) == 5      # stops when 15 tokens are cached
+    assert eng.steps[-1] == [(0, [113], [0])] and len(eng.steps) == 5                  # the fifth token is not fed: nothing follows it
     with pytest.raises(GenerationError, match="prompt too long: 16 tokens"):
         generate(eng, ScriptSampler(), [[1] * 16], [cfg])
     with pytest.raises(GenerationError, match="empty prompt"):
@@ -254,14 +345,17 @@ def test_loop_context_end_and_errors():
         generate(FakeEngine(max_ctx=4096, pages=1), ScriptSampler(), [[1] * 70], [cfg])
     zero, _ = generate(eng, ScriptSampler(), [[1] * 3], [GenerateConfig(max_tokens=0)])
     assert zero[0].tokens == [] and zero[0].finish_reason == "length" and not eng.held
+    # a prompt that fills the context but for one place: nothing can be chosen
+    full, _ = generate(eng, ScriptSampler(), [[1] * 15], [cfg])
+    assert full[0].tokens == [] and full[0].finish_reason == "context" and not eng.held
 
 
 def test_loop_gives_slots_back_when_a_step_fails():
     class Failing(FakeEngine):
-        def step(self, entries):
+        def decode(self, slots, ids):
             if len(self.steps) == 2:
                 raise RuntimeError("boom")
-            return super().step(entries)
+            return super().decode(slots, ids)
     eng = Failing()
     cfg = GenerateConfig(max_tokens=5, sampler=SamplerConfig(temperature=0))
     with pytest.raises(RuntimeError, match="boom"):
@@ -277,7 +371,7 @@ def test_draws_are_per_request_and_seeded():
     assert u0[0] == [uniform(77, 0, 0), uniform(77, 1, 0)] and u0[2] == [uniform(77, 0, 2), uniform(77, 1, 2)]
     assert all(0.0 <= x < 1.0 for call in u0 for x in call)
     assert np.float32(u0[1][0]) == u0[1][0]                      # representable in float32
-    assert samp.calls[2][2] == [[104, 105], [102, 103]]          # the tokens so far, for the repetition penalty
+    assert samp.calls[2][2] == [[104, 105], [102, 103]]          # the tokens so far, kept under each request's key
     vals = [uniform(1, 0, s) for s in range(4000)]
     assert abs(np.mean(vals) - 0.5) < 0.02 and len(set(vals)) > 3990
 

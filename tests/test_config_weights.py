@@ -44,7 +44,7 @@ def test_config_defaults_are_derived_not_invented(tiny_a):
     ({"num_key_value_heads": 3}, "multiple of num_key_value_heads"),
     ({"head_dim": 15}, "even"),
     ({"hidden_act": "gelu"}, "hidden_act"),
-    ({"attention_bias": True}, "attention_bias"),
+    ({"attention_bias": "yes"}, "attention_bias"),
     ({"mlp_bias": True}, "mlp_bias"),
     ({"rope_scaling": {"rope_type": "yarn", "factor": 2.0}}, "rope_type"),
     ({"rope_scaling": {"rope_type": "llama3", "factor": 2.0}}, "low_freq_factor"),
@@ -221,3 +221,93 @@ def test_rotary_frequencies_blend_on_constructed_wavelengths():
     # no scaling block, and a factor of one, leave the plain frequencies
     cfg = config_from_dict(dict(TINY_A))
     assert list(rotary_frequencies(16, 10000.0, None)) == [1.0 / math.pow(10000.0, 2.0 * i / 16) for i in range(8)]
+
+
+def test_attention_bias_is_an_option_of_the_architecture(tiny_a, tmp_path):
+    """config.json's attention_bias gives the four attention projections a bias each: the model expects the tensors, the
+    random-weights mode writes them, and a folder without them is refused by name."""
+    c = config_from_dict(dict(tiny_a, attention_bias=True))
+    assert c.attention_bias and config_from_dict(c.to_dict()) == c and not config_from_dict(tiny_a).attention_bias
+    names = build_model(c).expected_tensors()
+    assert names["model.layers.1.self_attn.k_proj.bias"].shape == (c.kv_dim,)
+    assert names["model.layers.0.self_attn.o_proj.bias"].shape == (c.hidden_size,)
+    assert not any(n.endswith(".bias") for n in build_model(config_from_dict(tiny_a)).expected_tensors())
+    folder = write_random_model(c, 4, str(tmp_path / "with_bias"))
+    with SafetensorsFile(os.path.join(folder, "model.safetensors")) as f:
+        assert "model.layers.0.self_attn.q_proj.bias" in f.names()
+    plain_folder = write_random_model(config_from_dict(tiny_a), 4, str(tmp_path / "without"))
+    with open(os.path.join(plain_folder, "config.json"), "w") as f:
+        json.dump(c.to_dict(), f)
+    with pytest.raises(WeightsError, match="q_proj.bias"):
+        load_weights(build_model(c), plain_folder, "cpu", torch.float32)
+
+
+def test_random_weights_do_not_depend_on_the_device_and_fill_integer_tables():
+    from dlgo_amd.parts import TensorSpec
+    from dlgo_amd.weights.random_weights import _generator, _table
+    t = _table(TensorSpec((3, 17), kind="table"), _generator(5, "x"))
+    assert t.dtype == torch.int32 and t.shape == (3, 17)
+    assert all(sorted(row.tolist()) == list(range(17)) for row in t)
+    assert torch.equal(t, _table(TensorSpec((3, 17), kind="table"), _generator(5, "x")))
+    assert not torch.equal(t, _table(TensorSpec((3, 17), kind="table"), _generator(6, "x")))
+    # the stream is keyed by seed and name and runs on the host: the same call gives the same values
+    c = config_from_dict(TINY_A)
+    a, b = random_tensors(c, 9), random_tensors(c, 9)
+    assert all(torch.equal(a[k], b[k]) for k in a) and not torch.equal(a["model.norm.weight"], random_tensors(c, 9, norm_jitter=0.1)["model.norm.weight"])
+
+
+def _rewrite_header(path, change):
+    """Write the file again with its JSON header passed through `change` (the data stays as it is)."""
+    import struct
+    raw = open(path, "rb").read()
+    (hlen,) = struct.unpack("<Q", raw[:8])
+    header = json.loads(raw[8:8 + hlen])
+    change(header)
+    blob = json.dumps(header, separators=(",", ":")).encode()
+    with open(path, "wb") as f:
+        f.write(struct.pack("<Q", len(blob)) + blob + raw[8 + hlen:])
+
+
+def test_a_header_whose_offsets_disagree_with_the_shape_is_refused(tmp_path, tiny_a):
+    from dlgo_amd.weights.safetensors_io import SafetensorsError
+    for i, (what, needle) in enumerate([
+            (lambda h: h["model.norm.weight"].__setitem__("data_offsets", [0, 8]), "needs"),          # another tensor's bytes
+            (lambda h: h["model.norm.weight"].__setitem__("shape", [65]), "needs"),
+            (lambda h: h["model.norm.weight"].__setitem__("data_offsets", [16, 8]), "offsets"),
+            (lambda h: h["model.norm.weight"].__setitem__("data_offsets", [-4, 252]), "offsets"),
+            (lambda h: h["model.norm.weight"].pop("shape"), "malformed")]):
+        folder = make_folder(tiny_a, 5, tmp_path / f"case{i}")
+        _rewrite_header(os.path.join(folder, "model.safetensors"), what)
+        with pytest.raises(SafetensorsError, match=needle):
+            SafetensorsFile(os.path.join(folder, "model.safetensors"))
+        with pytest.raises(WeightsError, match="model.norm.weight"):
+            load_weights(build_model(load_config(folder)), folder, "cpu", torch.float32)
+
+
+def test_an_index_that_names_a_shard_outside_the_folder_is_refused(tmp_path, tiny_a):
+    folder = make_folder(tiny_a, 5, tmp_path / "m")
+    os.rename(os.path.join(folder, "model.safetensors"), str(tmp_path / "elsewhere.safetensors"))
+    for shard in ("../elsewhere.safetensors", str(tmp_path / "elsewhere.safetensors"), "sub/../../elsewhere.safetensors"):
+        json.dump({"weight_map": {"model.norm.weight": shard}}, open(os.path.join(folder, "model.safetensors.index.json"), "w"))
+        with pytest.raises(WeightsError, match="outside the folder"):
+            load_weights(build_model(load_config(folder)), folder, "cpu", torch.float32)
+
+
+def test_a_float16_file_loads_and_widens_exactly(tmp_path, tiny_a):
+    """Tensors stored in float16 are accepted: matrices go to the run dtype, norm weights to float32, bit for bit the
+    values the file holds."""
+    cfg = config_from_dict(tiny_a)
+    folder = write_random_model(cfg, 8, str(tmp_path), dtype=torch.float16, norm_jitter=0.1)
+    with SafetensorsFile(os.path.join(folder, "model.safetensors")) as f:
+        assert {i.dtype for i in f.infos.values()} == {"F16"}
+        held = {n: f.tensor(n).clone() for n in f.names()}
+    m = build_model(load_config(folder))
+    load_weights(m, folder, "cpu", torch.float32)
+    assert m.final_norm.weight.dtype == torch.float32 and torch.equal(m.final_norm.weight, held["model.norm.weight"].float())
+    assert m.embedding.weight.dtype == torch.float32 and torch.equal(m.embedding.weight, held["model.embed_tokens.weight"].float())
+    attn = m.layers[0][1].mixer
+    assert torch.equal(attn.w_qkv[:cfg.q_dim], held["model.layers.0.self_attn.q_proj.weight"].float())
+    m2 = build_model(load_config(folder))
+    load_weights(m2, folder, "cpu", torch.bfloat16)
+    assert m2.embedding.weight.dtype == torch.bfloat16 and m2.final_norm.weight.dtype == torch.float32
+    assert torch.equal(m2.embedding.weight, held["model.embed_tokens.weight"].to(torch.bfloat16))

@@ -86,10 +86,11 @@ def test_last_tokens_one_by_one(folders, oracle, name, dtype, graphs):
     want = oracle(name, dtype, tokens)
     (slot,) = eng.open(1)
     head = len(tokens) - 32
-    rows = [eng.step([Entry(slot, tokens[:head], list(range(head)))]).cpu().numpy()]
+    # the results are looked at only after the last step: each step's logits are the caller's to keep
+    rows = [eng.step([Entry(slot, tokens[:head], list(range(head)))])]
     for t in tokens[head:]:
-        rows.append(eng.step([Entry(slot, [t], [0])]).cpu().numpy().copy())
-    got = np.concatenate(rows)
+        rows.append(eng.step([Entry(slot, [t], [0])]))
+    got = np.concatenate([r.cpu().numpy() for r in rows])
     assert rel_err(got, want) <= TOL[dtype]
     # whole against one-by-one: the same numbers beyond rounding, also where the plain one is further away
     eng.close([slot])
@@ -199,7 +200,7 @@ def test_thousands_of_tokens(tmp_path, dtype):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_more_sequences_than_a_recorded_step_takes(folders, oracle, dtype):
     """150 sequences that start together and go on one token at a time: more than the largest batch for which single
-    tokens are recorded and replayed, so the steps take the general way; a few of them checked against the plain one."""
+    tokens are recorded and replayed, so each step goes in several runs; a few of them checked against the plain one."""
     from dlgo_amd.engine import Entry
     n = 150
     eng = engine_for(folders["A", dtype], dtype, max_tokens=n * 64, max_slots=n, graph_max_batch=64)
@@ -250,6 +251,10 @@ def test_sizes_the_kernels_cannot_take_are_refused_at_once(tmp_path):
     folder = make_folder(raw, 1, tmp_path, dtype="float32")
     with pytest.raises(EngineError, match="multiple of 8"):
         Engine.from_folder(folder, "bfloat16", max_tokens=128)
+    big_head = make_folder(dict(TINY_A, hidden_size=64, num_attention_heads=1, num_key_value_heads=1, head_dim=528), 1,
+                           tmp_path / "big_head", dtype="float32")
+    with pytest.raises(EngineError, match="head size 528"):
+        Engine.from_folder(big_head, "float32", max_tokens=128)
     eng = Engine.from_folder(folder, "float32", max_tokens=128)       # 68 and 100 are multiples of 4: float32 runs
     from dlgo_amd.engine import Entry
     (slot,) = eng.open(1)
@@ -274,3 +279,34 @@ def test_wanted_places_in_any_order_with_an_odd_vocabulary(folders, oracle, dtyp
     for r, (i, p) in enumerate(rows):
         assert rel_err(out[r], oracle("C", dtype, seqs[i])[p]) <= TOL[dtype], (r, i, p)
     assert [eng.length(s) for s in slots] == [90, 41, 7]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_model_with_attention_biases(tmp_path, dtype):
+    """config.json's attention_bias: the four attention projections have a bias each.  Whole, in a batch of unequal
+    lengths, and the last tokens one by one (a recorded step included), against the plain implementation."""
+    from dlgo_amd.engine import Engine, Entry
+    raw = dict(TINY_B, attention_bias=True)
+    folder = make_folder(raw, 17, tmp_path, dtype=dtype, std=0.08, norm_jitter=0.1)
+    cfg, w = plain.read_model(folder)
+    assert "model.layers.2.self_attn.o_proj.bias" in w
+    seqs = prompts_for(raw, [70, 9, 33], seed=12)
+    want = [plain.forward(cfg, w, t) for t in seqs]
+    # the biases matter: without them the logits are far away
+    stripped = {k: v for k, v in w.items() if not k.endswith(".bias")}
+    assert rel_err(plain.forward(cfg, stripped, seqs[1]), want[1]) > 10 * TOL[dtype]
+    eng = Engine.from_folder(folder, dtype, max_tokens=1024)
+    slots = eng.open(3)
+    out = eng.step([Entry(s, t, list(range(len(t)))) for s, t in zip(slots, seqs)]).cpu().numpy()
+    o = 0
+    for t, wnt in zip(seqs, want):
+        assert rel_err(out[o:o + len(t)], wnt) <= TOL[dtype]
+        o += len(t)
+    eng.close(slots)
+    (slot,) = eng.open(1)
+    rows = [eng.step([Entry(slot, seqs[0][:60], list(range(60)))])]
+    for t in seqs[0][60:]:
+        rows.append(eng.step([Entry(slot, [t], [0])]))
+    assert rel_err(np.concatenate([r.cpu().numpy() for r in rows]), want[0]) <= TOL[dtype]
+    assert 1 in eng._graphs
+    eng.close([slot])

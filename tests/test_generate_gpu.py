@@ -117,6 +117,82 @@ def test_long_decoding_and_context_end(folder_a):
         llm.generate([1] * 128, dlgo_amd.with_greedy())
 
 
+def _check_against_margin(cfg, w, prompt, tokens, tol):
+    """Greedy tokens of a reduced-precision run, against the plain logits of the same sequence: where the plain
+    implementation's best token leads by more than the run's error bound the run must have chosen it, elsewhere a
+    token within the bound of the best."""
+    seq = list(prompt)
+    decided = 0
+    for tok in tokens:
+        logits = plain.forward(cfg, w, seq)[-1]
+        bound = 2.0 * tol * np.abs(logits).max()
+        best = int(np.argmax(logits))
+        if logits[best] - np.partition(logits, -2)[-2] > bound:
+            assert tok == best, (len(seq), tok, best)
+            decided += 1
+        else:
+            assert logits[tok] >= logits[best] - bound, (len(seq), tok, best)
+        seq.append(tok)
+    return decided
+
+
+def test_bfloat16_generation_follows_the_plain_logits_where_their_margin_allows(folder_a):
+    import dlgo_amd
+    cfg, w = plain.read_model(folder_a)
+    llm = dlgo_amd.load_llm(folder_a, dtype="bfloat16", max_tokens=512)
+    prompts = _prompts(TINY_A, [5, 9, 1, 30], seed=7)
+    results = llm.generate(prompts, dlgo_amd.with_greedy(), dlgo_amd.with_max_tokens(24), dlgo_amd.with_ignore_eos())
+    decided = sum(_check_against_margin(cfg, w, p, r.tokens, 3e-2) for p, r in zip(prompts, results))
+    assert all(len(r.tokens) == 24 for r in results)
+    assert decided >= 48, "too few tokens had a margin: the check says little"      # most steps of this model are clear
+
+
+def test_the_repetition_penalty_looks_back_64_tokens_also_after_the_ring_wraps(folder_a):
+    """More than 64 generated tokens with a penalty: the device's ring of recent tokens wraps, and every choice still is
+    the plain pipeline's over the last 64 tokens."""
+    import dlgo_amd
+    from dlgo_amd.sampling import uniform
+    cfg, w = plain.read_model(folder_a)
+    llm = dlgo_amd.load_llm(folder_a, dtype="float32", max_tokens=512, max_batch=2)
+    prompts = _prompts(TINY_A, [4, 11, 2], seed=8)
+    n = 90
+    opts = [dlgo_amd.with_temperature(0.9), dlgo_amd.with_top_k(0), dlgo_amd.with_top_p(1.0), dlgo_amd.with_repetition_penalty(1.5),
+            dlgo_amd.with_seed(77), dlgo_amd.with_max_tokens(n), dlgo_amd.with_ignore_eos()]
+    results = llm.generate(prompts, *opts)
+    for i, (p, r) in enumerate(zip(prompts, results)):
+        seq, want = list(p), []
+        for step in range(n):
+            tok = plain.sample_token(plain.forward(cfg, w, seq)[-1], uniform(77, i, step), 0.9, 0, 1.0, 0.0, 1.5, want[-64:])
+            want.append(tok)
+            seq.append(tok)
+        assert r.tokens == want, i
+        # the window matters here: with the whole history penalised the run would differ
+        seq, other = list(p), []
+        for step in range(n):
+            tok = plain.sample_token(plain.forward(cfg, w, seq)[-1], uniform(77, i, step), 0.9, 0, 1.0, 0.0, 1.5, other)
+            other.append(tok)
+            seq.append(tok)
+        if i == 0:
+            assert other != want
+
+
+@pytest.mark.parametrize("options", [dict(graph_max_batch=4), dict(max_step_tokens=3), dict(use_graphs=False)])
+def test_more_sequences_than_a_recorded_step_holds(folder_a, options):
+    """Seven sequences decode together where a recorded step has fixed arrays for four (or the workspace rows for
+    three): the step runs in several runs and generation gives the plain tokens."""
+    import dlgo_amd
+    cfg, w = plain.read_model(folder_a)
+    llm = dlgo_amd.load_llm(folder_a, dtype="float32", max_tokens=1024, max_batch=7, **options)
+    prompts = _prompts(TINY_A, [5, 9, 1, 12, 3, 30, 2], seed=9)
+    results = llm.generate(prompts, dlgo_amd.with_greedy(), dlgo_amd.with_max_tokens(6), dlgo_amd.with_ignore_eos())
+    for p, r in zip(prompts, results):
+        assert r.tokens == plain.greedy_generate(cfg, w, p, 6)
+    assert llm.engine.free_slots() == llm.engine.cache.max_slots
+    b = llm.benchmark(prompts[0], dlgo_amd.with_greedy(), dlgo_amd.with_max_tokens(6), dlgo_amd.with_ignore_eos())
+    assert b.tokens == results[0].tokens and len(b.step_ms) == 1 + 6 and b.total_ms >= b.prefill_ms + b.generate_ms - 1e-3
+    assert b.architecture == "LlamaForCausalLM" and b.output_tokens == 6 and b.prompt_tokens == 5
+
+
 def test_command_line(folder_a):
     out = subprocess.run([sys.executable, "-m", "dlgo_amd", "--greedy", "--max-tokens", "4", "--dtype", "float32", "--ignore-eos",
                           "--prompt-ids", "5,6,7", "--prompt-ids", "9", folder_a], cwd=ROOT, capture_output=True, text=True,
@@ -149,6 +225,9 @@ def test_trace_replay(folder_b, tmp_path, dtype):
     steps = [{"step": i, "entries": [{"id": k, "tokens": v, "want": list(range(len(v)))}], "end": [k]}
              for i, (k, v) in enumerate(seqs.items())]
     _replay(folder_b, dtype, steps, tmp_path / "whole", 128)
+    index = json.load(open(tmp_path / "whole" / "index.json"))
+    assert index["vocab"] == V and index["dtype"] == dtype and sorted(index["steps"]) == ["0", "1", "2", "3"]
+    assert index["steps"]["2"] == {"file": "2.f32", "shape": [9, V], "rows": [["c", i] for i in range(9)]}
     for i, k in enumerate(seqs):
         got = np.fromfile(tmp_path / "whole" / f"{i}.f32", dtype="<f4").reshape(-1, V)
         assert np.abs(got - want[k]).max() <= tol * np.abs(want[k]).max()
@@ -178,6 +257,9 @@ def test_trace_replay(folder_b, tmp_path, dtype):
         n += 1
     steps.append({"step": n, "entries": [{"id": "d", "tokens": seqs["d"], "want": [99]}], "end": ["d"]})
     _replay(folder_b, dtype, steps, tmp_path / "batch", 256)
+    index = json.load(open(tmp_path / "batch" / "index.json"))
+    assert index["steps"]["0"]["rows"] == [["a", 59], ["b", 34], ["c", 0]] and index["steps"]["0"]["shape"] == [3, V]
+    assert len(index["steps"]) == len(steps)
     got0 = np.fromfile(tmp_path / "batch" / "0.f32", dtype="<f4").reshape(-1, V)
     for r, (k, p) in enumerate(first.items()):
         assert np.abs(got0[r] - want[k][p - 1]).max() <= tol * np.abs(want[k]).max()

@@ -627,7 +627,7 @@ def _sample(logits, temp, top_k=0, top_p=1.0, min_p=0.0, pen=1.0, recent=None, u
         rec = torch.tensor(recent, dtype=torch.int32, device=DEV)
     uu = torch.tensor(u if isinstance(u, list) else [u] * n, dtype=torch.float32, device=DEV)
     out = torch.empty(n, dtype=torch.int32, device=DEV)
-    ops.sample(lg, torch.empty(n, v, device=DEV), torch.empty(n, v, device=DEV), f(temp),
+    ops.sample(lg, torch.empty(n, v, device=DEV), f(temp),
                torch.full((n,), top_k, dtype=torch.int32, device=DEV), f(top_p), f(min_p), f(pen), rec, uu, out)
     return out.tolist()
 

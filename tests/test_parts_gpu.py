@@ -120,28 +120,44 @@ def test_rotary_tables_follow_the_configuration():
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("window", [None, 37])
-def test_attention_part_alone(dtype, window):
-    """Whole rows, then a continuation in pieces, for two sequences of unequal lengths, against plain attention with rotation."""
+@pytest.mark.parametrize("between", [False, True])
+def test_attention_part_alone(dtype, window, between):
+    """Whole rows, then a continuation in pieces, for two sequences of unequal lengths, against plain attention with rotation.
+    between: the layer also has what the reference puts between projection and rotation where a layer's tensors ask
+    for it (models/llm/forward.go:227-244): biases of the projections, and an RMSNorm of every q and k head over the
+    head's own elements; the output projection has a bias too."""
     from dlgo_amd.parts import Attention, Rotary
     H, KV, hd, d = 6, 2, 32, 48
+    eps = 1e-4
     g = torch.Generator().manual_seed(1)
     r = lambda *s: torch.randn(*s, generator=g)
-    att = Attention(d, H, KV, hd, Rotary(hd, 10000.0), window=window)
+    extra = dict(bias=True, out_bias=True, qk_norm_eps=eps) if between else {}
+    att = Attention(d, H, KV, hd, Rotary(hd, 10000.0), window=window, **extra)
     w = {"q_proj.weight": (0.3 * r(H * hd, d)).to(dtype), "k_proj.weight": (0.3 * r(KV * hd, d)).to(dtype),
          "v_proj.weight": (0.3 * r(KV * hd, d)).to(dtype), "o_proj.weight": (0.2 * r(d, H * hd)).to(dtype)}
+    if between:
+        w.update({"q_proj.bias": r(H * hd).to(dtype), "k_proj.bias": r(KV * hd).to(dtype), "v_proj.bias": (0.5 * r(KV * hd)).to(dtype),
+                  "o_proj.bias": (0.5 * r(d)).to(dtype), "q_norm.weight": (1 + 0.3 * r(hd)).to(dtype), "k_norm.weight": (1 + 0.3 * r(hd)).to(dtype)})
+    assert set(att.tensor_specs()) == set(w)
     att.load(w, DEV, dtype)
     att.prepare(512, torch.device(DEV))
     lens = [100, 70]
     xs = [r(n, d).to(dtype) for n in lens]
     inv = plain.rope_inv_freq(hd, 10000.0)
+    f64 = lambda name: w[name].double().numpy()
     want = []
     for x in xs:
         xd = x.double().numpy()
-        q, k, v = (xd @ w[n].double().numpy().T for n in ("q_proj.weight", "k_proj.weight", "v_proj.weight"))
+        q, k, v = (xd @ f64(n).T for n in ("q_proj.weight", "k_proj.weight", "v_proj.weight"))
+        if between:
+            q, k, v = q + f64("q_proj.bias"), k + f64("k_proj.bias"), v + f64("v_proj.bias")
+            q = plain.rmsnorm(q.reshape(-1, H, hd), f64("q_norm.weight"), eps).reshape(-1, H * hd)
+            k = plain.rmsnorm(k.reshape(-1, KV, hd), f64("k_norm.weight"), eps).reshape(-1, KV * hd)
         for t in range(len(xd)):
             q[t] = plain.rope_apply(q[t].reshape(H, hd), t, inv).reshape(-1)
             k[t] = plain.rope_apply(k[t].reshape(KV, hd), t, inv).reshape(-1)
-        want.append(plain.attention(q, k, v, H, KV, hd, window) @ w["o_proj.weight"].double().numpy().T)
+        out = plain.attention(q, k, v, H, KV, hd, window) @ f64("o_proj.weight").T
+        want.append(out + f64("o_proj.bias") if between else out)
     ctx = _Ctx(dtype, [att.cache_needs()], [60, 70], [0, 0])
     # (sequences in the step, their rows, their starts): both whole-ish, then the first goes on alone: a piece, a single row
     steps = [([0, 1], [60, 70], [0, 0]), ([0], [39], [60]), ([0], [1], [99])]
@@ -172,6 +188,8 @@ def _register_toy():
     class DecayMixer(Mixer):
         """A mixer with state of its own: s_t = decay * s_{t-1} + x_t per sequence, out_t = W s_t.
         The state lives in the cache's per-slot state area; rows of a sequence are taken in order."""
+
+        graph_safe = False       # forward() walks the step's host-side lengths and slots: nothing to record and replay
 
         def __init__(self, width, decay):
             self.width, self.decay = width, decay
@@ -366,7 +384,9 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path):
     cfg = config_from_dict(TOY)
     folder = write_random_model(cfg, 3, str(tmp_path), norm_jitter=0.1)
     _, w = plain.read_model(folder)
-    eng = Engine.from_folder(folder, "float32", max_tokens=1024, use_graphs=False)
+    # recording is asked for (the default), but one part says its launches depend on host-side numbers: every step runs as it is
+    eng = Engine.from_folder(folder, "float32", max_tokens=1024, use_graphs=True)
+    assert not eng.use_graphs and eng.eager_because == ["blocks.1.mixer"]
     assert len(eng.cache.groups) == 2 and len(eng.cache.state) == 2           # full and windowed keys/values; two runs with state
     assert eng.model.run_unit == [0, 1, 2, 3, 0] and eng.model.run_owns == [True, True, True, True, False]
     rng = np.random.default_rng(0)
@@ -387,5 +407,6 @@ def test_toy_architecture_is_registered_built_and_stepped(tmp_path):
     for t in seqs[0][50:]:
         got.append(eng.step([Entry(slot, [t], [0])]).cpu().numpy())
     assert _rel(np.concatenate(got), want[0]) <= 2e-5
+    assert not eng._graphs
     eng.close([slot])
     eng.cache.check_consistent()

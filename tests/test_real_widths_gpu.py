@@ -81,7 +81,7 @@ def test_real_widths_batches_reuse_slots_and_pages(wide, dtype, tol):
     folder, seqs, want = wide
     eng = Engine.from_folder(folder, dtype, max_tokens=192, max_slots=2)      # 70 -> two pages, 9 -> one
     err = lambda got, ref: np.abs(got.astype(np.float64) - ref).max() / np.abs(ref).max()
-    assert eng.free_pages() == 3
+    assert eng.free_pages() == (3,)
     for order in ((0, 1), (1, 0)):
         slots = eng.open(2)
         assert eng.free_slots() == 0
@@ -99,7 +99,7 @@ def test_real_widths_batches_reuse_slots_and_pages(wide, dtype, tol):
             got.append(eng.step([Entry(long_slot, [t], [0])]).cpu().numpy().copy())
         assert err(np.concatenate(got), want[0]) <= tol
         eng.close([long_slot])
-        assert eng.free_pages() == 3 and eng.free_slots() == 2
+        assert eng.free_pages() == (3,) and eng.free_slots() == 2
         eng.cache.check_consistent()
 
 
