@@ -70,11 +70,22 @@ class _Graph:
     ctx: StepContext
 
 
+@dataclass
+class _PromptGraph:
+    graph: "torch.cuda.CUDAGraph"
+    meta: torch.Tensor           # the step's int32 arrays, at the addresses the recorded kernels read
+    logits: torch.Tensor         # where the recorded step leaves its logits
+    ctx: StepContext
+
+
 class Engine:
     def __init__(self, model, dtype="bfloat16", device="cuda:0", max_tokens: int = 8192, max_ctx: Optional[int] = None,
                  max_slots: Optional[int] = None, max_step_tokens: int = 8192, logits_rows: int = 1024,
-                 use_graphs: bool = True, graph_max_batch: int = 128):
-        """`model` holds its weights already (see from_folder / from_random)."""
+                 use_graphs: bool = True, graph_max_batch: int = 128, prompt_graph_max_tokens: int = 1024,
+                 prompt_graph_limit: int = 32):
+        """`model` holds its weights already (see from_folder / from_random).  use_graphs: steps of single tokens are
+        recorded per batch size, and steps of fresh prompts of up to prompt_graph_max_tokens rows per shape (the
+        prompt_graph_limit most recently used shapes are kept), the second time a size or shape is seen."""
         _require_gpu()
         self.model = model
         self.dtype = run_dtype(dtype)
@@ -102,6 +113,11 @@ class Engine:
         self.eager_because = unsafe
         self.graph_max_batch = min(graph_max_batch, self.max_step_tokens)
         self._graphs: Dict[int, _Graph] = {}
+        # recorded steps of fresh prompts, by shape (rows per sequence, wanted places); the least recently used one goes
+        self.prompt_graph_max_tokens = prompt_graph_max_tokens
+        self.prompt_graph_limit = max(1, prompt_graph_limit)
+        self._prompt_graphs: Dict[tuple, _PromptGraph] = {}
+        self._prompt_seen: Dict[tuple, int] = {}
         self._graph_seen: Dict[int, int] = {}
         self._static: Optional[Dict[str, torch.Tensor]] = None
         self._static_logits: Optional[torch.Tensor] = None
@@ -241,14 +257,21 @@ class Engine:
         cu = np.concatenate([[0], np.cumsum(q_lens)])
         wanted = [(int(cu[i]) + w) for i, e in enumerate(entries) for w in e.want]
         n_out = len(wanted)
-        out = None
-        if sink is None:
-            out = torch.empty((n_out, self.vocab), dtype=torch.float32, device=self.device)
         wanted_arr = np.asarray(wanted, dtype=np.int64)
-
         total = int(cu[-1])
         seq_of = np.repeat(np.arange(len(entries)), q_lens)
         pos_all = np.concatenate([np.arange(s, s + n) for s, n in zip(starts, q_lens)])
+
+        # Fresh prompts of a shape seen before: the launches depend on the rows per sequence and the wanted places only,
+        # so the step is recorded the second time the shape comes and replayed from then on.
+        shape = None
+        if (self.use_graphs and sink is None and n_out and total <= min(self.max_step_tokens, self.prompt_graph_max_tokens)
+                and not any(starts)):
+            shape = (tuple(q_lens), tuple(wanted))
+        out = None
+        if sink is None and (shape is None or shape not in self._prompt_graphs):
+            out = torch.empty((n_out, self.vocab), dtype=torch.float32, device=self.device)
+
         for c0 in range(0, total, self.max_step_tokens):
             c1 = min(total, c0 + self.max_step_tokens)
             seqs = np.unique(seq_of[c0:c1])                     # sequences with rows in this piece, ascending
@@ -269,29 +292,76 @@ class Engine:
                 "cu_q": np.concatenate([[0], np.cumsum(piece_q)]).astype(np.int32),
                 "rows": (wanted_arr[sel] - c0).astype(np.int32),
             }
-            arrays = self._upload(fields)
             host = {"q_lens": piece_q, "start_pos": piece_start, "slots": slots}
-            ctx = StepContext(self, len(seqs), c1 - c0, arrays, host)
-            x = self.model.hidden(ctx, ctx.token_ids)
-            # runs of consecutive output rows, at most logits_rows each
-            i = 0
-            while i < len(sel):
-                j = i + 1
-                while j < len(sel) and sel[j] == sel[j - 1] + 1 and j - i < self.logits_rows:
-                    j += 1
-                o0 = int(sel[i])
-                if out is not None:
-                    self.model.logits(ctx, x, arrays["rows"][i:j], out[o0:o0 + (j - i)])
-                else:
-                    if self._logits_piece is None:
-                        self._logits_piece = torch.empty((self.logits_rows, self.vocab), dtype=torch.float32, device=self.device)
-                    piece = self._logits_piece[:j - i]
-                    self.model.logits(ctx, x, arrays["rows"][i:j], piece)
-                    sink(o0, piece)
-                i = j
+            if shape is not None:
+                out = self._prompt_step(shape, fields, host, len(seqs), c1 - c0, sel, out)
+            else:
+                arrays = self._upload(fields)
+                self._run_piece(StepContext(self, len(seqs), c1 - c0, arrays, host), arrays, sel, out, sink)
             for sl, q in zip(slots, piece_q):
                 self.cache.advance(int(sl), int(q))
         return out
+
+    def _run_piece(self, ctx: StepContext, arrays: Dict[str, torch.Tensor], sel: np.ndarray, out: Optional[torch.Tensor],
+                   sink: Optional[Callable[[int, torch.Tensor], None]]) -> None:
+        """The model on the rows of one piece of a step, and the logits of the wanted rows that lie in it (output rows
+        `sel`), in runs of consecutive output rows of at most logits_rows each."""
+        x = self.model.hidden(ctx, ctx.token_ids)
+        i = 0
+        while i < len(sel):
+            j = i + 1
+            while j < len(sel) and sel[j] == sel[j - 1] + 1 and j - i < self.logits_rows:
+                j += 1
+            o0 = int(sel[i])
+            if out is not None:
+                self.model.logits(ctx, x, arrays["rows"][i:j], out[o0:o0 + (j - i)])
+            else:
+                if self._logits_piece is None:
+                    self._logits_piece = torch.empty((self.logits_rows, self.vocab), dtype=torch.float32, device=self.device)
+                piece = self._logits_piece[:j - i]
+                self.model.logits(ctx, x, arrays["rows"][i:j], piece)
+                sink(o0, piece)
+            i = j
+
+    def _prompt_step(self, shape, fields: Dict[str, np.ndarray], host: Dict[str, np.ndarray], n_seq: int, n_rows: int,
+                     sel: np.ndarray, out: Optional[torch.Tensor]) -> torch.Tensor:
+        """A whole step of fresh prompts whose shape may be recorded: replayed if it is, recorded the second time it is
+        seen, run as it is the first time.  Returns the logits (the caller's own tensor)."""
+        g = self._prompt_graphs.get(shape)
+        if g is not None:
+            self._prompt_graphs[shape] = self._prompt_graphs.pop(shape)       # most recently used last
+            self._upload(fields, dest=g.meta)
+            g.graph.replay()
+            return g.logits.clone()
+        seen = self._prompt_seen.get(shape, 0) + 1
+        self._prompt_seen[shape] = seen
+        if len(self._prompt_seen) > 4096:
+            self._prompt_seen.clear()
+        if seen < 2:
+            arrays = self._upload(fields)
+            self._run_piece(StepContext(self, n_seq, n_rows, arrays, host), arrays, sel, out, None)
+            return out
+        total = sum((len(v) + 3) // 4 * 4 for v in fields.values())
+        meta = torch.zeros(total, dtype=torch.int32, device=self.device)
+        logits = torch.empty((len(sel), self.vocab), dtype=torch.float32, device=self.device)
+        arrays = self._upload(fields, dest=meta)
+        ctx = StepContext(self, n_seq, n_rows, arrays, host)
+        graph = torch.cuda.CUDAGraph()
+        torch.cuda.synchronize()
+        gc.collect()
+        was_enabled = gc.isenabled()
+        gc.disable()            # as in _capture: nothing may be collected while the stream records
+        try:
+            with torch.cuda.graph(graph):
+                self._run_piece(ctx, arrays, sel, logits, None)
+        finally:
+            if was_enabled:
+                gc.enable()
+        while len(self._prompt_graphs) >= self.prompt_graph_limit:
+            self._prompt_graphs.pop(next(iter(self._prompt_graphs)))
+        self._prompt_graphs[shape] = _PromptGraph(graph, meta, logits, ctx)
+        graph.replay()
+        return logits.clone()
 
     # -- single tokens, captured ---------------------------------------------------
     def _static_arrays(self) -> Dict[str, torch.Tensor]:

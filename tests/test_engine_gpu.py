@@ -310,3 +310,49 @@ def test_a_model_with_attention_biases(tmp_path, dtype):
     assert rel_err(np.concatenate([r.cpu().numpy() for r in rows]), want[0]) <= TOL[dtype]
     assert 1 in eng._graphs
     eng.close([slot])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prompt_steps_of_a_shape_seen_before_are_replayed(folders, oracle, dtype):
+    """A step of fresh prompts is recorded the second time its shape (rows per sequence, wanted places) comes and replayed
+    afterwards.  Every run of the shape, with other token ids each time and with other steps, other shapes and waits
+    for the device between them, gives the plain logits; only two shapes are kept, so a third pushes the oldest out."""
+    from dlgo_amd.engine import Entry
+    raw = CONFIGS["B"][0]
+    eng = engine_for(folders["B", dtype], dtype, max_tokens=4096, prompt_graph_limit=2)
+    shapes = {"x": [17, 3, 40, 1], "y": [5], "z": [64, 65]}
+
+    def run(name, seed):
+        seqs = prompts_for(raw, shapes[name], seed=seed)
+        slots = eng.open(len(seqs))
+        got = eng.step([Entry(s, t, [0, len(t) - 1] if len(t) > 1 else [0]) for s, t in zip(slots, seqs)])
+        # decoding goes on from a replayed prompt as from any other: one more token for the first sequence
+        more = eng.step([Entry(slots[0], [7], [0])])
+        torch.cuda.synchronize()
+        got, more = got.cpu().numpy(), more.cpu().numpy()
+        row = 0
+        for t in seqs:
+            want = oracle("B", dtype, t)
+            for place in ([0, len(t) - 1] if len(t) > 1 else [0]):
+                assert rel_err(got[row], want[place]) <= TOL[dtype], (name, seed, len(t), place)
+                row += 1
+        assert rel_err(more[0], oracle("B", dtype, seqs[0] + [7])[-1]) <= TOL[dtype], (name, seed)
+        eng.close(slots)
+
+    order = [("x", 1), ("y", 2), ("x", 3), ("x", 4), ("y", 5), ("z", 6), ("y", 7), ("z", 8), ("x", 9), ("x", 10), ("z", 11)]
+    for name, seed in order:
+        run(name, seed)
+    recorded = {len(k[0]) for k in eng._prompt_graphs}
+    assert len(eng._prompt_graphs) == 2 and recorded <= {4, 1, 2}
+    eng.cache.check_consistent()
+    # the same with recording switched off gives the same numbers
+    plain_eng = engine_for(folders["B", dtype], dtype, max_tokens=4096, use_graphs=False)
+    seqs = prompts_for(raw, shapes["x"], seed=3)
+    for e in (eng, plain_eng):
+        slots = e.open(4)
+        e.last = e.step([Entry(s, t, [len(t) - 1]) for s, t in zip(slots, seqs)]).cpu().numpy()
+        e.close(slots)
+    slots = eng.open(4)
+    again = eng.step([Entry(s, t, [len(t) - 1]) for s, t in zip(slots, seqs)]).cpu().numpy()     # replayed now
+    eng.close(slots)
+    assert np.array_equal(again, plain_eng.last) and np.array_equal(eng.last, plain_eng.last)

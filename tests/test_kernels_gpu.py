@@ -70,6 +70,53 @@ def test_rmsnorm_reference_vectors():
     close(out, w.double()[None] / math.sqrt(1 + 1e-5), 1e-6)
 
 
+@pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("rows,cols", [(1, 5), (9, 300), (3, 1030)])
+def test_bias_add(dtype, _, rel, rows, cols):
+    """y += b on rows in the run dtype and on float32 rows, also where the rows are a slice of wider ones
+    (ops.AddBias, ops/ops.go; used by models/llm/forward.go:227-235)."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(rows * cols)
+    wide = torch.randn(rows, cols + 7, generator=g).to(dtype).to(DEV)
+    b = torch.randn(cols, generator=g).to(DEV)
+    y = wide[:, 3:3 + cols]
+    before = wide.clone()
+    ops.bias_add(y, b)
+    close(y, before[:, 3:3 + cols].double() + b.double(), rel, "bias")
+    assert torch.equal(wide[:, :3], before[:, :3]) and torch.equal(wide[:, 3 + cols:], before[:, 3 + cols:])
+    res = torch.randn(rows, cols, generator=g).to(DEV)
+    want = res.double() + b.double()
+    ops.bias_add(res, b)
+    close(res, want, 1e-6, "bias on float32 rows")
+    with pytest.raises(ops.KernelError, match="does not fit"):
+        ops.bias_add(res, b[:-1].contiguous())
+
+
+@pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("heads,kv,hd", [(3, 1, 16), (5, 5, 80), (2, 1, 200)])
+def test_head_rmsnorm(dtype, _, rel, heads, kv, hd):
+    """Every q head and every k head normalised over its own elements with one weight vector of the head's size
+    (models/llm/forward.go:236-244); the value heads behind them stay as they are."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(heads * hd)
+    t = 6
+    qkv = (2 * torch.randn(t, (heads + 2 * kv) * hd, generator=g)).to(dtype).to(DEV)
+    wq, wk = (1 + 0.3 * torch.randn(hd, generator=g)).to(DEV), (1 + 0.3 * torch.randn(hd, generator=g)).to(DEV)
+    before = qkv.clone()
+    eps = 1e-3
+    ops.head_rmsnorm(qkv, 0, heads, hd, wq, eps)
+    ops.head_rmsnorm(qkv, heads * hd, kv, hd, wk, eps)
+
+    def plain_heads(x, n, w):
+        x = x.double().reshape(t, n, hd)
+        return (x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w.double()).reshape(t, n * hd)
+    close(qkv[:, :heads * hd], plain_heads(before[:, :heads * hd], heads, wq), rel, "q heads")
+    close(qkv[:, heads * hd:(heads + kv) * hd], plain_heads(before[:, heads * hd:(heads + kv) * hd], kv, wk), rel, "k heads")
+    assert torch.equal(qkv[:, (heads + kv) * hd:], before[:, (heads + kv) * hd:])
+    with pytest.raises(ops.KernelError, match="do not fit"):
+        ops.head_rmsnorm(qkv, hd, heads + 2 * kv, hd, wq, eps)
+
+
 GEMM_SHAPES = [(200, 37, 96), (130, 5, 40), (64, 1, 64), (388, 130, 352), (34, 8, 160), (512, 257, 128), (6, 3, 8),
                (32790, 20, 2048)]      # wide enough for the kernel that gives a block four groups of rows
 
