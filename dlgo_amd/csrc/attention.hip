@@ -834,6 +834,362 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_kernel(
   }
 }
 
+// The same step with the pages going through LDS.  attn_decode_kernel reads a page's keys as 16 rows x 64 bytes per
+// instruction and its values in 8-byte pieces, which is what the MFMA operands look like; memory gives whole 1 KB runs
+// 15 to 20% faster.  Here a wave copies its page, keys and values, into its own part of LDS with global_load_lds_dwordx4
+// (1 KB of memory in a row per instruction, no registers in between), reads the operands back from there, and asks for its
+// next page as soon as it holds them: the next page streams in while this one is multiplied.  A row's 16-byte
+// pieces sit in LDS at slot (piece ^ f(row)), which spreads the rows a quarter wave reads at once over the banks; the
+// lane that fills a slot fetches the piece that belongs there.  The keys of a page are dealt to the rows of the score
+// tiles so that the eight scores a lane ends up with belong to eight consecutive tokens (tile 2u and 2u+1, rows 4G..4G+3:
+// tokens 32u + 8G ..+7); the value operand of a lane is then one 16-byte piece.  Everything after the scores, the merge
+// of the waves and the partial results are attn_decode_kernel's.
+template <int SLOTS> struct SlotSwizzle {
+  // rows whose slots share banks get different slots: the low bits of (row >> SHIFT) are XORed into the piece number, as
+  // many bits as the number of pieces of a row has factors of two (at most four: sixteen 16-byte slots span the banks)
+  static constexpr int P2 = (SLOTS & -SLOTS) > 16 ? 16 : (SLOTS & -SLOTS);
+  static constexpr int MASK = P2 - 1;
+  static constexpr int SHIFT = P2 >= 16 ? 0 : (P2 == 8 ? 1 : (P2 == 4 ? 2 : (P2 == 2 ? 3 : 0)));
+  static __device__ __forceinline__ int of(int row) { return (row >> SHIFT) & MASK; }
+};
+
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+static __device__ __forceinline__ uint4 lds_read16(const __attribute__((address_space(3))) char* p) {
+  const u32x4_t v = *(const __attribute__((address_space(3))) u32x4_t*)p;
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+// a pointer that is the same in every lane, as the scalar registers want it
+static __device__ __forceinline__ const void* uniform_ptr(const void* p) {
+  const uint64_t v = (uint64_t)(uintptr_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+  return (const void*)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+static __device__ __forceinline__ void page_to_lds(const void* base, uint32_t voff, uint32_t lds_base) {
+  // 16 bytes per lane from base + voff to LDS at lds_base + lane * 16 (lds_base travels in M0, the same for the wave)
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(base) : "memory");
+}
+
+// what rotated8 reads, separated from what it computes, so that the loads can stand in front of a page's loads
+struct Rot8In {
+  uint4 x, p;
+  float4 c0, c1, s0, s1;
+};
+__device__ __forceinline__ Rot8In rot8_load(const bf16_t* __restrict__ vec, int d0, const float* __restrict__ cs,
+                                            const float* __restrict__ sn, int rot, int interleaved) {
+  Rot8In r;
+  r.x = *(const uint4*)(vec + d0);
+  r.p = r.x;
+  r.c0 = r.c1 = r.s0 = r.s1 = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (cs == nullptr || d0 >= rot) return r;
+  if (interleaved) {
+    r.c0 = *(const float4*)(cs + d0 / 2);
+    r.s0 = *(const float4*)(sn + d0 / 2);
+  } else {
+    const int half = rot / 2;
+    const bool low = d0 < half;
+    const int i0 = low ? d0 : d0 - half;
+    r.p = *(const uint4*)(vec + (low ? d0 + half : d0 - half));
+    r.c0 = *(const float4*)(cs + i0);
+    r.c1 = *(const float4*)(cs + i0 + 4);
+    r.s0 = *(const float4*)(sn + i0);
+    r.s1 = *(const float4*)(sn + i0 + 4);
+  }
+  return r;
+}
+__device__ __forceinline__ void unpack8(const uint4& u, float* f) {
+  f[0] = __uint_as_float(u.x << 16); f[1] = __uint_as_float(u.x & 0xffff0000u);
+  f[2] = __uint_as_float(u.y << 16); f[3] = __uint_as_float(u.y & 0xffff0000u);
+  f[4] = __uint_as_float(u.z << 16); f[5] = __uint_as_float(u.z & 0xffff0000u);
+  f[6] = __uint_as_float(u.w << 16); f[7] = __uint_as_float(u.w & 0xffff0000u);
+}
+__device__ __forceinline__ uint4 rot8_apply(const Rot8In& r, int d0, bool rotate, int rot, int interleaved) {
+  if (!rotate || d0 >= rot) return r.x;
+  float x[8], y[8];
+  unpack8(r.x, x);
+  if (interleaved) {
+    const float c[4] = {r.c0.x, r.c0.y, r.c0.z, r.c0.w}, sv[4] = {r.s0.x, r.s0.y, r.s0.z, r.s0.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      y[2 * i] = rotated_lo(x[2 * i], x[2 * i + 1], c[i], sv[i]);
+      y[2 * i + 1] = rotated_hi(x[2 * i], x[2 * i + 1], c[i], sv[i]);
+    }
+  } else {
+    const bool low = d0 < rot / 2;
+    float p[8];
+    unpack8(r.p, p);
+    const float c[8] = {r.c0.x, r.c0.y, r.c0.z, r.c0.w, r.c1.x, r.c1.y, r.c1.z, r.c1.w};
+    const float sv[8] = {r.s0.x, r.s0.y, r.s0.z, r.s0.w, r.s1.x, r.s1.y, r.s1.z, r.s1.w};
+#pragma unroll
+    for (int e = 0; e < 8; ++e) y[e] = low ? rotated_lo(x[e], p[e], c[e], sv[e]) : rotated_hi(p[e], x[e], c[e], sv[e]);
+  }
+  union { uint4 u; bf16x8_t v; } o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) o.v[e] = (__bf16)y[e];
+  return o.u;
+}
+
+template <int NWV, bool FUSED>
+__global__ __launch_bounds__(NWV* WAVE) void attn_decode_lds_kernel(
+    const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, float* __restrict__ part,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, const int32_t* __restrict__ page_table,
+    int max_pages, bf16_t* __restrict__ cache, long long page_stride, long long v_off, int n_heads, int group,
+    int head_blocks, int n_splits, int window, float scale_log2e, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, int rot, int interleaved, int new_kv, int k_col, int v_col) {
+  constexpr int HD = HEAD_DIM;
+  constexpr int KS = (HD + 31) / 32;   // k steps of K Q^T (16x16x32)
+  constexpr int DT = HD / 16;          // 16-row tiles of the output's head dimension
+  constexpr int LS = HD + 2;           // floats a wave leaves in LDS per head: values, max, sum
+  constexpr int KSLOTS = HD / 8;       // 16-byte pieces of a key row
+  constexpr int KBYTES = PAGE * HD * 2, VBYTES = HD * PAGE * 2;   // a page's keys and values of one kv head
+  constexpr int NLOAD = KBYTES / 1024;                            // 1 KB instructions for each of the two
+  using KSw = SlotSwizzle<KSLOTS>;
+  using VSw = SlotSwizzle<8>;
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int split = blockIdx.x, seq = blockIdx.z;
+  const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
+  const int pos = positions[seq];
+  const int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
+  const int first_pg = lo / PAGE, last_pg = pos / PAGE;
+  const int span = (last_pg - first_pg + n_splits) / n_splits;
+  const int pg0 = first_pg + split * span;
+  const int pg1 = pg0 + span - 1 < last_pg ? pg0 + span - 1 : last_pg;
+  if (pg0 > pg1) return;               // the whole block: fewer pages than splits
+  const int slot = slots[seq];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, j = lane & 15, G = lane >> 4;
+  const int hig = hb * 16 + j;                    // head within the group
+  const int heads_here = group - hb * 16 < 16 ? group - hb * 16 : 16;
+  const bool head_ok = j < heads_here;
+  const int head = kvh * group + hig;
+  const int32_t* my_pages = page_table + (size_t)slot * max_pages;
+
+  typedef __attribute__((address_space(3))) char lds_char;
+  lds_char* wbuf = (lds_char*)lds + (size_t)wave * (KBYTES + VBYTES);      // this wave's page: keys, then values
+  const uint32_t wbase = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)wbuf);
+  // which piece of the page each lane fetches with load number c: the one that belongs at LDS slot c * 64 + lane
+  uint32_t koff[NLOAD], voff[NLOAD];
+#pragma unroll
+  for (int c = 0; c < NLOAD; ++c) {
+    const int L = c * 64 + lane;
+    const int krow = L / KSLOTS, ks_ = L % KSLOTS;
+    koff[c] = (uint32_t)(krow * (HD * 2) + ((ks_ ^ KSw::of(krow)) << 4));
+    const int vrow = L >> 3, vs_ = L & 7;
+    voff[c] = (uint32_t)(vrow * (PAGE * 2) + ((vs_ ^ VSw::of(vrow)) << 4));
+  }
+  auto issue = [&](int page) {
+    const void* kp = uniform_ptr(cache + (size_t)page * page_stride + (size_t)kvh * PAGE * HD);
+    const void* vp = uniform_ptr(cache + v_off + (size_t)page * page_stride + (size_t)kvh * HD * PAGE);
+#pragma unroll
+    for (int c = 0; c < NLOAD; ++c) page_to_lds(kp, koff[c], wbase + c * 1024);
+#pragma unroll
+    for (int c = 0; c < NLOAD; ++c) page_to_lds(vp, voff[c], wbase + KBYTES + c * 1024);
+  };
+
+  const float* cs = cos_t ? cos_t + (size_t)pos * (rot / 2) : nullptr;
+  const float* sn = cos_t ? sin_t + (size_t)pos * (rot / 2) : nullptr;
+  // the queries' loads stand in front of the first page's; what they are turned into is computed behind them
+  Rot8In qin[KS];
+  const bf16_t* qrow = q + (size_t)seq * ldq + (size_t)(head_ok ? head : kvh * group) * HD;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d0 = ks * 32 + G * 8 < HD ? ks * 32 + G * 8 : 0;
+    qin[ks] = FUSED ? rot8_load(qrow, d0, cs, sn, rot, interleaved) : Rot8In{*(const uint4*)(qrow + d0)};
+  }
+  int pg = pg0 + wave;
+  int page_cur = pg <= pg1 ? __builtin_amdgcn_readfirstlane(my_pages[pg]) : -1;
+  int page_next = pg + NWV <= pg1 ? my_pages[pg + NWV] : -1;
+  if (page_cur >= 0) issue(page_cur);
+
+  uint4 qf[KS];
+  bool have_q = false;
+  f32x4_t o[DT];
+#pragma unroll
+  for (int d = 0; d < DT; ++d) o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int own = pos % PAGE;          // the token's own row in its page
+  const int own_t = 2 * (own >> 5) + ((own >> 2) & 1), own_j = 4 * ((own >> 3) & 3) + (own & 3);     // where it sits in the score tiles
+
+  for (; pg <= pg1; pg += NWV) {
+    const int page = page_cur;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // the page is in LDS (and the next page's number is here)
+    page_cur = __builtin_amdgcn_readfirstlane(page_next);
+    if (page < 0) {                                      // a page that is not there holds no key
+      page_next = pg + 2 * NWV <= pg1 ? my_pages[pg + 2 * NWV] : -1;
+      if (page_cur >= 0) issue(page_cur);
+      continue;
+    }
+    bf16_t* kpage = cache + (size_t)page * page_stride + (size_t)kvh * PAGE * HD;
+    bf16_t* vpage = cache + v_off + (size_t)page * page_stride + (size_t)kvh * HD * PAGE;
+    const int key0 = pg * PAGE;
+    uint4 kf[4][KS];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int row = 32 * (t >> 1) + 8 * (j >> 2) + 4 * (t & 1) + (j & 3);       // the token that is row j of score tile t
+      const lds_char* kr = wbuf + row * (HD * 2);
+      const int sw = KSw::of(row);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        kf[t][ks] = (ks * 32 + G * 8 < HD) ? lds_read16(kr + (((ks * 4 + G) ^ sw) << 4)) : make_uint4(0, 0, 0, 0);
+    }
+    uint4 vf[2][DT];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int d = 0; d < DT; ++d) {
+        const int row = d * 16 + j;
+        vf[u][d] = lds_read16(wbuf + KBYTES + row * (PAGE * 2) + (((4 * u + G) ^ VSw::of(row)) << 4));
+      }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the operands are in registers: the wave's part of LDS is free
+    page_next = pg + 2 * NWV <= pg1 ? my_pages[pg + 2 * NWV] : -1;
+    if (page_cur >= 0) issue(page_cur);
+    if (!have_q) {
+      have_q = true;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        qf[ks] = !(head_ok && ks * 32 + G * 8 < HD) ? make_uint4(0, 0, 0, 0)
+                 : rot8_apply(qin[ks], ks * 32 + G * 8, FUSED && cs != nullptr, rot, interleaved);
+    }
+    if (FUSED && new_kv && pg == last_pg) {
+      // the token's own key and value come from the step's row, not from the cache; head block 0 stores them
+      const bf16_t* row = q + (size_t)seq * ldq;
+      const bf16_t* krow_new = row + k_col + (size_t)kvh * HD;
+      const bf16_t* vrow_new = row + v_col + (size_t)kvh * HD;
+      if (j == own_j) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          if (t == own_t) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+              if (ks * 32 + G * 8 < HD) {
+                kf[t][ks] = rotated8(krow_new, ks * 32 + G * 8, cs, sn, rot, interleaved);
+                if (hb == 0) *(uint4*)(kpage + (size_t)own * HD + ks * 32 + G * 8) = kf[t][ks];
+              }
+          }
+      }
+      if (G == ((own >> 3) & 3)) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+          if (u == (own >> 5)) {
+#pragma unroll
+            for (int d = 0; d < DT; ++d) {
+              const bf16_t val = vrow_new[d * 16 + j];
+              uint32_t w4[4] = {vf[u][d].x, vf[u][d].y, vf[u][d].z, vf[u][d].w};
+              const int e = own & 7;
+#pragma unroll
+              for (int i = 0; i < 4; ++i)
+                if (i == (e >> 1)) w4[i] = (e & 1) ? ((w4[i] & 0x0000ffffu) | ((uint32_t)val << 16)) : ((w4[i] & 0xffff0000u) | val);
+              vf[u][d] = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+              if (hb == 0) vpage[(size_t)(d * 16 + j) * PAGE + own] = val;
+            }
+          }
+      }
+    }
+    f32x4_t s[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      s[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(kf[t][ks]), as_bf16x8(qf[ks]), s[t], 0, 0, 0);
+    }
+    // lane: head = lane%16; element v of tile t is key  key0 + 32 (t/2) + 8 G + 4 (t%2) + v
+    const bool need_mask = key0 + PAGE - 1 > pos || key0 < lo;
+    float mx = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        float sv = s[t][v] * scale_log2e;
+        if (need_mask) {
+          const int key = key0 + 32 * (t >> 1) + 8 * G + 4 * (t & 1) + v;
+          sv = (key <= pos && key >= lo) ? sv : -INFINITY;
+        }
+        s[t][v] = sv;
+        mx = fmaxf(mx, sv);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = fmaxf(m, mx);      // finite: every page of the range holds a valid key
+    const float alpha = fast_exp2(m - m_new);
+    float rs = 0.f;
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const float p = fast_exp2(s[t][v] - m_new);
+        s[t][v] = p;
+        rs += p;
+      }
+    rs += __shfl_xor(rs, 16, WAVE);
+    rs += __shfl_xor(rs, 32, WAVE);
+    l = l * alpha + rs;
+    m = m_new;
+#pragma unroll
+    for (int d = 0; d < DT; ++d) o[d] *= alpha;
+    const bool tail = key0 + PAGE - 1 > pos;   // keys beyond the sequence: their values must not reach the product
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {              // 32 keys each: tiles 2u and 2u+1
+      bf16x8_t pb;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        pb[e] = (__bf16)s[2 * u][e];
+        pb[4 + e] = (__bf16)s[2 * u + 1][e];
+      }
+      const int ka = key0 + 32 * u + 8 * G;    // the first of the lane's eight keys
+#pragma unroll
+      for (int d = 0; d < DT; ++d) {
+        uint4 a = vf[u][d];
+        if (tail) {
+          uint32_t* w4 = (uint32_t*)&a;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (ka + 2 * e > pos) w4[e] = 0;
+            else if (ka + 2 * e + 1 > pos) w4[e] &= 0xffffu;
+          }
+        }
+        o[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a), pb, o[d], 0, 0, 0);
+      }
+    }
+  }
+  __syncthreads();                      // every wave is done with its pages: the same LDS now takes the waves' results
+  // each wave leaves (values, max, sum) per head in LDS; a wave that saw no page leaves (0, -inf, 0)
+  if (head_ok) {
+    float* dst = lds + (size_t)(wave * heads_here + j) * LS;
+#pragma unroll
+    for (int d = 0; d < DT; ++d)
+#pragma unroll
+      for (int v = 0; v < 4; ++v) dst[d * 16 + 4 * G + v] = o[d][v];
+    if (G == 0) {
+      dst[HD] = m;
+      dst[HD + 1] = l;
+    }
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < heads_here * HD; idx += NWV * WAVE) {
+    const int hh = idx / HD, d = idx - hh * HD;
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < NWV; ++w) M = fmaxf(M, lds[(size_t)(w * heads_here + hh) * LS + HD]);
+    float L = 0.f, acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < NWV; ++w) {
+      const float* src = lds + (size_t)(w * heads_here + hh) * LS;
+      const float wt = fast_exp2(src[HD] - M);
+      L = fmaf(wt, src[HD + 1], L);
+      acc = fmaf(wt, src[d], acc);
+    }
+    const int hd_ = kvh * group + hb * 16 + hh;
+    if (n_splits == 1) {
+      out[(size_t)seq * ldo + (size_t)hd_ * HD + d] = f32_to_bf16(acc / L);
+    } else {
+      float* dst = part + ((size_t)(seq * n_heads + hd_) * n_splits + split) * (HD + 4);
+      dst[d] = acc;
+      if (d == 0) {
+        dst[HD] = M;
+        dst[HD + 1] = L;
+      }
+    }
+  }
+}
+
 // float32, one token per sequence, head sizes up to 128: attn_decode_kernel's arrangement (the pages of a split go to the
 // block's waves in turn, all heads of the group are the MFMA's 16 columns, the waves merge through LDS in wave order)
 // with v_mfma_f32_16x16x4_f32, a true float32 product, and expf.  A wave holds the keys and values of KT 16-key tiles
@@ -1178,27 +1534,30 @@ extern "C" const char* dlgo_attention_prefill_f32(const void* q, int ldq, void* 
 // max_pages_used bounds the pages of any sequence of the step (a recorded
 // launch passes the context's bound).  part: float32 scratch, used when the pages are split over several
 // blocks: n_seq * n_heads * n_splits * (hd + 4) with n_splits = dlgo_attention_decode_splits(...).
-static void decode_plan(int n_pairs, int group, int max_pages_used, bool fused, int* nwv, int* n_splits) {
+static void decode_plan(int n_pairs, int group, int max_pages_used, bool fused, bool through_lds, int* nwv, int* n_splits) {
   const int heads_here = group < 16 ? group : 16;
   const int per_wave = heads_here * (HEAD_DIM + 2) * 4;      // bytes of LDS a wave needs for the merge
   // the registers a wave needs grow with the head size (a page's keys and values are held at once), and a block
   // of w waves leaves each 2048 / w of them; the variant that rotates needs about a third more
   int w = HEAD_DIM <= 64 ? 16 : (HEAD_DIM <= 128 ? 8 : 4);
   if (fused) w >>= 1;
+  // pages through LDS: a wave's page (keys and values, 256 bytes per element of the head) times the waves within 128 KB
+  if (through_lds) w = HEAD_DIM <= 32 ? 16 : (HEAD_DIM <= 64 ? 8 : (HEAD_DIM <= 128 ? 4 : 2));
   while (w > 1 && w * per_wave > 60 * 1024) w >>= 1;
   // enough blocks to fill the chip: with few (sequence, kv head) pairs each pair's pages go to several blocks
   int splits = n_pairs >= 256 ? 1 : (256 + n_pairs - 1) / n_pairs;
   if (splits > max_pages_used) splits = max_pages_used;
   if (max_pages_used > w * 8 && splits < (max_pages_used + w * 8 - 1) / (w * 8)) splits = (max_pages_used + w * 8 - 1) / (w * 8);
-  if (splits > 1 && w > 8) w = 8;
+  if (splits > 1 && w > 8 && !through_lds) w = 8;
   *nwv = w;
   *n_splits = splits;
 }
 
-extern "C" int dlgo_attention_decode_splits(int n_seq, int n_heads, int n_kv, int max_pages_used, int fused) {
+// variant: 0 or 2 = the pages go through LDS, 1 = they are read straight into the operands' registers
+extern "C" int dlgo_attention_decode_splits(int n_seq, int n_heads, int n_kv, int max_pages_used, int fused, int variant) {
   int nwv, n_splits;
   const int group = n_heads / n_kv;
-  decode_plan(n_seq * n_kv * ((group + 15) / 16), group, max_pages_used, fused != 0, &nwv, &n_splits);
+  decode_plan(n_seq * n_kv * ((group + 15) / 16), group, max_pages_used, fused != 0, variant != 1, &nwv, &n_splits);
   return n_splits;
 }
 
@@ -1207,9 +1566,10 @@ extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, 
                                              const int32_t* slots, const int32_t* page_table, int max_pages,
                                              int max_pages_used, void* cache, long long page_stride, long long v_off,
                                              int window, float scale, const float* cos_t, const float* sin_t, int table_rows,
-                                             int rot, int interleaved, int new_kv, hipStream_t stream) {
+                                             int rot, int interleaved, int new_kv, int variant, hipStream_t stream) {
   DLGO_REQUIRE(head_dim == HEAD_DIM, "attention: this library is built for head size %d, got %d", HEAD_DIM, head_dim);
   DLGO_REQUIRE(HEAD_DIM <= 256, "attention: the split kernel takes head sizes up to 256");
+  DLGO_REQUIRE(variant >= 0 && variant <= 2, "attention: unknown variant %d of the split kernel", variant);
   DLGO_REQUIRE(n_seq >= 0 && n_heads > 0 && n_kv > 0 && n_heads % n_kv == 0, "attention: bad sizes");
   DLGO_REQUIRE(max_pages_used >= 1 && max_pages_used <= max_pages, "attention: bad bound on the pages of a sequence");
   DLGO_REQUIRE((cos_t == nullptr) == (sin_t == nullptr), "attention: cos and sin tables come together");
@@ -1223,7 +1583,8 @@ extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, 
   const int head_blocks = (group + 15) / 16;
   int nwv, n_splits;
   const bool fused = cos_t != nullptr || new_kv;
-  decode_plan(n_seq * n_kv * head_blocks, group, max_pages_used, fused, &nwv, &n_splits);
+  const bool through_lds = variant != 1;
+  decode_plan(n_seq * n_kv * head_blocks, group, max_pages_used, fused, through_lds, &nwv, &n_splits);
   DLGO_REQUIRE(n_splits == 1 || (part && part_elems >= (long long)n_seq * n_heads * n_splits * (HEAD_DIM + 4)),
                "attention: scratch for partial results too small");
   DLGO_REQUIRE((long long)n_kv * head_blocks <= 65535 && n_seq <= 65535 && n_heads <= 65535, "attention: grid too large");
@@ -1236,7 +1597,36 @@ extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, 
                      part, positions, slots, page_table, max_pages, (bf16_t*)cache, page_stride, v_off, n_heads, group,        \
                      head_blocks, n_splits, window, scale * LOG2E, cos_t, sin_t, rot, interleaved, new_kv,                    \
                      n_heads * head_dim, (n_heads + n_kv) * head_dim)
-  if (fused) {
+  if (through_lds) {
+    const size_t pages = (size_t)nwv * 2 * PAGE * HEAD_DIM * 2;       // a page's keys and values of one kv head for every wave
+    const size_t lds_bytes = pages > smem ? pages : smem;
+#define DECODE_LDS_GO(W_, F_)                                                                                                  \
+  do {                                                                                                                         \
+    auto kernel = attn_decode_lds_kernel<W_, F_>;                                                                              \
+    static bool raised = false;          /* more than 64 KB of LDS has to be asked for once per kernel */                      \
+    if (!raised) {                                                                                                             \
+      hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);         \
+      if (e != hipSuccess) DLGO_FAIL("attention: cannot get %d bytes of LDS: %s", 160 * 1024, hipGetErrorString(e));           \
+      raised = true;                                                                                                           \
+    }                                                                                                                          \
+    hipLaunchKernelGGL(kernel, grid, dim3(W_* WAVE), lds_bytes, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo, part,        \
+                       positions, slots, page_table, max_pages, (bf16_t*)cache, page_stride, v_off, n_heads, group,            \
+                       head_blocks, n_splits, window, scale* LOG2E, cos_t, sin_t, rot, interleaved, new_kv,                    \
+                       n_heads* head_dim, (n_heads + n_kv) * head_dim);                                                        \
+  } while (0)
+    if (fused) {
+      if (nwv == 16) DECODE_LDS_GO(16, true);
+      else if (nwv == 8) DECODE_LDS_GO(8, true);
+      else if (nwv == 4) DECODE_LDS_GO(4, true);
+      else DECODE_LDS_GO(2, true);
+    } else {
+      if (nwv == 16) DECODE_LDS_GO(16, false);
+      else if (nwv == 8) DECODE_LDS_GO(8, false);
+      else if (nwv == 4) DECODE_LDS_GO(4, false);
+      else DECODE_LDS_GO(2, false);
+    }
+#undef DECODE_LDS_GO
+  } else if (fused) {
     if (nwv == 8) DECODE_GO(8, true);
     else if (nwv == 4) DECODE_GO(4, true);
     else if (nwv == 2) DECODE_GO(2, true);
@@ -1276,7 +1666,7 @@ extern "C" const char* dlgo_attention_decode_f32(const void* q, int ldq, void* o
   const int group = n_heads / n_kv;
   const int head_blocks = (group + 15) / 16;
   int nwv, n_splits;
-  decode_plan(n_seq * n_kv * head_blocks, group, max_pages_used, false, &nwv, &n_splits);
+  decode_plan(n_seq * n_kv * head_blocks, group, max_pages_used, false, false, &nwv, &n_splits);
   if (nwv > 8) nwv = 8;                // a wave holds 128 registers of keys and values: two waves to a SIMD
   DLGO_REQUIRE(n_splits == 1 || (part && part_elems >= (long long)n_seq * n_heads * n_splits * (HEAD_DIM + 4)),
                "attention: scratch for partial results too small");

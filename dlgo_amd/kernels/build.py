@@ -219,7 +219,7 @@ def variant(module: str, dtype=None, defines: Defines = ()) -> Variant:
 
 
 #: head sizes compiled ahead by build_all(): those of the test configurations and of the benchmark shapes
-DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128)
+DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128, 256)
 
 
 def all_variants(head_dims: Sequence[int] = DEFAULT_HEAD_DIMS) -> list[Variant]:

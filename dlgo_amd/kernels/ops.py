@@ -384,7 +384,8 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
               v_off: int, q_lens: Sequence[int], start_pos: Sequence[int], window: int = 0,
               scale: Optional[float] = None, cu_q: Optional[torch.Tensor] = None,
               start_pos_dev: Optional[torch.Tensor] = None, scratch=None,
-              max_pages_used: Optional[int] = None, kernel: str = "auto", rotation=None, new_kv: bool = False) -> torch.Tensor:
+              max_pages_used: Optional[int] = None, kernel: str = "auto", rotation=None, new_kv: bool = False,
+              split_variant: int = 0) -> torch.Tensor:
     """Attention of a step's query rows over the cache, with the kernel chosen by the step's shape and dtype.
 
     q_lens, start_pos: per sequence, on the host (rows of the step, and the length before it).  cu_q and
@@ -395,6 +396,8 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
     rotation = (cos, sin, width, interleaved) and new_kv: only where attention_fuses_rotation() says so; then q
     holds the step's unrotated [q | k | v] rows, which the kernel rotates, and with new_kv it also takes each
     token's own key and value from its row and writes them to the cache (what rope_kv() does otherwise).
+    split_variant (bfloat16 split kernel): 0 or 2 = a page goes through LDS in whole 1 KB runs, 1 = it is read straight
+    into the operands' registers.
     """
     n_seq = len(q_lens)
     max_q = int(max(q_lens)) if n_seq else 0
@@ -449,7 +452,8 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
             if cos.shape != sin.shape or cos.shape[1] != rot_width // 2 or not cos.is_contiguous() or not sin.is_contiguous():
                 raise KernelError(f"attention: tables {tuple(cos.shape)} do not fit a rotated width of {rot_width}")
         lib.dlgo_attention_decode_splits.restype = ctypes.c_int
-        n_splits = lib.dlgo_attention_decode_splits(n_seq, n_heads, n_kv, max_pages_used, int(rotation is not None or new_kv))
+        variant = split_variant if q.dtype == torch.bfloat16 else 1
+        n_splits = lib.dlgo_attention_decode_splits(n_seq, n_heads, n_kv, max_pages_used, int(rotation is not None or new_kv), variant)
         part = None
         if n_splits > 1:
             need = n_seq * n_heads * n_splits * (head_dim + 4)
@@ -467,7 +471,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
                                          head_dim, _ptr(positions), _ptr(slots), _ptr(page_table), max_pages, max_pages_used,
                                          _ptr(cache), ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(window),
                                          ctypes.c_float(scale), _ptr(cos), _ptr(sin), cos.shape[0] if cos is not None else 0,
-                                         int(rot_width), int(interleaved), int(new_kv), _stream()))
+                                         int(rot_width), int(interleaved), int(new_kv), int(variant), _stream()))
         return out
     if kernel != "tiled":
         raise KernelError(f"attention: unknown kernel {kernel!r}")

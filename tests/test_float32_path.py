@@ -18,7 +18,7 @@ from dlgo_amd.kernels import build
 CSRC = build.CSRC
 
 # kernels that may use bfloat16 MFMA and the hardware's exp2: they only ever run on bfloat16 operands
-BF16_ONLY = {"attn_prefill_kernel", "attn_decode_kernel"}
+BF16_ONLY = {"attn_prefill_kernel", "attn_decode_kernel", "attn_decode_lds_kernel"}
 
 
 def _regions(path):

@@ -499,9 +499,11 @@ ATT_CASES = [  # H, KV, hd, window, [(cached length, rows of this step)]
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
 @pytest.mark.parametrize("H,KV,hd,window,seqs", ATT_CASES)
-@pytest.mark.parametrize("kernel", ["rows", "auto"])
+@pytest.mark.parametrize("kernel", ["rows", "auto", "registers"])
 def test_attention_over_pages(dtype, _, rel, H, KV, hd, window, seqs, kernel):
     ops = _ops()
+    if kernel == "registers" and (dtype != torch.bfloat16 or any(r != 1 for _, r in seqs)):
+        pytest.skip("the variant is the bfloat16 split kernel's: one row per sequence")
     lens = [l for l, _ in seqs]
     table, slots, storage, page_stride, unit_off, v_off = _paged_setup(dtype, lens, KV, hd, seed=hd)
     g = torch.Generator().manual_seed(H * 100 + hd)
@@ -527,18 +529,21 @@ def test_attention_over_pages(dtype, _, rel, H, KV, hd, window, seqs, kernel):
     else:
         q_lens = [r for _, r in seqs]
         starts = [l - r for l, r in seqs]
-        ops.attention(*args, q_lens=q_lens, start_pos=starts, window=window)
+        # "registers": the split kernel that reads pages straight into its operands (the default sends them through LDS)
+        ops.attention(*args, q_lens=q_lens, start_pos=starts, window=window, split_variant=1 if kernel == "registers" else 0)
     close(out, torch.from_numpy(np.concatenate(want)), rel if dtype == torch.float32 else 2e-2, "attention")
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
-@pytest.mark.parametrize("kernel", ["rows", "auto"])
+@pytest.mark.parametrize("kernel", ["rows", "auto", "registers"])
 def test_attention_finds_a_far_key_and_respects_the_window_edge(dtype, _, rel, kernel):
     """Random scores hide a key that is skipped or read twice.  Here one key among hundreds matches the query
     so strongly that the output is that key's value: the first key, one in the middle of a page, the last key
     of a page, the first of the next, the token itself; with a window, the key at its edge counts and the one just
     outside does not."""
     ops = _ops()
+    if kernel == "registers" and dtype != torch.bfloat16:
+        pytest.skip("the variant is the bfloat16 split kernel's")
     H, KV, hd = 4, 2, 32
     length = 450
     g = torch.Generator().manual_seed(9)
@@ -566,7 +571,7 @@ def test_attention_finds_a_far_key_and_respects_the_window_edge(dtype, _, rel, k
         if kernel == "rows" or len(queries) > 1:
             ops.attention_rows(*args, window=window)
         else:
-            ops.attention(*args, q_lens=[1], start_pos=positions, window=window)
+            ops.attention(*args, q_lens=[1], start_pos=positions, window=window, split_variant=1 if kernel == "registers" else 0)
         return out.float().cpu()
     tol = 1e-4 if dtype == torch.float32 else 2e-2
     for i, t in enumerate(marks):            # a single row at the last position sees every marked key
@@ -581,9 +586,11 @@ def test_attention_finds_a_far_key_and_respects_the_window_edge(dtype, _, rel, k
     assert not torch.allclose(run([4], [449], 149)[0, :hd], v[300, :hd].float(), atol=0.2)
 
 
+@pytest.mark.parametrize("variant", [0, 1])
 @pytest.mark.parametrize("H,KV,hd,rot,inter,window", [(4, 2, 16, 16, False, 0), (32, 8, 64, 64, False, 0), (6, 3, 48, 32, True, 0),
-                                                       (40, 2, 32, 32, False, 0), (8, 8, 128, 128, True, 50), (4, 1, 80, 0, False, 0)])
-def test_decode_attention_that_rotates_and_stores_by_itself(H, KV, hd, rot, inter, window):
+                                                       (40, 2, 32, 32, False, 0), (8, 8, 128, 128, True, 50), (4, 1, 80, 0, False, 0),
+                                                       (6, 2, 80, 48, False, 0), (2, 1, 256, 256, False, 0)])
+def test_decode_attention_that_rotates_and_stores_by_itself(H, KV, hd, rot, inter, window, variant):
     """One row per sequence: the split kernel given unrotated [q | k | v] rows against the two-kernel way
     (rotate and store, then attend): the same output, the same cache afterwards."""
     ops = _ops()
@@ -610,7 +617,7 @@ def test_decode_attention_that_rotates_and_stores_by_itself(H, KV, hd, rot, inte
         store = storage.clone().to(DEV)
         rows = qkv.clone().to(DEV)
         out = torch.empty(len(lens), H * hd, dtype=dtype, device=DEV)
-        common = dict(q_lens=[1] * len(lens), start_pos=[n - 1 for n in lens], window=window, kernel="split")
+        common = dict(q_lens=[1] * len(lens), start_pos=[n - 1 for n in lens], window=window, kernel="split", split_variant=variant)
         if fused:
             ops.attention(rows, out, H, KV, hd, positions, tok_seq, dslots, table.to(DEV), store[unit_off:], page_stride, v_off,
                           rotation=(cos, sin, rot, inter) if rot else None, new_kv=True, **common)
