@@ -858,12 +858,6 @@ static __device__ __forceinline__ uint4 lds_read16(const __attribute__((address_
   const u32x4_t v = *(const __attribute__((address_space(3))) u32x4_t*)p;
   return make_uint4(v.x, v.y, v.z, v.w);
 }
-// a pointer that is the same in every lane, as the scalar registers want it
-static __device__ __forceinline__ const void* uniform_ptr(const void* p) {
-  const uint64_t v = (uint64_t)(uintptr_t)p;
-  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-  return (const void*)(uintptr_t)(((uint64_t)hi << 32) | lo);
-}
 static __device__ __forceinline__ void page_to_lds(const void* base, uint32_t voff, uint32_t lds_base) {
   // 16 bytes per lane from base + voff to LDS at lds_base + lane * 16 (lds_base travels in M0, the same for the wave)
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(base) : "memory");

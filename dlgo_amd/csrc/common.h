@@ -31,6 +31,15 @@ __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
 __device__ __forceinline__ float rotated_lo(float x0, float x1, float c, float s) { return __builtin_fmaf(-x1, s, x0 * c); }
 __device__ __forceinline__ float rotated_hi(float x0, float x1, float c, float s) { return __builtin_fmaf(x0, s, x1 * c); }
 
+// A pointer that is the same in every lane of the wave, made so for an instruction that wants it in scalar registers.
+// The halves are taken as unsigned: readfirstlane returns an int, which would be sign-extended into the upper half.
+__device__ __forceinline__ const void* uniform_ptr(const void* p) {
+  const uint64_t v = (uint64_t)(uintptr_t)p;
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+  return (const void*)(uintptr_t)(((uint64_t)hi << 32) | (uint64_t)lo);
+}
+
 template <typename T> struct Elem;
 template <> struct Elem<float> {
   static constexpr int code = DLGO_DTYPE_F32;

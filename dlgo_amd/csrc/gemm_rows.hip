@@ -255,6 +255,180 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_kernel(const T* __restrict__ 
     }
 }
 
+// The same product for rows of W that are a whole number of kilobytes, with W going through LDS.  skinny_kernel reads
+// W as 16 rows x 64 bytes per instruction, which is what the MFMA's row operand looks like; memory gives whole 1 KB runs
+// about 20% faster on a matrix of tens of megabytes.  Here a block owns 16 rows, wave w their w-th kilobyte: sixteen
+// global_load_lds_dwordx4, one row's kilobyte each, straight into the wave's own 16 KB of LDS, and the operands come back
+// with ds_read_b128.  A row's 16-byte pieces sit at slot (piece ^ row), so that the sixteen rows a quarter wave reads at
+// once lie in different banks; the lane that fills a slot fetches the piece that belongs there.  X, the sums over the
+// waves and the epilogue are skinny_kernel's (up to 16 tokens).
+static __device__ __forceinline__ void row_to_lds(const void* base, uint32_t voff, uint32_t lds_base) {
+  // 16 bytes per lane from base + voff to LDS at lds_base + lane * 16 (lds_base travels in M0, the same for the wave)
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(base) : "memory");
+}
+typedef uint32_t rows_u32x4_t __attribute__((ext_vector_type(4)));
+
+template <typename T, int NW, int EPI, bool NORM>
+__global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __restrict__ W, const void* __restrict__ Xv,
+                                                                  const float* __restrict__ norm_w, float eps,
+                                                                  void* __restrict__ Y, int N, int Tn, int K, int ldw, int ldx,
+                                                                  int ldy) {
+  constexpr int EPC = 16 / sizeof(T);          // elements of a 16-byte operand
+  constexpr int CH = 1024 / sizeof(T);         // elements of a row's kilobyte
+  constexpr int STEPS = 16;                    // MFMA steps of a kilobyte: four 16-byte pieces each
+  typedef __attribute__((address_space(3))) char lds_char;
+  extern __shared__ __attribute__((aligned(16))) char lds_raw[];
+  lds_char* wbuf = (lds_char*)lds_raw + (size_t)(threadIdx.x >> 6) * 16384;
+  const uint32_t wbase = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)wbuf);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int j = lane & 15, G = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int k0 = wave * CH;                    // this wave's part of k
+  // load c brings row c's kilobyte; the lane fetches the piece that belongs at its slot.  Rows beyond N repeat the last.
+  {
+    const char* base = (const char*)uniform_ptr(W + (size_t)n0 * ldw + k0);
+    const uint32_t last_row = (uint32_t)(N - 1 - n0);
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+      const uint32_t row = (uint32_t)c < last_row ? (uint32_t)c : last_row;
+      row_to_lds(base, row * (uint32_t)ldw * (uint32_t)sizeof(T) + (uint32_t)((lane ^ c) << 4), wbase + c * 1024);
+    }
+  }
+  f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float ss = 0.f;
+  const lds_char* arow = wbuf + j * 1024;
+  const bool tok = j < Tn;
+  auto products = [&](int half, const uint4* b) {        // eight steps of the wave's kilobyte against eight operands of X
+#pragma unroll
+    for (int s_ = 0; s_ < STEPS / 2; ++s_) {
+      const int piece = (half * (STEPS / 2) + s_) * 4 + G;
+      const rows_u32x4_t a4 = *(const __attribute__((address_space(3))) rows_u32x4_t*)(arow + ((piece ^ j) << 4));
+      Mma16<T>::run(make_uint4(a4.x, a4.y, a4.z, a4.w), b[s_], acc);
+    }
+  };
+  if (NORM) {
+    // x and the norm's weights in two halves (the registers do not hold both): the second half is on its way while the
+    // first is multiplied.  The wait counts the second half's loads: everything older, W's kilobytes first of all, is there.
+    const float* xr = (const float*)Xv + (size_t)(tok ? j : 0) * ldx + k0;
+    constexpr int HALF_LOADS = (STEPS / 2) * (EPC / 4) * 2;
+    float4 xv[2][STEPS / 2][EPC / 4], wv[2][STEPS / 2][EPC / 4];
+    uint4 b[STEPS / 2];
+    auto fetch = [&](int half) {
+#pragma unroll
+      for (int s_ = 0; s_ < STEPS / 2; ++s_) {
+        const int k = (half * (STEPS / 2) + s_) * 4 * EPC + G * EPC;
+#pragma unroll
+        for (int e = 0; e < EPC / 4; ++e) {
+          xv[half][s_][e] = *(const float4*)(xr + k + 4 * e);
+          wv[half][s_][e] = *(const float4*)(norm_w + k0 + k + 4 * e);
+        }
+      }
+    };
+    auto pack = [&](int half) {
+#pragma unroll
+      for (int s_ = 0; s_ < STEPS / 2; ++s_) {
+        float f[EPC];
+#pragma unroll
+        for (int e = 0; e < EPC / 4; ++e) {
+          const float4 x4 = xv[half][s_][e], w4 = wv[half][s_][e];
+          ss = fmaf(x4.x, x4.x, ss);
+          ss = fmaf(x4.y, x4.y, ss);
+          ss = fmaf(x4.z, x4.z, ss);
+          ss = fmaf(x4.w, x4.w, ss);
+          f[4 * e] = x4.x * w4.x;
+          f[4 * e + 1] = x4.y * w4.y;
+          f[4 * e + 2] = x4.z * w4.z;
+          f[4 * e + 3] = x4.w * w4.w;
+        }
+        b[s_] = tok ? Mma16<T>::pack(f) : make_uint4(0, 0, 0, 0);
+      }
+    };
+    fetch(0);
+    pack(0);
+    fetch(1);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(HALF_LOADS) : "memory");
+    products(0, b);
+    pack(1);
+    products(1, b);
+  } else {
+    const T* xr = (const T*)Xv + (size_t)(tok ? j : 0) * ldx + k0;
+    uint4 b[STEPS];
+#pragma unroll
+    for (int s_ = 0; s_ < STEPS; ++s_) {
+      const uint4 v = *(const uint4*)(xr + s_ * 4 * EPC + G * EPC);
+      b[s_] = tok ? v : make_uint4(0, 0, 0, 0);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // the wave's kilobytes are in LDS, and its part of X is here
+    products(0, b);
+    products(1, b + STEPS / 2);
+  }
+  // lane: token j, rows 4 G + v.  The waves' partial sums go through LDS (the rows' place, once every wave is done with
+  // them); wave 0 adds them in wave order.
+  __syncthreads();
+  float* red = (float*)lds_raw;                // [NW][16][17]
+  float* ssq = red + NW * 16 * 17;             // [NW][16]
+#pragma unroll
+  for (int v = 0; v < 4; ++v) red[(wave * 16 + 4 * G + v) * 17 + j] = acc[v];
+  if (NORM) {
+    float s2 = ss;
+    s2 += __shfl_xor(s2, 16, WAVE);
+    s2 += __shfl_xor(s2, 32, WAVE);
+    if (G == 0) ssq[wave * 16 + j] = s2;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int w = 0; w < NW; ++w)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] += red[(w * 16 + 4 * G + q) * 17 + j];
+    if (NORM) {
+      float s2 = 0.f;
+      for (int w = 0; w < NW; ++w) s2 += ssq[w * 16 + j];
+      const float sc = 1.0f / sqrtf(s2 / (float)K + eps);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) v[q] *= sc;
+    }
+    if (tok) epilogue4<T, EPI>(Y, ldy, N, j, n0 + 4 * G, v[0], v[1], v[2], v[3]);
+  }
+}
+
+// Whether skinny_stream_kernel takes a product, and with how many waves: up to 16 tokens, rows of 2 to 8 whole kilobytes
+// (a wave keeps 16 KB of LDS; eight of them fill a compute unit's).
+template <typename T>
+static int stream_waves(int Tn, int K, int ldw) {
+  const long long bytes = (long long)K * sizeof(T);
+  if (Tn < 1 || Tn > 16 || bytes % 1024 || bytes < 2048 || bytes > 8192) return 0;
+  if ((long long)ldw * sizeof(T) * 16 >= (1ll << 32)) return 0;
+  const int nw = (int)(bytes / 1024);
+  return nw == 2 || nw == 3 || nw == 4 || nw == 6 || nw == 8 ? nw : 0;
+}
+
+template <typename T, int EPI, bool NORM>
+static const char* launch_skinny_stream(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K,
+                                        int ldw, int ldx, int ldy, int nw, hipStream_t stream) {
+  dim3 g((N + 15) / 16);
+#define STREAM_GO(NW_)                                                                                                          \
+  do {                                                                                                                          \
+    auto kernel = skinny_stream_kernel<T, NW_, EPI, NORM>;                                                                      \
+    static bool raised = false;          /* more than 64 KB of LDS has to be asked for once per kernel */                       \
+    if (NW_ * 16384 > 65536 && !raised) {                                                                                       \
+      hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, NW_ * 16384);         \
+      if (e != hipSuccess) DLGO_FAIL("gemm_rows: cannot get %d bytes of LDS: %s", NW_ * 16384, hipGetErrorString(e));           \
+      raised = true;                                                                                                            \
+    }                                                                                                                           \
+    hipLaunchKernelGGL(kernel, g, dim3(NW_* WAVE), NW_ * 16384, stream, (const T*)W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy); \
+  } while (0)
+  switch (nw) {
+    case 2: STREAM_GO(2); break;
+    case 3: STREAM_GO(3); break;
+    case 4: STREAM_GO(4); break;
+    case 6: STREAM_GO(6); break;
+    default: STREAM_GO(8); break;
+  }
+#undef STREAM_GO
+  return nullptr;
+}
+
 template <typename T, int NW, int R, int EPI, bool NORM>
 static void launch_skinny_nw(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K, int ldw,
                              int ldx, int ldy, hipStream_t stream) {
@@ -271,11 +445,19 @@ static void launch_skinny_nw(const void* W, const void* X, const float* norm_w, 
 // The number of waves that share a block's rows is a function of N and K alone, so the order of the sums does
 // not depend on the step (few rows of long k: 16 waves, so that the few blocks keep more loads in flight).  force_nw (1, 2, 4, 8) is for tuning and tests.
 template <typename T, int EPI, bool NORM>
-static void launch_skinny(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K, int ldw,
-                          int ldx, int ldy, hipStream_t stream, int force_nw = 0) {
+static const char* launch_skinny(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K, int ldw,
+                                 int ldx, int ldy, hipStream_t stream, int force_nw = 0) {
   const int pieces = (K * (int)sizeof(T) + 127) / 128;
   int nw = pieces >= 128 && N <= 4096 ? 16 : (pieces >= 32 ? 8 : (pieces >= 16 ? 4 : (pieces >= 8 ? 2 : 1)));
-  if (force_nw) nw = force_nw;
+  // rows of whole kilobytes and few tokens: W goes through LDS in whole 1 KB runs, where the matrix is large enough
+  // for that to pay (force_nw 32 asks for it wherever it applies, 64 rules it out; other values choose the waves)
+  // (measured on the products of 1B to 8B Llamas: with X in the run dtype it wins for every matrix; with the norm riding
+  // in the product, whose float32 x and weights are four times the loads, it loses)
+  const int sw = stream_waves<T>(Tn, K, ldw);
+  if (sw && (force_nw == 32 || (force_nw == 0 && !NORM))) {
+    return launch_skinny_stream<T, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, sw, stream);
+  }
+  if (force_nw && force_nw < 32) nw = force_nw;
   // many rows: each block takes 2 or 4 groups of 16, which divides the traffic of X (a function of N alone)
   const bool wide = N >= 32768 && nw == 8, mid = N >= 8192 && nw == 8;
   if (nw == 16) launch_skinny_nw<T, 16, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
@@ -285,6 +467,7 @@ static void launch_skinny(const void* W, const void* X, const float* norm_w, flo
   else if (nw == 4) launch_skinny_nw<T, 4, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
   else if (nw == 2) launch_skinny_nw<T, 2, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
   else launch_skinny_nw<T, 1, 1, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream);
+  return nullptr;
 }
 
 template <typename T, int EPI>
@@ -299,21 +482,27 @@ static void launch_gemv(const void* W, const void* X, void* Y, int N, int Tn, in
 }
 
 template <typename T, int EPI>
-static void dispatch_rows(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy, int kind,
-                          hipStream_t stream) {
-  // kind: 0 = the MFMA kernel, 1 = the vector kernel (at most 8 rows), 6..9 = the MFMA kernel with 1, 2, 4, 8 waves per block
-  if (kind == 1) launch_gemv<T, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
-  else launch_skinny<T, EPI, false>(W, X, nullptr, 0.f, Y, N, Tn, K, ldw, ldx, ldy, stream, kind == 0 ? 0 : 1 << (kind - 6));
+static const char* dispatch_rows(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy, int kind,
+                                 hipStream_t stream) {
+  // kind: 0 = the MFMA kernels, 1 = the vector kernel (at most 8 rows), 6..9 = the MFMA kernel that reads W into registers,
+  // with 1, 2, 4, 8 waves per block, 10 = the MFMA kernel that sends W through LDS (where it applies, else as 0),
+  // 11 = never that one
+  if (kind == 1) {
+    launch_gemv<T, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
+    return nullptr;
+  }
+  return launch_skinny<T, EPI, false>(W, X, nullptr, 0.f, Y, N, Tn, K, ldw, ldx, ldy, stream,
+                                      kind == 0 ? 0 : (kind == 10 ? 32 : (kind == 11 ? 64 : 1 << (kind - 6))));
 }
 
 template <typename T>
 static const char* rows_by_epilogue(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy,
                                     int epi, int kind, hipStream_t stream) {
   switch (epi) {
-    case EPI_STORE: dispatch_rows<T, EPI_STORE>(W, X, Y, N, Tn, K, ldw, ldx, ldy, kind, stream); break;
-    case EPI_ACCUM_F32: dispatch_rows<T, EPI_ACCUM_F32>(W, X, Y, N, Tn, K, ldw, ldx, ldy, kind, stream); break;
-    case EPI_SWIGLU: dispatch_rows<T, EPI_SWIGLU>(W, X, Y, N, Tn, K, ldw, ldx, ldy, kind, stream); break;
-    case EPI_STORE_F32: dispatch_rows<T, EPI_STORE_F32>(W, X, Y, N, Tn, K, ldw, ldx, ldy, kind, stream); break;
+    case EPI_STORE: return dispatch_rows<T, EPI_STORE>(W, X, Y, N, Tn, K, ldw, ldx, ldy, kind, stream);
+    case EPI_ACCUM_F32: return dispatch_rows<T, EPI_ACCUM_F32>(W, X, Y, N, Tn, K, ldw, ldx, ldy, kind, stream);
+    case EPI_SWIGLU: return dispatch_rows<T, EPI_SWIGLU>(W, X, Y, N, Tn, K, ldw, ldx, ldy, kind, stream);
+    case EPI_STORE_F32: return dispatch_rows<T, EPI_STORE_F32>(W, X, Y, N, Tn, K, ldw, ldx, ldy, kind, stream);
     default: DLGO_FAIL("gemm_rows: unknown epilogue %d", epi);
   }
   return nullptr;
@@ -332,7 +521,7 @@ extern "C" const char* dlgo_gemm_rows(const void* W, const void* X, void* Y, int
   DLGO_REQUIRE(((uintptr_t)Y & 3) == 0 || (dtype == DLGO_DTYPE_BF16 && ((uintptr_t)Y & 1) == 0), "gemm: Y must be aligned to its elements");
   DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm: SwiGLU epilogue needs an even N and ldy >= N/2");
   DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm: ldy %d shorter than N %d", ldy, N);
-  DLGO_REQUIRE(kind == 0 || kind == 1 || (kind >= 6 && kind <= 9), "gemm_rows: unknown kernel choice %d", kind);
+  DLGO_REQUIRE(kind == 0 || kind == 1 || (kind >= 6 && kind <= 11), "gemm_rows: unknown kernel choice %d", kind);
   DLGO_REQUIRE(kind != 1 || Tn <= 8, "gemm: the vector kernel takes at most 8 rows, got %d", Tn);
   if (Tn == 0) return nullptr;
   const char* err = rows_by_epilogue<elem_t>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, kind, stream);
@@ -343,8 +532,10 @@ extern "C" const char* dlgo_gemm_rows(const void* W, const void* X, void* Y, int
 
 // Y (epilogue)= (rmsnorm(X) * norm_w) W^T for up to 64 rows of the float32 residual stream X [T, K], without
 // writing the normed rows.  Epilogues as dlgo_gemm.
+// kind: 0 = the kernel is chosen by the shape, 10 = W through LDS wherever that applies, 11 = never.
 extern "C" const char* dlgo_gemm_rmsnorm(const void* W, const float* X, const float* norm_w, float eps, void* Y, int dtype, int N,
-                                         int Tn, int K, int ldw, int ldx, int ldy, int epilogue, hipStream_t stream) {
+                                         int Tn, int K, int ldw, int ldx, int ldy, int epilogue, int kind, hipStream_t stream) {
+  DLGO_REQUIRE(kind == 0 || kind == 10 || kind == 11, "gemm_rmsnorm: unknown kernel choice %d", kind);
   DLGO_REQUIRE(N > 0 && Tn >= 0 && Tn <= 64 && K > 0, "gemm_rmsnorm: bad sizes N=%d T=%d K=%d (at most 64 rows)", N, Tn, K);
   DLGO_REQUIRE(dtype == DLGO_ELEM, "gemm_rmsnorm: this library is built for dtype code %d, got %d", DLGO_ELEM, dtype);
   const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
@@ -355,15 +546,18 @@ extern "C" const char* dlgo_gemm_rmsnorm(const void* W, const float* X, const fl
   DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm_rmsnorm: SwiGLU epilogue needs an even N and ldy >= N/2");
   DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm_rmsnorm: ldy %d shorter than N %d", ldy, N);
   if (Tn == 0) return nullptr;
-#define NORM_GO(E_) launch_skinny<elem_t, E_, true>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream)
+  const int force = kind == 0 ? 0 : (kind == 10 ? 32 : 64);
+#define NORM_GO(E_) launch_skinny<elem_t, E_, true>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, stream, force)
+  const char* err = nullptr;
   switch (epilogue) {
-    case EPI_STORE: NORM_GO(EPI_STORE); break;
-    case EPI_ACCUM_F32: NORM_GO(EPI_ACCUM_F32); break;
-    case EPI_SWIGLU: NORM_GO(EPI_SWIGLU); break;
-    case EPI_STORE_F32: NORM_GO(EPI_STORE_F32); break;
+    case EPI_STORE: err = NORM_GO(EPI_STORE); break;
+    case EPI_ACCUM_F32: err = NORM_GO(EPI_ACCUM_F32); break;
+    case EPI_SWIGLU: err = NORM_GO(EPI_SWIGLU); break;
+    case EPI_STORE_F32: err = NORM_GO(EPI_STORE_F32); break;
     default: DLGO_FAIL("gemm_rmsnorm: unknown epilogue %d", epilogue);
   }
 #undef NORM_GO
+  if (err) return err;
   DLGO_LAUNCH_CHECK("gemm_rmsnorm");
   return nullptr;
 }

@@ -151,9 +151,12 @@ def _streams_rows(weight: torch.Tensor, t: int, kind: int, has_scratch: bool, sp
     nk = k // piece if k % piece == 0 else 0
     can_split = has_scratch and splits != 1 and nk >= 32 and n <= 4096
     if kind != GEMM_AUTO or splits > 1:
-        return kind in (GEMM_STREAM, 5, 6, 7, 8, 9)
+        return kind in (GEMM_STREAM, 5, 6, 7, 8, 9, 10, 11)
     if t <= GEMM_FEW_ROWS_WIDE:         # measured on the shapes of a 1B Llama: a long inner size is better split,
-        return not (can_split and nk >= 64) and not (n >= GEMM_VERY_WIDE and nk > 0)   # a vocabulary better tiled
+        row_kb = k * weight.element_size() / 1024.0
+        if t <= 8 and n >= GEMM_VERY_WIDE and row_kb in (2.0, 3.0, 4.0, 6.0, 8.0):
+            return True                 # a vocabulary of rows that go through LDS whole: streamed faster than tiled
+        return not (can_split and nk >= 64) and not (n >= GEMM_VERY_WIDE and nk > 0)   # else a vocabulary is better tiled
     if t <= GEMM_FEW_ROWS:
         return n < 16384 and not (can_split and (nk >= 64 or t >= 24)) and (t <= 40 or nk == 0)
     return False
@@ -270,9 +273,10 @@ def fused_norm_pays(weight: torch.Tensor, rows: int) -> bool:
 
 
 def gemm_rmsnorm(weight: torch.Tensor, x: torch.Tensor, norm_weight: torch.Tensor, eps: float, out: torch.Tensor,
-                 epilogue: int = EPI_STORE) -> torch.Tensor:
+                 epilogue: int = EPI_STORE, kind: int = GEMM_AUTO) -> torch.Tensor:
     """out (epilogue)= (rmsnorm(x) * norm_weight) @ weight.T for up to 64 rows x of the float32 residual stream,
-    without writing the normed rows.  Epilogues as gemm()."""
+    without writing the normed rows.  Epilogues as gemm().  kind: 0 = chosen by the shape, 10 = the weights go through
+    LDS in whole 1 KB runs wherever that kernel applies (up to 16 rows, weight rows of 2 to 16 whole KB), 11 = never."""
     _need(weight, "gemm weight", dims=2)
     _need(x, "residual rows", torch.float32, 2)
     _need(norm_weight, "norm weight", torch.float32, 1)
@@ -287,7 +291,7 @@ def gemm_rmsnorm(weight: torch.Tensor, x: torch.Tensor, norm_weight: torch.Tenso
         raise KernelError(f"gemm_rmsnorm: output {tuple(out.shape)}, expected {(t, cols)}")
     _check(_lib("gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),)).dlgo_gemm_rmsnorm(_ptr(weight), _ptr(x), _ptr(norm_weight), ctypes.c_float(eps), _ptr(out),
                                           dtype_code(weight.dtype), n, t, k, _rows(weight, "gemm weight"),
-                                          _rows(x, "residual rows"), _rows(out, "gemm output"), epilogue, _stream()))
+                                          _rows(x, "residual rows"), _rows(out, "gemm output"), epilogue, kind, _stream()))
     return out
 
 

@@ -118,15 +118,17 @@ def test_head_rmsnorm(dtype, _, rel, heads, kv, hd):
 
 
 GEMM_SHAPES = [(200, 37, 96), (130, 5, 40), (64, 1, 64), (388, 130, 352), (34, 8, 160), (512, 257, 128), (6, 3, 8),
-               (32790, 20, 2048)]      # wide enough for the kernel that gives a block four groups of rows
+               (32790, 20, 2048),      # wide enough for the kernel that gives a block four groups of rows
+               # few tokens and weight rows of whole kilobytes (2, 3, 6 and 16 KB in bfloat16): these go through LDS
+               (100, 11, 1024), (8200, 16, 1536), (40, 3, 3072), (72, 1, 8192), (50, 8, 512)]
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
-@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 12, 14])
+@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 14])
 @pytest.mark.parametrize("n,t,k", GEMM_SHAPES)
 def test_gemm_store_and_accumulate(dtype, _, rel, kind, n, t, k):
     ops = _ops()
-    if (kind == 1 and t > 8) or (5 <= kind <= 9 and t > 64):
+    if (kind == 1 and t > 8) or (5 <= kind <= 11 and t > 64):
         pytest.skip("the streaming kernels take a few rows only")
     if dtype == torch.bfloat16 and k % 8:
         pytest.skip("bfloat16 rows come in 16-byte pieces")
@@ -275,9 +277,12 @@ def test_gemm_swiglu(dtype, _, rel, kind, f, t, k):
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
-@pytest.mark.parametrize("n,t,k", [(200, 8, 96), (130, 1, 40), (96, 17, 2048), (388, 64, 352), (34, 48, 160), (32780, 3, 2048)])
-def test_gemm_with_fused_rmsnorm(dtype, _, rel, n, t, k):
-    """The product with the normed rows that are never written, in every epilogue."""
+@pytest.mark.parametrize("kind", [0, 10, 11])
+@pytest.mark.parametrize("n,t,k", [(200, 8, 96), (130, 1, 40), (96, 17, 2048), (388, 64, 352), (34, 48, 160), (32780, 3, 2048),
+                                   (8204, 9, 1024), (72, 16, 1536), (100, 1, 4096), (50, 7, 3072), (40, 5, 512)])
+def test_gemm_with_fused_rmsnorm(dtype, _, rel, n, t, k, kind):
+    """The product with the normed rows that are never written, in every epilogue, by both kernels (the weights read
+    straight into registers; the weights going through LDS in whole 1 KB runs, for the shapes that kernel takes)."""
     ops = _ops()
     g = torch.Generator().manual_seed(n + t)
     w = (0.5 * torch.randn(n, k, generator=g)).to(dtype).to(DEV)
@@ -289,17 +294,17 @@ def test_gemm_with_fused_rmsnorm(dtype, _, rel, n, t, k):
     want = xn @ w.double().T
     tol = 1e-5 if dtype == torch.float32 else 1.5e-2
     out = torch.empty(t, n, dtype=dtype, device=DEV)
-    ops.gemm_rmsnorm(w, x, nw, eps, out)
+    ops.gemm_rmsnorm(w, x, nw, eps, out, kind=kind)
     close(out, want, tol, "store")
     out32 = torch.empty(t, n, device=DEV)
-    ops.gemm_rmsnorm(w, x, nw, eps, out32, ops.EPI_STORE_F32)
+    ops.gemm_rmsnorm(w, x, nw, eps, out32, ops.EPI_STORE_F32, kind=kind)
     close(out32, want, tol, "store f32")
     res = torch.randn(t, n, generator=g).to(DEV)
     res0 = res.clone()
-    ops.gemm_rmsnorm(w, x, nw, eps, res, ops.EPI_ACCUM_F32)
+    ops.gemm_rmsnorm(w, x, nw, eps, res, ops.EPI_ACCUM_F32, kind=kind)
     close(res, res0.double() + want, tol, "accumulate")
     hid = torch.empty(t, n // 2, dtype=dtype, device=DEV)
-    ops.gemm_rmsnorm(w, x, nw, eps, hid, ops.EPI_SWIGLU)
+    ops.gemm_rmsnorm(w, x, nw, eps, hid, ops.EPI_SWIGLU, kind=kind)
     gd, ud = want[:, 0::2], want[:, 1::2]
     close(hid, gd / (1 + torch.exp(-gd)) * ud, tol * 2, "swiglu")
 
