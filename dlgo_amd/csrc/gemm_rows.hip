@@ -10,6 +10,7 @@
 //
 // Every reduction order is a function of N and K alone: a row of Y never depends on the other rows of the step.
 #include "gemm_common.h"
+#include <initializer_list>
 
 // ----------------------------------------------------------------------------
 // weight-streaming kernel for up to 8 tokens
@@ -268,9 +269,8 @@ static __device__ __forceinline__ void row_to_lds(const void* base, uint32_t vof
 }
 typedef uint32_t rows_u32x4_t __attribute__((ext_vector_type(4)));
 
-template <typename T, int NW, int EPI, bool NORM>
+template <typename T, int NW, int EPI>
 __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __restrict__ W, const void* __restrict__ Xv,
-                                                                  const float* __restrict__ norm_w, float eps,
                                                                   void* __restrict__ Y, int N, int Tn, int K, int ldw, int ldx,
                                                                   int ldy) {
   constexpr int EPC = 16 / sizeof(T);          // elements of a 16-byte operand
@@ -295,7 +295,6 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __rest
     }
   }
   f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  float ss = 0.f;
   const lds_char* arow = wbuf + j * 1024;
   const bool tok = j < Tn;
   auto products = [&](int half, const uint4* b) {        // eight steps of the wave's kilobyte against eight operands of X
@@ -306,51 +305,7 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __rest
       Mma16<T>::run(make_uint4(a4.x, a4.y, a4.z, a4.w), b[s_], acc);
     }
   };
-  if (NORM) {
-    // x and the norm's weights in two halves (the registers do not hold both): the second half is on its way while the
-    // first is multiplied.  The wait counts the second half's loads: everything older, W's kilobytes first of all, is there.
-    const float* xr = (const float*)Xv + (size_t)(tok ? j : 0) * ldx + k0;
-    constexpr int HALF_LOADS = (STEPS / 2) * (EPC / 4) * 2;
-    float4 xv[2][STEPS / 2][EPC / 4], wv[2][STEPS / 2][EPC / 4];
-    uint4 b[STEPS / 2];
-    auto fetch = [&](int half) {
-#pragma unroll
-      for (int s_ = 0; s_ < STEPS / 2; ++s_) {
-        const int k = (half * (STEPS / 2) + s_) * 4 * EPC + G * EPC;
-#pragma unroll
-        for (int e = 0; e < EPC / 4; ++e) {
-          xv[half][s_][e] = *(const float4*)(xr + k + 4 * e);
-          wv[half][s_][e] = *(const float4*)(norm_w + k0 + k + 4 * e);
-        }
-      }
-    };
-    auto pack = [&](int half) {
-#pragma unroll
-      for (int s_ = 0; s_ < STEPS / 2; ++s_) {
-        float f[EPC];
-#pragma unroll
-        for (int e = 0; e < EPC / 4; ++e) {
-          const float4 x4 = xv[half][s_][e], w4 = wv[half][s_][e];
-          ss = fmaf(x4.x, x4.x, ss);
-          ss = fmaf(x4.y, x4.y, ss);
-          ss = fmaf(x4.z, x4.z, ss);
-          ss = fmaf(x4.w, x4.w, ss);
-          f[4 * e] = x4.x * w4.x;
-          f[4 * e + 1] = x4.y * w4.y;
-          f[4 * e + 2] = x4.z * w4.z;
-          f[4 * e + 3] = x4.w * w4.w;
-        }
-        b[s_] = tok ? Mma16<T>::pack(f) : make_uint4(0, 0, 0, 0);
-      }
-    };
-    fetch(0);
-    pack(0);
-    fetch(1);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(HALF_LOADS) : "memory");
-    products(0, b);
-    pack(1);
-    products(1, b);
-  } else {
+  {
     const T* xr = (const T*)Xv + (size_t)(tok ? j : 0) * ldx + k0;
     uint4 b[STEPS];
 #pragma unroll
@@ -369,26 +324,141 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __rest
   float* ssq = red + NW * 16 * 17;             // [NW][16]
 #pragma unroll
   for (int v = 0; v < 4; ++v) red[(wave * 16 + 4 * G + v) * 17 + j] = acc[v];
-  if (NORM) {
-    float s2 = ss;
-    s2 += __shfl_xor(s2, 16, WAVE);
-    s2 += __shfl_xor(s2, 32, WAVE);
-    if (G == 0) ssq[wave * 16 + j] = s2;
-  }
   __syncthreads();
   if (wave == 0) {
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     for (int w = 0; w < NW; ++w)
 #pragma unroll
       for (int q = 0; q < 4; ++q) v[q] += red[(w * 16 + 4 * G + q) * 17 + j];
-    if (NORM) {
+    if (tok) epilogue4<T, EPI>(Y, ldy, N, j, n0 + 4 * G, v[0], v[1], v[2], v[3]);
+  }
+}
+
+// The same with the RMSNorm of the float32 residual rows riding in the product (see skinny_kernel).  A wave needs the
+// part of every token's row that belongs to its kilobyte of k: it loads that part with all its lanes, 16 bytes each in
+// whole runs (and the norm's weights once, not once per token), multiplies, gathers each token's sum of squares, and
+// leaves the column operands in LDS behind its kilobytes of W, a kilobyte per token, pieces placed as W's are.  X's
+// loads stand in front of W's in program order, so that working on X waits for X only while W streams in.
+template <typename T, int NW, int R, int EPI>
+__global__ __launch_bounds__(NW* WAVE) void skinny_stream_norm_kernel(const T* __restrict__ W, const float* __restrict__ X,
+                                                                       const float* __restrict__ norm_w, float eps,
+                                                                       void* __restrict__ Y, int N, int Tn, int K, int ldw,
+                                                                       int ldx, int ldy) {
+  constexpr int EPC = 16 / sizeof(T);          // elements of a 16-byte operand
+  constexpr int CH = 1024 / sizeof(T);         // elements of a row's kilobyte
+  constexpr int STEPS = 16;                    // MFMA steps of a kilobyte: four 16-byte pieces each
+  constexpr int LPT = CH / 4 / WAVE;           // loads of four floats per lane that bring one token's part of x (2 or 1)
+  typedef __attribute__((address_space(3))) char lds_char;
+  extern __shared__ __attribute__((aligned(16))) char lds_raw[];
+  const int wstride = 16384 + Tn * 1024;       // a wave's LDS: its kilobytes of W, then a kilobyte of operands per token
+  lds_char* wbuf = (lds_char*)lds_raw + (size_t)(threadIdx.x >> 6) * wstride;
+  lds_char* xbuf = wbuf + 16384;
+  const uint32_t wbase = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)wbuf);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int j = lane & 15, G = lane >> 4;
+  const int n0 = blockIdx.x * 16 * R;          // the block's R groups of 16 rows take the wave's operands of X in turn
+  const int k0 = wave * CH;                    // this wave's part of k
+  // x first: load number c of a lane brings four floats of token c / LPT
+  float4 xv[16 * LPT], wv[LPT];
+#pragma unroll
+  for (int u = 0; u < LPT; ++u) wv[u] = *(const float4*)(norm_w + k0 + (u * WAVE + lane) * 4);
+#pragma unroll
+  for (int c = 0; c < 16 * LPT; ++c) {
+    const int t = c / LPT, u = c % LPT;
+    xv[c] = t < Tn ? *(const float4*)(X + (size_t)t * ldx + k0 + (u * WAVE + lane) * 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  const char* base = (const char*)uniform_ptr(W + (size_t)n0 * ldw + k0);
+  const uint32_t last_row = (uint32_t)(N - 1 - n0);
+  auto issue = [&](int r) {                    // group r's kilobytes: load c brings row 16 r + c (rows beyond N repeat the last)
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+      const uint32_t row = (uint32_t)(16 * r + c) < last_row ? (uint32_t)(16 * r + c) : last_row;
+      row_to_lds(base, row * (uint32_t)ldw * (uint32_t)sizeof(T) + (uint32_t)((lane ^ c) << 4), wbase + c * 1024);
+    }
+  };
+  issue(0);
+  // x * w in the run dtype into LDS: four elements of token t at element (u * 64 + lane) * 4 of the wave's kilobyte, that
+  // is piece p = that / EPC, which sits at slot p ^ t
+  float ssum[16];
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    float ss = 0.f;
+#pragma unroll
+    for (int u = 0; u < LPT; ++u) {
+      const float4 x4 = xv[t * LPT + u], w4 = wv[u];
+      ss = fmaf(x4.x, x4.x, ss);
+      ss = fmaf(x4.y, x4.y, ss);
+      ss = fmaf(x4.z, x4.z, ss);
+      ss = fmaf(x4.w, x4.w, ss);
+      const int e0 = (u * WAVE + lane) * 4;
+      const int piece = e0 / EPC, within = e0 % EPC;          // within: 0 or 4 (bfloat16), 0 (float32)
+      lds_char* dst = xbuf + t * 1024 + ((piece ^ t) << 4) + within * (int)sizeof(T);
+      if (t < Tn) {
+        if constexpr (sizeof(T) == 4) {
+          *(__attribute__((address_space(3))) rows_u32x4_t*)dst =
+              rows_u32x4_t{__float_as_uint(x4.x * w4.x), __float_as_uint(x4.y * w4.y), __float_as_uint(x4.z * w4.z), __float_as_uint(x4.w * w4.w)};
+        } else {
+          const float f[4] = {x4.x * w4.x, x4.y * w4.y, x4.z * w4.z, x4.w * w4.w};
+          typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+          *(__attribute__((address_space(3))) u32x2_t*)dst = u32x2_t{Elem<T>::pair(f[0], f[1]), Elem<T>::pair(f[2], f[3])};
+        }
+      }
+    }
+    ssum[t] = ss;
+  }
+  // the lane's column operands, once for all the groups of rows
+  const bool tok = j < Tn;
+  const lds_char* brow = xbuf + (tok ? j : 0) * 1024;
+  uint4 bop[STEPS];
+#pragma unroll
+  for (int s_ = 0; s_ < STEPS; ++s_) {
+    const rows_u32x4_t b4 = *(const __attribute__((address_space(3))) rows_u32x4_t*)(brow + (((s_ * 4 + G) ^ (tok ? j : 0)) << 4));
+    bop[s_] = tok ? make_uint4(b4.x, b4.y, b4.z, b4.w) : make_uint4(0, 0, 0, 0);
+  }
+  f32x4_t acc[R];
+  const lds_char* arow = wbuf + j * 1024;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    acc[r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // group r's kilobytes are in LDS
+    uint4 aop[STEPS];
+#pragma unroll
+    for (int s_ = 0; s_ < STEPS; ++s_) {
+      const rows_u32x4_t a4 = *(const __attribute__((address_space(3))) rows_u32x4_t*)(arow + (((s_ * 4 + G) ^ j) << 4));
+      aop[s_] = make_uint4(a4.x, a4.y, a4.z, a4.w);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // ... and in registers: the next group's may take their place
+    if (r + 1 < R) issue(r + 1);
+#pragma unroll
+    for (int s_ = 0; s_ < STEPS; ++s_) Mma16<T>::run(aop[s_], bop[s_], acc[r]);
+  }
+  // each token's sum of squares over this wave's part of k, then everything through LDS as in the kernel above
+#pragma unroll
+  for (int t = 0; t < 16; ++t) ssum[t] = wave_sum(ssum[t]);
+  __syncthreads();
+  float* red = (float*)lds_raw;                // [NW][16][17]
+  float* ssq = red + NW * 16 * 17;             // [NW][16]
+#pragma unroll
+  for (int t = 0; t < 16; ++t)
+    if (lane == t) ssq[wave * 16 + t] = ssum[t];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    if (r) __syncthreads();                    // wave 0 has read the group before
+#pragma unroll
+    for (int v = 0; v < 4; ++v) red[(wave * 16 + 4 * G + v) * 17 + j] = acc[r][v];
+    __syncthreads();
+    if (wave == 0) {
+      float v[4] = {0.f, 0.f, 0.f, 0.f};
+      for (int w = 0; w < NW; ++w)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] += red[(w * 16 + 4 * G + q) * 17 + j];
       float s2 = 0.f;
       for (int w = 0; w < NW; ++w) s2 += ssq[w * 16 + j];
       const float sc = 1.0f / sqrtf(s2 / (float)K + eps);
 #pragma unroll
       for (int q = 0; q < 4; ++q) v[q] *= sc;
+      if (tok) epilogue4<T, EPI>(Y, ldy, N, j, n0 + r * 16 + 4 * G, v[0], v[1], v[2], v[3]);
     }
-    if (tok) epilogue4<T, EPI>(Y, ldy, N, j, n0 + 4 * G, v[0], v[1], v[2], v[3]);
   }
 }
 
@@ -398,7 +468,7 @@ template <typename T>
 static int stream_waves(int Tn, int K, int ldw) {
   const long long bytes = (long long)K * sizeof(T);
   if (Tn < 1 || Tn > 16 || bytes % 1024 || bytes < 2048 || bytes > 8192) return 0;
-  if ((long long)ldw * sizeof(T) * 16 >= (1ll << 32)) return 0;
+  if ((long long)ldw * sizeof(T) * 64 >= (1ll << 32)) return 0;      // row offsets within a block are 32 bits
   const int nw = (int)(bytes / 1024);
   return nw == 2 || nw == 3 || nw == 4 || nw == 6 || nw == 8 ? nw : 0;
 }
@@ -406,17 +476,37 @@ static int stream_waves(int Tn, int K, int ldw) {
 template <typename T, int EPI, bool NORM>
 static const char* launch_skinny_stream(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K,
                                         int ldw, int ldx, int ldy, int nw, hipStream_t stream) {
-  dim3 g((N + 15) / 16);
+  // with the norm a block takes several groups of 16 rows, which share the work on X (a function of N alone)
+  const int groups = !NORM ? 1 : (N >= 16384 ? 4 : (N >= 8192 ? 2 : 1));
+  dim3 g((N + 16 * groups - 1) / (16 * groups));
+  // a wave's LDS: 16 KB of W and, with the norm, a kilobyte of column operands per token
+  const int lds = nw * (16384 + (NORM ? Tn * 1024 : 0));
 #define STREAM_GO(NW_)                                                                                                          \
   do {                                                                                                                          \
-    auto kernel = skinny_stream_kernel<T, NW_, EPI, NORM>;                                                                      \
     static bool raised = false;          /* more than 64 KB of LDS has to be asked for once per kernel */                       \
-    if (NW_ * 16384 > 65536 && !raised) {                                                                                       \
-      hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, NW_ * 16384);         \
-      if (e != hipSuccess) DLGO_FAIL("gemm_rows: cannot get %d bytes of LDS: %s", NW_ * 16384, hipGetErrorString(e));           \
-      raised = true;                                                                                                            \
+    if constexpr (NORM) {                                                                                                       \
+      auto k1 = skinny_stream_norm_kernel<T, NW_, 1, EPI>;                                                                      \
+      auto k2 = skinny_stream_norm_kernel<T, NW_, 2, EPI>;                                                                      \
+      auto k4 = skinny_stream_norm_kernel<T, NW_, 4, EPI>;                                                                      \
+      if (!raised) {                                                                                                            \
+        for (const void* k : {(const void*)k1, (const void*)k2, (const void*)k4}) {                                             \
+          hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                        \
+          if (e != hipSuccess) DLGO_FAIL("gemm_rows: cannot get %d bytes of LDS: %s", 160 * 1024, hipGetErrorString(e));        \
+        }                                                                                                                       \
+        raised = true;                                                                                                          \
+      }                                                                                                                         \
+      auto kernel = groups == 4 ? k4 : (groups == 2 ? k2 : k1);                                                                 \
+      hipLaunchKernelGGL(kernel, g, dim3(NW_* WAVE), lds, stream, (const T*)W, (const float*)X, norm_w, eps, Y, N, Tn, K, ldw,  \
+                         ldx, ldy);                                                                                             \
+    } else {                                                                                                                    \
+      auto kernel = skinny_stream_kernel<T, NW_, EPI>;                                                                          \
+      if (NW_ * 16384 > 65536 && !raised) {                                                                                     \
+        hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, NW_ * 16384);       \
+        if (e != hipSuccess) DLGO_FAIL("gemm_rows: cannot get %d bytes of LDS: %s", NW_ * 16384, hipGetErrorString(e));         \
+        raised = true;                                                                                                          \
+      }                                                                                                                         \
+      hipLaunchKernelGGL(kernel, g, dim3(NW_* WAVE), lds, stream, (const T*)W, X, Y, N, Tn, K, ldw, ldx, ldy);                  \
     }                                                                                                                           \
-    hipLaunchKernelGGL(kernel, g, dim3(NW_* WAVE), NW_ * 16384, stream, (const T*)W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy); \
   } while (0)
   switch (nw) {
     case 2: STREAM_GO(2); break;
@@ -451,10 +541,9 @@ static const char* launch_skinny(const void* W, const void* X, const float* norm
   int nw = pieces >= 128 && N <= 4096 ? 16 : (pieces >= 32 ? 8 : (pieces >= 16 ? 4 : (pieces >= 8 ? 2 : 1)));
   // rows of whole kilobytes and few tokens: W goes through LDS in whole 1 KB runs, where the matrix is large enough
   // for that to pay (force_nw 32 asks for it wherever it applies, 64 rules it out; other values choose the waves)
-  // (measured on the products of 1B to 8B Llamas: with X in the run dtype it wins for every matrix; with the norm riding
-  // in the product, whose float32 x and weights are four times the loads, it loses)
-  const int sw = stream_waves<T>(Tn, K, ldw);
-  if (sw && (force_nw == 32 || (force_nw == 0 && !NORM))) {
+  int sw = stream_waves<T>(Tn, K, ldw);
+  if (NORM && sw * (16384 + Tn * 1024) > 160 * 1024) sw = 0;      // the tokens' operands have to fit in LDS beside W
+  if (sw && (force_nw == 32 || force_nw == 0)) {
     return launch_skinny_stream<T, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, sw, stream);
   }
   if (force_nw && force_nw < 32) nw = force_nw;
