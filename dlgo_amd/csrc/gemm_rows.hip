@@ -269,10 +269,77 @@ static __device__ __forceinline__ void row_to_lds(const void* base, uint32_t vof
 }
 typedef uint32_t rows_u32x4_t __attribute__((ext_vector_type(4)));
 
-template <typename T, int NW, int EPI>
+// What a product may do for the norm that follows it, or take from the product before it (see dlgo_gemm_rows_leave_parts and dlgo_gemm_rows_scaled):
+//   MODE 1 (with the epilogue that adds into the float32 residual rows): beside the new residual rows it leaves
+//     x * norm_w of them in the run dtype, not yet scaled, and each block its 16 columns' share of every row's sum of squares;
+//   MODE 2: its X are such unscaled rows; the shares are added up in a fixed order and the scale 1/sqrt(sum/width + eps)
+//     multiplies the finished sums (it is a scalar per token), before the epilogue.
+static __device__ __forceinline__ uint4 lds_operand(const __attribute__((address_space(3))) char* p) {
+  const rows_u32x4_t v = *(const __attribute__((address_space(3))) rows_u32x4_t*)p;
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+constexpr int NORM_PARTS_MAX = 256;   // most shares of a row's sum of squares (a normed width of 4096)
+
+struct NormParts {
+  const float* norm_w;     // mode 1: the following norm's weights [N]
+  void* unscaled;          // mode 1: [T, ld_unscaled] in the run dtype
+  int ld_unscaled;
+  float* parts;            // mode 1: written, mode 2: read; [T, n_parts]
+  int n_parts;
+  int width;               // mode 2: the normed width (the number of elements the shares were summed over)
+  float eps;               // mode 2
+};
+
+// The end of a streamed product for one group of 16 rows: the waves' partial sums go through LDS (the rows' place, once
+// every wave is done with them, which the caller's barrier has made sure of); wave 0 adds them in wave order and runs the
+// epilogue.  lane: token j = lane % 16, rows 4 G + v of the group.  part_index: where this group's share goes (mode 1).
+template <typename T, int NW, int EPI, int MODE>
+__device__ __forceinline__ void stream_finish(float* red, const f32x4_t& acc, void* __restrict__ Y, int ldy, int N, int n_first,
+                                              bool tok, float sc, const NormParts& np, int part_index) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int j = lane & 15, G = lane >> 4;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) red[(wave * 16 + 4 * G + v) * 17 + j] = acc[v];
+  __syncthreads();
+  if (wave != 0) return;
+  float v[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int w = 0; w < NW; ++w)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) v[q] += red[(w * 16 + 4 * G + q) * 17 + j];
+  const int n = n_first + 4 * G;
+  if (MODE == 2) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) v[q] *= sc;
+  }
+  if (MODE == 1) {
+    // EPI is the sum into the residual rows: the new values themselves, their product with the norm's weights, and
+    // the share of these four columns in the row's sum of squares
+    float p = 0.f;
+    if (tok) {
+      float* y = (float*)Y + (size_t)j * ldy + n;
+      T* u = (T*)np.unscaled + (size_t)j * np.ld_unscaled + n;
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (n + q < N) {
+          const float x = y[q] + v[q];
+          y[q] = x;
+          p = fmaf(x, x, p);
+          Elem<T>::store(u + q, x * np.norm_w[n + q]);
+        }
+    }
+    p += __shfl_xor(p, 16, WAVE);
+    p += __shfl_xor(p, 32, WAVE);
+    if (tok && G == 0) np.parts[(size_t)j * np.n_parts + part_index] = p;
+  } else if (tok) {
+    epilogue4<T, EPI>(Y, ldy, N, j, n, v[0], v[1], v[2], v[3]);
+  }
+}
+
+template <typename T, int NW, int R, int EPI, int MODE>
 __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __restrict__ W, const void* __restrict__ Xv,
                                                                   void* __restrict__ Y, int N, int Tn, int K, int ldw, int ldx,
-                                                                  int ldy) {
+                                                                  int ldy, NormParts np) {
   constexpr int EPC = 16 / sizeof(T);          // elements of a 16-byte operand
   constexpr int CH = 1024 / sizeof(T);         // elements of a row's kilobyte
   constexpr int STEPS = 16;                    // MFMA steps of a kilobyte: four 16-byte pieces each
@@ -282,56 +349,147 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __rest
   const uint32_t wbase = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)wbuf);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = lane & 15, G = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * R;          // the block's R groups of 16 rows take the wave's operands of X in turn
   const int k0 = wave * CH;                    // this wave's part of k
-  // load c brings row c's kilobyte; the lane fetches the piece that belongs at its slot.  Rows beyond N repeat the last.
-  {
-    const char* base = (const char*)uniform_ptr(W + (size_t)n0 * ldw + k0);
-    const uint32_t last_row = (uint32_t)(N - 1 - n0);
-#pragma unroll
-    for (int c = 0; c < 16; ++c) {
-      const uint32_t row = (uint32_t)c < last_row ? (uint32_t)c : last_row;
-      row_to_lds(base, row * (uint32_t)ldw * (uint32_t)sizeof(T) + (uint32_t)((lane ^ c) << 4), wbase + c * 1024);
-    }
-  }
-  f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  const lds_char* arow = wbuf + j * 1024;
   const bool tok = j < Tn;
-  auto products = [&](int half, const uint4* b) {        // eight steps of the wave's kilobyte against eight operands of X
-#pragma unroll
-    for (int s_ = 0; s_ < STEPS / 2; ++s_) {
-      const int piece = (half * (STEPS / 2) + s_) * 4 + G;
-      const rows_u32x4_t a4 = *(const __attribute__((address_space(3))) rows_u32x4_t*)(arow + ((piece ^ j) << 4));
-      Mma16<T>::run(make_uint4(a4.x, a4.y, a4.z, a4.w), b[s_], acc);
-    }
-  };
+  // the lane's operands of X, once for all the groups: token j, the wave's kilobyte of k
+  uint4 b[STEPS];
   {
     const T* xr = (const T*)Xv + (size_t)(tok ? j : 0) * ldx + k0;
-    uint4 b[STEPS];
 #pragma unroll
-    for (int s_ = 0; s_ < STEPS; ++s_) {
-      const uint4 v = *(const uint4*)(xr + s_ * 4 * EPC + G * EPC);
-      b[s_] = tok ? v : make_uint4(0, 0, 0, 0);
+    for (int s_ = 0; s_ < STEPS; ++s_) b[s_] = *(const uint4*)(xr + s_ * 4 * EPC + G * EPC);
+  }
+  // mode 2: each token's shares of its sum of squares are added up by 16 lanes, each its every 16th in order, then
+  // across the lanes in a fixed pattern.  The loads are asked for here, in front of W's, and used once W's first are in.
+  constexpr int TOK_STEP = NW * WAVE / 16;     // tokens that the block takes at a time
+  constexpr int TOK_TURNS = (16 + TOK_STEP - 1) / TOK_STEP;
+  constexpr int SHARES = MODE == 2 ? NORM_PARTS_MAX / 16 : 1;
+  __shared__ float sumsq[16];
+  float share[TOK_TURNS][SHARES];
+  if (MODE == 2) {
+#pragma unroll
+    for (int turn = 0; turn < TOK_TURNS; ++turn) {
+      const int t = turn * TOK_STEP + (threadIdx.x >> 4);
+      const float* p = np.parts + (size_t)(t < Tn ? t : 0) * np.n_parts;
+#pragma unroll
+      for (int u = 0; u < SHARES; ++u) {
+        const int i = u * 16 + (threadIdx.x & 15);
+        share[turn][u] = t < Tn && i < np.n_parts ? p[i] : 0.f;
+      }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // the wave's kilobytes are in LDS, and its part of X is here
-    products(0, b);
-    products(1, b + STEPS / 2);
   }
-  // lane: token j, rows 4 G + v.  The waves' partial sums go through LDS (the rows' place, once every wave is done with
-  // them); wave 0 adds them in wave order.
+  // load c brings row c's kilobyte of a group; the lane fetches the piece that belongs at its slot.  Rows beyond N repeat the last.
+  const char* base = (const char*)uniform_ptr(W + (size_t)n0 * ldw + k0);
+  const uint32_t last_row = (uint32_t)(N - 1 - n0);
+  auto issue = [&](int r) {
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+      const uint32_t row = (uint32_t)(16 * r + c) < last_row ? (uint32_t)(16 * r + c) : last_row;
+      row_to_lds(base, row * (uint32_t)ldw * (uint32_t)sizeof(T) + (uint32_t)((lane ^ c) << 4), wbase + c * 1024);
+    }
+  };
+  issue(0);
+  f32x4_t acc[R];
+  const lds_char* arow = wbuf + j * 1024;
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    acc[r] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // group r's kilobytes are in LDS (and X is here)
+    if (r == 0 && !tok) {
+#pragma unroll
+      for (int s_ = 0; s_ < STEPS; ++s_) b[s_] = make_uint4(0, 0, 0, 0);
+    }
+    if (R == 1) {                                          // one group: multiply as the operands come from LDS
+#pragma unroll
+      for (int s_ = 0; s_ < STEPS; ++s_)
+        Mma16<T>::run(lds_operand(arow + (((s_ * 4 + G) ^ j) << 4)), b[s_], acc[r]);
+    } else {
+      uint4 aop[STEPS];
+#pragma unroll
+      for (int s_ = 0; s_ < STEPS; ++s_) aop[s_] = lds_operand(arow + (((s_ * 4 + G) ^ j) << 4));
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // ... and in registers: the next group's may take their place
+      if (r + 1 < R) issue(r + 1);
+#pragma unroll
+      for (int s_ = 0; s_ < STEPS; ++s_) Mma16<T>::run(aop[s_], b[s_], acc[r]);
+    }
+  }
+  if (MODE == 2) {
+#pragma unroll
+    for (int turn = 0; turn < TOK_TURNS; ++turn) {
+      float sh = 0.f;
+#pragma unroll
+      for (int u = 0; u < SHARES; ++u) sh += share[turn][u];
+      sh += __shfl_xor(sh, 1, WAVE);
+      sh += __shfl_xor(sh, 2, WAVE);
+      sh += __shfl_xor(sh, 4, WAVE);
+      sh += __shfl_xor(sh, 8, WAVE);
+      const int t = turn * TOK_STEP + (threadIdx.x >> 4);
+      if ((threadIdx.x & 15) == 0 && t < 16) sumsq[t] = sh;
+    }
+  }
   __syncthreads();
+  const float sc = MODE == 2 ? 1.0f / sqrtf(sumsq[j] / (float)np.width + np.eps) : 1.f;
   float* red = (float*)lds_raw;                // [NW][16][17]
-  float* ssq = red + NW * 16 * 17;             // [NW][16]
 #pragma unroll
-  for (int v = 0; v < 4; ++v) red[(wave * 16 + 4 * G + v) * 17 + j] = acc[v];
-  __syncthreads();
-  if (wave == 0) {
-    float v[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int w = 0; w < NW; ++w)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) v[q] += red[(w * 16 + 4 * G + q) * 17 + j];
-    if (tok) epilogue4<T, EPI>(Y, ldy, N, j, n0 + 4 * G, v[0], v[1], v[2], v[3]);
+  for (int r = 0; r < R; ++r) {
+    if (r) __syncthreads();                    // wave 0 has read the group before
+    stream_finish<T, NW, EPI, MODE>(red, acc[r], Y, ldy, N, n0 + r * 16, tok, sc, np, blockIdx.x * R + r);
   }
+}
+
+// The same for rows of more kilobytes than a block has waves: wave w takes kilobytes w, w + NW, ... of the block's 16
+// rows in turn (turns of them each), into the same 16 KB of LDS; the next one streams in while this one is multiplied,
+// and its operands of X, which are asked for in front of it, wait in a second set of registers.
+template <typename T, int NW, int EPI, int MODE>
+__global__ __launch_bounds__(NW* WAVE) void skinny_stream_long_kernel(const T* __restrict__ W, const void* __restrict__ Xv,
+                                                                       void* __restrict__ Y, int N, int Tn, int turns, int ldw,
+                                                                       int ldx, int ldy, NormParts np) {
+  constexpr int EPC = 16 / sizeof(T);
+  constexpr int CH = 1024 / sizeof(T);
+  constexpr int STEPS = 16;
+  typedef __attribute__((address_space(3))) char lds_char;
+  extern __shared__ __attribute__((aligned(16))) char lds_raw[];
+  lds_char* wbuf = (lds_char*)lds_raw + (size_t)(threadIdx.x >> 6) * 16384;
+  const uint32_t wbase = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)wbuf);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int j = lane & 15, G = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const bool tok = j < Tn;
+  const T* xr = (const T*)Xv + (size_t)(tok ? j : 0) * ldx + G * EPC;
+  const char* base = (const char*)uniform_ptr(W + (size_t)n0 * ldw);
+  const uint32_t last_row = (uint32_t)(N - 1 - n0);
+  uint32_t woff[16];                           // where load c of a kilobyte starts within it
+#pragma unroll
+  for (int c = 0; c < 16; ++c)
+    woff[c] = ((uint32_t)c < last_row ? (uint32_t)c : last_row) * (uint32_t)ldw * (uint32_t)sizeof(T) + (uint32_t)((lane ^ c) << 4);
+  auto ask = [&](int turn, uint4* b) {         // a turn's operands of X and its kilobytes of W
+    const int k0 = (turn * NW + wave) * CH;
+#pragma unroll
+    for (int s_ = 0; s_ < STEPS; ++s_) b[s_] = *(const uint4*)(xr + k0 + s_ * 4 * EPC);
+    const uint32_t kb = (uint32_t)k0 * (uint32_t)sizeof(T);
+#pragma unroll
+    for (int c = 0; c < 16; ++c) row_to_lds(base, woff[c] + kb, wbase + c * 1024);
+  };
+  f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const lds_char* arow = wbuf + j * 1024;
+  auto multiply = [&](int turn, const uint4* b, uint4* b_next) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // this turn's kilobytes are in LDS, its X in registers
+    uint4 aop[STEPS];
+#pragma unroll
+    for (int s_ = 0; s_ < STEPS; ++s_) aop[s_] = lds_operand(arow + (((s_ * 4 + G) ^ j) << 4));
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // ... and in registers: the next turn's may take their place
+    if (turn + 1 < turns) ask(turn + 1, b_next);
+#pragma unroll
+    for (int s_ = 0; s_ < STEPS; ++s_) Mma16<T>::run(aop[s_], tok ? b[s_] : make_uint4(0, 0, 0, 0), acc);
+  };
+  uint4 b0[STEPS], b1[STEPS];
+  ask(0, b0);
+  for (int turn = 0; turn < turns; turn += 2) {
+    multiply(turn, b0, b1);
+    if (turn + 1 < turns) multiply(turn + 1, b1, b0);
+  }
+  __syncthreads();
+  stream_finish<T, NW, EPI, MODE>((float*)lds_raw, acc, Y, ldy, N, n0, tok, 1.f, np, blockIdx.x);
 }
 
 // The same with the RMSNorm of the float32 residual rows riding in the product (see skinny_kernel).  A wave needs the
@@ -462,52 +620,87 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_norm_kernel(const T* _
   }
 }
 
-// Whether skinny_stream_kernel takes a product, and with how many waves: up to 16 tokens, rows of 2 to 8 whole kilobytes
-// (a wave keeps 16 KB of LDS; eight of them fill a compute unit's).
+// Whether the streaming kernels take a product, and with how many waves: up to 16 tokens and rows of whole kilobytes.
+// Rows of 2, 3, 4, 6 or 8 KB: a wave per kilobyte (a wave keeps 16 KB of LDS; eight of them fill a compute unit's),
+// *turns = 1.  Other lengths, if some number of waves from 8 down to 4 divides them: each wave takes *turns kilobytes.
 template <typename T>
-static int stream_waves(int Tn, int K, int ldw) {
+static int stream_waves(int Tn, int K, int ldw, int* turns = nullptr) {
   const long long bytes = (long long)K * sizeof(T);
-  if (Tn < 1 || Tn > 16 || bytes % 1024 || bytes < 2048 || bytes > 8192) return 0;
+  if (turns) *turns = 1;
+  if (Tn < 1 || Tn > 16 || bytes % 1024 || bytes < 2048) return 0;
   if ((long long)ldw * sizeof(T) * 64 >= (1ll << 32)) return 0;      // row offsets within a block are 32 bits
-  const int nw = (int)(bytes / 1024);
-  return nw == 2 || nw == 3 || nw == 4 || nw == 6 || nw == 8 ? nw : 0;
+  const int kb = (int)(bytes / 1024);
+  if (kb == 2 || kb == 3 || kb == 4 || kb == 6 || kb == 8) return kb;
+  if (!turns || kb > 8 * 64) return 0;
+  for (int nw = 8; nw >= 4; --nw)
+    if (kb % nw == 0) {
+      *turns = kb / nw;
+      return nw;
+    }
+  return 0;
 }
 
-template <typename T, int EPI, bool NORM>
+template <typename T, int EPI, bool NORM, int MODE = 0>
 static const char* launch_skinny_stream(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K,
-                                        int ldw, int ldx, int ldy, int nw, hipStream_t stream) {
-  // with the norm a block takes several groups of 16 rows, which share the work on X (a function of N alone)
-  const int groups = !NORM ? 1 : (N >= 16384 ? 4 : (N >= 8192 ? 2 : 1));
+                                        int ldw, int ldx, int ldy, int nw, hipStream_t stream, NormParts np = NormParts{},
+                                        int turns = 1) {
+  const bool is_long = turns > 1 || nw == 5 || nw == 7;
+  // with the norm, done here or left by the product before, a block takes several groups of 16 rows, which share the
+  // work on X (a function of N alone)
+  const int groups = (!NORM && MODE != 2) || is_long ? 1 : (N >= 16384 ? 4 : (N >= 8192 ? 2 : 1));
   dim3 g((N + 16 * groups - 1) / (16 * groups));
   // a wave's LDS: 16 KB of W and, with the norm, a kilobyte of column operands per token
   const int lds = nw * (16384 + (NORM ? Tn * 1024 : 0));
+#define STREAM_RAISE(LIMIT_, ...)                                                                                               \
+  do {                                                                                                                          \
+    static bool raised = false;          /* 64 KB of LDS and more have to be asked for once per kernel */                       \
+    if (!raised) {                                                                                                              \
+      for (const void* k : {__VA_ARGS__}) {                                                                                     \
+        hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, LIMIT_);                              \
+        if (e != hipSuccess) DLGO_FAIL("gemm_rows: cannot get %d bytes of LDS: %s", LIMIT_, hipGetErrorString(e));              \
+      }                                                                                                                         \
+      raised = true;                                                                                                            \
+    }                                                                                                                           \
+  } while (0)
+#define STREAM_LONG_GO(NW_)                                                                                                     \
+  do {                                                                                                                          \
+    if constexpr (!NORM && MODE != 2) {                                                                                         \
+      auto kernel = skinny_stream_long_kernel<T, NW_, EPI, MODE>;                                                               \
+      STREAM_RAISE(NW_ * 16384, (const void*)kernel);                                                                           \
+      hipLaunchKernelGGL(kernel, g, dim3(NW_* WAVE), lds, stream, (const T*)W, X, Y, N, Tn, turns, ldw, ldx, ldy, np);          \
+    } else {                                                                                                                    \
+      DLGO_FAIL("gemm_rows: rows of %d KB are not streamed with a norm", nw * turns);                                           \
+    }                                                                                                                           \
+  } while (0)
 #define STREAM_GO(NW_)                                                                                                          \
   do {                                                                                                                          \
-    static bool raised = false;          /* more than 64 KB of LDS has to be asked for once per kernel */                       \
     if constexpr (NORM) {                                                                                                       \
       auto k1 = skinny_stream_norm_kernel<T, NW_, 1, EPI>;                                                                      \
       auto k2 = skinny_stream_norm_kernel<T, NW_, 2, EPI>;                                                                      \
       auto k4 = skinny_stream_norm_kernel<T, NW_, 4, EPI>;                                                                      \
-      if (!raised) {                                                                                                            \
-        for (const void* k : {(const void*)k1, (const void*)k2, (const void*)k4}) {                                             \
-          hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                        \
-          if (e != hipSuccess) DLGO_FAIL("gemm_rows: cannot get %d bytes of LDS: %s", 160 * 1024, hipGetErrorString(e));        \
-        }                                                                                                                       \
-        raised = true;                                                                                                          \
-      }                                                                                                                         \
+      STREAM_RAISE(160 * 1024, (const void*)k1, (const void*)k2, (const void*)k4);                                              \
       auto kernel = groups == 4 ? k4 : (groups == 2 ? k2 : k1);                                                                 \
       hipLaunchKernelGGL(kernel, g, dim3(NW_* WAVE), lds, stream, (const T*)W, (const float*)X, norm_w, eps, Y, N, Tn, K, ldw,  \
                          ldx, ldy);                                                                                             \
     } else {                                                                                                                    \
-      auto kernel = skinny_stream_kernel<T, NW_, EPI>;                                                                          \
-      if (NW_ * 16384 > 65536 && !raised) {                                                                                     \
-        hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, NW_ * 16384);       \
-        if (e != hipSuccess) DLGO_FAIL("gemm_rows: cannot get %d bytes of LDS: %s", NW_ * 16384, hipGetErrorString(e));         \
-        raised = true;                                                                                                          \
-      }                                                                                                                         \
-      hipLaunchKernelGGL(kernel, g, dim3(NW_* WAVE), lds, stream, (const T*)W, X, Y, N, Tn, K, ldw, ldx, ldy);                  \
+      auto k1 = skinny_stream_kernel<T, NW_, 1, EPI, MODE>;                                                                     \
+      auto k2 = skinny_stream_kernel<T, NW_, MODE == 2 ? 2 : 1, EPI, MODE>;                                                     \
+      auto k4 = skinny_stream_kernel<T, NW_, MODE == 2 ? 4 : 1, EPI, MODE>;                                                     \
+      STREAM_RAISE(NW_ * 16384, (const void*)k1, (const void*)k2, (const void*)k4);                                             \
+      auto kernel = groups == 4 ? k4 : (groups == 2 ? k2 : k1);                                                                 \
+      hipLaunchKernelGGL(kernel, g, dim3(NW_* WAVE), lds, stream, (const T*)W, X, Y, N, Tn, K, ldw, ldx, ldy, np);              \
     }                                                                                                                           \
   } while (0)
+  if (is_long) {
+    switch (nw) {
+      case 4: STREAM_LONG_GO(4); break;
+      case 5: STREAM_LONG_GO(5); break;
+      case 6: STREAM_LONG_GO(6); break;
+      case 7: STREAM_LONG_GO(7); break;
+      default: STREAM_LONG_GO(8); break;
+    }
+    return nullptr;
+  }
   switch (nw) {
     case 2: STREAM_GO(2); break;
     case 3: STREAM_GO(3); break;
@@ -516,6 +709,8 @@ static const char* launch_skinny_stream(const void* W, const void* X, const floa
     default: STREAM_GO(8); break;
   }
 #undef STREAM_GO
+#undef STREAM_LONG_GO
+#undef STREAM_RAISE
   return nullptr;
 }
 
@@ -541,10 +736,11 @@ static const char* launch_skinny(const void* W, const void* X, const float* norm
   int nw = pieces >= 128 && N <= 4096 ? 16 : (pieces >= 32 ? 8 : (pieces >= 16 ? 4 : (pieces >= 8 ? 2 : 1)));
   // rows of whole kilobytes and few tokens: W goes through LDS in whole 1 KB runs, where the matrix is large enough
   // for that to pay (force_nw 32 asks for it wherever it applies, 64 rules it out; other values choose the waves)
-  int sw = stream_waves<T>(Tn, K, ldw);
+  int turns = 1;
+  int sw = stream_waves<T>(Tn, K, ldw, NORM ? nullptr : &turns);
   if (NORM && sw * (16384 + Tn * 1024) > 160 * 1024) sw = 0;      // the tokens' operands have to fit in LDS beside W
   if (sw && (force_nw == 32 || force_nw == 0)) {
-    return launch_skinny_stream<T, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, sw, stream);
+    return launch_skinny_stream<T, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, sw, stream, NormParts{}, turns);
   }
   if (force_nw && force_nw < 32) nw = force_nw;
   // many rows: each block takes 2 or 4 groups of 16, which divides the traffic of X (a function of N alone)
@@ -648,6 +844,73 @@ extern "C" const char* dlgo_gemm_rmsnorm(const void* W, const float* X, const fl
 #undef NORM_GO
   if (err) return err;
   DLGO_LAUNCH_CHECK("gemm_rmsnorm");
+  return nullptr;
+}
+
+
+// Whether the two entry points below take a product: up to 16 rows of X, weight rows of 2 to 8 whole kilobytes.
+// scaled: as the consumer (dlgo_gemm_rows_scaled), which takes fewer lengths of rows than the producer.
+extern "C" int dlgo_gemm_rows_streams(int dtype, int Tn, int K, int ldw, int scaled) {
+  int turns = 1;
+  return dtype == DLGO_ELEM && stream_waves<elem_t>(Tn, K, ldw, scaled ? nullptr : &turns) > 0 ? 1 : 0;
+}
+
+// residual [T, N] (float32) += X W^T, and for the norm that follows: unscaled [T, N] (run dtype) = new residual * norm_w,
+// parts [T, n_parts] = every block's share of each row's sum of squares (n_parts = (N + 15) / 16, returned).  The consumer
+// is dlgo_gemm_rows_scaled with these parts.
+extern "C" const char* dlgo_gemm_rows_leave_parts(const void* W, const void* X, float* residual, int dtype, int N, int Tn, int K,
+                                                  int ldw, int ldx, int ldy, const float* norm_w, void* unscaled, int ld_unscaled,
+                                                  float* parts, long long parts_elems, int* n_parts, hipStream_t stream) {
+  DLGO_REQUIRE(dtype == DLGO_ELEM, "gemm_rows: this library is built for dtype code %d, got %d", DLGO_ELEM, dtype);
+  DLGO_REQUIRE(N > 0 && Tn >= 0 && K > 0 && ldw >= K && ldx >= K && ldy >= N && ld_unscaled >= N, "gemm_rows_leave_parts: bad sizes");
+  int turns = 1;
+  const int sw = stream_waves<elem_t>(Tn, K, ldw, &turns);
+  DLGO_REQUIRE(sw > 0, "gemm_rows_leave_parts: up to 16 rows and weight rows of whole KB, got T=%d K=%d", Tn, K);
+  const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
+  DLGO_REQUIRE(ldw % epc == 0 && ldx % epc == 0 && ((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0,
+               "gemm_rows_leave_parts: W and X must be 16-byte aligned with row strides that keep them so");
+  const int np_ = (N + 15) / 16;
+  DLGO_REQUIRE(np_ <= NORM_PARTS_MAX, "gemm_rows_leave_parts: a width of up to %d, got %d", 16 * NORM_PARTS_MAX, N);
+  DLGO_REQUIRE(residual && norm_w && unscaled && parts && parts_elems >= (long long)Tn * np_, "gemm_rows_leave_parts: missing operand or scratch too small");
+  *n_parts = np_;
+  if (Tn == 0) return nullptr;
+  NormParts np{norm_w, unscaled, ld_unscaled, parts, np_, 0, 0.f};
+  const char* err = launch_skinny_stream<elem_t, EPI_ACCUM_F32, false, 1>(W, X, nullptr, 0.f, residual, N, Tn, K, ldw, ldx, ldy, sw, stream, np, turns);
+  if (err) return err;
+  DLGO_LAUNCH_CHECK("gemm_rows_leave_parts");
+  return nullptr;
+}
+
+// Y (epilogue)= scale[t] * (X W^T) where X are rows that dlgo_gemm_rows_leave_parts left unscaled and
+// scale[t] = 1 / sqrt(sum of the row's parts / width + eps).  Epilogues as dlgo_gemm_rows.
+extern "C" const char* dlgo_gemm_rows_scaled(const void* W, const void* X, void* Y, int dtype, int N, int Tn, int K, int ldw, int ldx,
+                                             int ldy, int epilogue, const float* parts, int n_parts, int width, float eps,
+                                             hipStream_t stream) {
+  DLGO_REQUIRE(dtype == DLGO_ELEM, "gemm_rows: this library is built for dtype code %d, got %d", DLGO_ELEM, dtype);
+  DLGO_REQUIRE(N > 0 && Tn >= 0 && K > 0 && ldw >= K && ldx >= K, "gemm_rows_scaled: bad sizes");
+  const int sw = stream_waves<elem_t>(Tn, K, ldw);
+  DLGO_REQUIRE(sw > 0, "gemm_rows_scaled: up to 16 rows and weight rows of 2 to 8 whole KB, got T=%d K=%d", Tn, K);
+  const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
+  DLGO_REQUIRE(ldw % epc == 0 && ldx % epc == 0 && ((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0,
+               "gemm_rows_scaled: W and X must be 16-byte aligned with row strides that keep them so");
+  DLGO_REQUIRE(parts && n_parts > 0 && n_parts <= NORM_PARTS_MAX && width > 0 && eps > 0.f,
+               "gemm_rows_scaled: parts, their number (up to %d, got %d), the width and eps", NORM_PARTS_MAX, n_parts);
+  DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm: SwiGLU epilogue needs an even N and ldy >= N/2");
+  DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm: ldy %d shorter than N %d", ldy, N);
+  if (Tn == 0) return nullptr;
+  NormParts np{nullptr, nullptr, 0, const_cast<float*>(parts), n_parts, width, eps};
+  const char* err = nullptr;
+#define SCALED_GO(E_) err = launch_skinny_stream<elem_t, E_, false, 2>(W, X, nullptr, 0.f, Y, N, Tn, K, ldw, ldx, ldy, sw, stream, np)
+  switch (epilogue) {
+    case EPI_STORE: SCALED_GO(EPI_STORE); break;
+    case EPI_ACCUM_F32: SCALED_GO(EPI_ACCUM_F32); break;
+    case EPI_SWIGLU: SCALED_GO(EPI_SWIGLU); break;
+    case EPI_STORE_F32: SCALED_GO(EPI_STORE_F32); break;
+    default: DLGO_FAIL("gemm_rows_scaled: unknown epilogue %d", epilogue);
+  }
+#undef SCALED_GO
+  if (err) return err;
+  DLGO_LAUNCH_CHECK("gemm_rows_scaled");
   return nullptr;
 }
 

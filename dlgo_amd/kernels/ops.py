@@ -79,7 +79,7 @@ def _lib(module: str, defines=()):
     lib = _libs.get(key)
     if lib is None:
         lib = build.load(module, defines)
-        for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_accum_norm", "dlgo_gemm_parts", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_attention_rows",
+        for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_accum_norm", "dlgo_gemm_parts", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_gemm_rows_leave_parts", "dlgo_gemm_rows_scaled", "dlgo_attention_rows",
                      "dlgo_attention_prefill", "dlgo_attention_prefill_f32", "dlgo_attention_decode", "dlgo_attention_decode_f32", "dlgo_argmax", "dlgo_sample", "dlgo_bias_add", "dlgo_head_rmsnorm"):
             if hasattr(lib, name):
                 getattr(lib, name).restype = ctypes.c_char_p
@@ -292,6 +292,74 @@ def gemm_rmsnorm(weight: torch.Tensor, x: torch.Tensor, norm_weight: torch.Tenso
     _check(_lib("gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),)).dlgo_gemm_rmsnorm(_ptr(weight), _ptr(x), _ptr(norm_weight), ctypes.c_float(eps), _ptr(out),
                                           dtype_code(weight.dtype), n, t, k, _rows(weight, "gemm weight"),
                                           _rows(x, "residual rows"), _rows(out, "gemm output"), epilogue, kind, _stream()))
+    return out
+
+
+class UnscaledNorm:
+    """What gemm_accum_leave_norm leaves of rmsnorm(residual) * norm_weight: the rows it wrote hold residual * norm_weight,
+    and `parts` [T, n_parts] (float32) each row's sum of squares in n_parts shares; rmsnorm's factor of row t is
+    1 / sqrt(sum(parts[t]) / width + eps).  It is a scalar per row, so a product of the rows can apply it to its sums:
+    gemm_scaled does."""
+    __slots__ = ("rows", "parts", "n_parts", "width", "eps")
+
+    def __init__(self, rows, parts, n_parts, width, eps):
+        self.rows, self.parts, self.n_parts, self.width, self.eps = rows, parts, n_parts, width, eps
+
+
+def streams_few_rows(weight: torch.Tensor, rows: int, scaled: bool = False) -> bool:
+    """Whether gemm_accum_leave_norm (scaled: gemm_scaled) takes this weight with this many rows of x: up to 16 rows and
+    weight rows of whole KB (for gemm_scaled: 2, 3, 4, 6 or 8 of them)."""
+    if weight.dim() != 2 or weight.stride(1) != 1 or not (1 <= rows <= 16):
+        return False
+    lib = _lib("gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),))
+    lib.dlgo_gemm_rows_streams.restype = ctypes.c_int
+    return bool(lib.dlgo_gemm_rows_streams(dtype_code(weight.dtype), rows, weight.shape[1], weight.stride(0), int(scaled)))
+
+
+def gemm_accum_leave_norm(weight: torch.Tensor, x: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor, eps: float,
+                          unscaled: torch.Tensor, parts: torch.Tensor) -> UnscaledNorm:
+    """residual += x @ weight.T, and of rmsnorm(residual) * norm_weight of the new rows what UnscaledNorm describes
+    (unscaled: [T, N] in the run dtype; parts: float32 scratch of at least T * ceil(N / 16) elements).  For weights
+    and rows that streams_few_rows accepts."""
+    _need(weight, "gemm weight", dims=2)
+    _need(x, "gemm input", weight.dtype, 2)
+    _need(residual, "residual rows", torch.float32, 2)
+    _need(norm_weight, "norm weight", torch.float32, 1)
+    _need(unscaled, "unscaled rows", weight.dtype, 2)
+    _need(parts, "norm parts", torch.float32, 1)
+    n, k = weight.shape
+    t = x.shape[0]
+    if x.shape[1] != k or tuple(residual.shape) != (t, n) or tuple(unscaled.shape) != (t, n) or norm_weight.shape[0] != n:
+        raise KernelError(f"gemm_accum_leave_norm: x {tuple(x.shape)}, residual {tuple(residual.shape)}, unscaled {tuple(unscaled.shape)} "
+                          f"and norm weight {tuple(norm_weight.shape)} do not fit weight {tuple(weight.shape)}")
+    n_parts = ctypes.c_int(0)
+    lib = _lib("gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),))
+    _check(lib.dlgo_gemm_rows_leave_parts(_ptr(weight), _ptr(x), _ptr(residual), dtype_code(weight.dtype), n, t, k,
+                                          _rows(weight, "gemm weight"), _rows(x, "gemm input"), _rows(residual, "residual rows"),
+                                          _ptr(norm_weight), _ptr(unscaled), _rows(unscaled, "unscaled rows"), _ptr(parts),
+                                          ctypes.c_longlong(parts.numel()), ctypes.byref(n_parts), _stream()))
+    return UnscaledNorm(unscaled, parts, n_parts.value, n, eps)
+
+
+def gemm_scaled(weight: torch.Tensor, left: UnscaledNorm, out: torch.Tensor, epilogue: int = EPI_STORE) -> torch.Tensor:
+    """out (epilogue)= rmsnorm's factor of each row * (left.rows @ weight.T): the product of the normed rows that `left`
+    describes.  Epilogues as gemm(); for weights and rows that streams_few_rows accepts."""
+    _need(weight, "gemm weight", dims=2)
+    x = left.rows
+    _need(x, "unscaled rows", weight.dtype, 2)
+    n, k = weight.shape
+    t = x.shape[0]
+    if x.shape[1] != k or left.width != k or left.parts.numel() < t * left.n_parts:
+        raise KernelError(f"gemm_scaled: rows {tuple(x.shape)} of a norm over {left.width} with {left.n_parts} parts do not fit weight {tuple(weight.shape)}")
+    want_dtype = torch.float32 if epilogue in (EPI_ACCUM_F32, EPI_STORE_F32) else weight.dtype
+    _need(out, "gemm output", want_dtype, 2)
+    cols = n // 2 if epilogue == EPI_SWIGLU else n
+    if tuple(out.shape) != (t, cols):
+        raise KernelError(f"gemm_scaled: output {tuple(out.shape)}, expected {(t, cols)}")
+    lib = _lib("gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),))
+    _check(lib.dlgo_gemm_rows_scaled(_ptr(weight), _ptr(x), _ptr(out), dtype_code(weight.dtype), n, t, k, _rows(weight, "gemm weight"),
+                                     _rows(x, "unscaled rows"), _rows(out, "gemm output"), epilogue, _ptr(left.parts), left.n_parts,
+                                     left.width, ctypes.c_float(left.eps), _stream()))
     return out
 
 

@@ -41,8 +41,10 @@ class Mixer(Part):
     `owns_cache` is False when the unit belongs to another run (then nothing is stored).
     A mixer with state must treat the rows of a sequence in order: ctx.cu_q gives each sequence's rows.
 
-    A mixer that sets `leaves_norm` also takes then=(norm part, rows): "if it costs you nothing, leave that norm of
-    the residual rows as they are after you in `rows`", and returns True if it did (the block then skips the norm).
+    A mixer that sets `leaves_norm` also takes then=(norm part, rows) or (norm part, rows, the part that will read
+    them): "if it costs you nothing, leave that norm of the residual rows as they are after you in `rows`", and returns
+    True if it did (the block then skips the norm), or, if the reading part takes_unscaled(), a kernels.ops.UnscaledNorm
+    that describes what it left instead (the block hands that to the reading part in place of the rows).
     """
     leaves_norm = False
 
@@ -147,8 +149,11 @@ class Attention(Mixer):
     def fuses_norm(self, norm, ctx) -> bool:
         return isinstance(norm, RMSNorm) and ops.fused_norm_pays(self.w_qkv, ctx.n_tokens)
 
-    def forward(self, xn, ctx, unit, residual, owns_cache=True, norm=None, then=None) -> bool:
-        t = xn.shape[0]
+    def takes_unscaled(self, ctx) -> bool:
+        return ops.streams_few_rows(self.w_qkv, ctx.n_tokens, scaled=True)
+
+    def forward(self, xn, ctx, unit, residual, owns_cache=True, norm=None, then=None):
+        t = residual.shape[0]
         n_kv = self.n_kv_heads if owns_cache else 0
         cols = self.q_dim + 2 * n_kv * self.head_dim
         qkv = ctx.buffer("attention.qkv", (t, self.q_dim + 2 * self.kv_dim), ctx.dtype)
@@ -159,7 +164,9 @@ class Attention(Mixer):
         fused = not self._between and ops.attention_fuses_rotation(ctx.dtype, self.head_dim, self.n_heads // self.n_kv_heads,
                                                                    ctx.max_q_len, rot.width if rot else 0, ctx.n_seq)
         unsummed = None
-        if norm is not None:      # xn are the float32 residual rows: the norm rides in the product
+        if isinstance(xn, ops.UnscaledNorm):   # the norm's factor is applied to the product's sums
+            ops.gemm_scaled(self.w_qkv[:cols], xn, qkv[:, :cols])
+        elif norm is not None:    # xn are the float32 residual rows: the norm rides in the product
             ops.gemm_rmsnorm(self.w_qkv[:cols], xn, norm.weight, norm.eps, qkv[:, :cols])
         else:
             # a product that shares k out over blocks leaves its runs to the rotation kernel, which adds them up as it reads
@@ -185,9 +192,12 @@ class Attention(Mixer):
             ops.gemm(self.w_o, out, residual, ops.EPI_ACCUM_F32, scratch=split)
             ops.bias_add(residual, self.b_o)
             return False
-        if then is not None and isinstance(then[0], RMSNorm) and ops.gemm_accum_then_norm(
-                self.w_o, out, residual, split, then[0].weight, then[0].eps, then[1]):
-            return True
+        if then is not None and isinstance(then[0], RMSNorm):
+            if len(then) > 2 and then[2] is not None and then[2].takes_unscaled(ctx) and ops.streams_few_rows(self.w_o, t):
+                shares = ctx.scratch("attention.norm_shares", t * ((self.width + 15) // 16), torch.float32)
+                return ops.gemm_accum_leave_norm(self.w_o, out, residual, then[0].weight, then[0].eps, then[1], shares)
+            if ops.gemm_accum_then_norm(self.w_o, out, residual, split, then[0].weight, then[0].eps, then[1]):
+                return True
         ops.gemm(self.w_o, out, residual, ops.EPI_ACCUM_F32, scratch=split)
         return False
 

@@ -54,6 +54,12 @@ class Part:
     def check(self, dtype: torch.dtype) -> None:
         """Raise ValueError if the kernels of this part cannot take its sizes at `dtype` (called before anything runs)."""
 
+    def takes_unscaled(self, ctx) -> bool:
+        """True if, for this step, the part's forward also takes, in place of normed rows, the description of a norm
+        whose factor is still to be applied (kernels.ops.UnscaledNorm: the rows times the norm's weights, and each
+        row's sum of squares in shares).  The part that runs before may then leave the norm that way."""
+        return False
+
     def kernel_variants(self, dtype: torch.dtype) -> Tuple[Tuple[str, Tuple[Tuple[str, int], ...]], ...]:
         """(module, defines) pairs to compile for this part at `dtype`."""
         from ..kernels.build import variant

@@ -17,8 +17,9 @@ class Block(Part):
     forward(x, ctx, unit, owns_cache) updates the float32 residual rows x in place.
 
     A block that sets `takes_normed` has an `entry_norm` (the norm it applies to x first) and a forward that also takes
-    normed= (rows that already hold entry_norm(x), left by the block before) and then=(the next block's entry norm,
-    rows), and returns True if it left that norm of its result in `rows`."""
+    normed= (rows that already hold entry_norm(x), left by the block before, or what that block returned in their
+    place) and then=(the next block's entry norm, rows, the part that will read them), and returns True if it left that
+    norm of its result in `rows`, or what its last part left instead (see Mixer)."""
     takes_normed = False
 
     def parts(self) -> List[Tuple[str, Part]]:
@@ -51,10 +52,10 @@ class PreNormBlock(Block):
     def entry_norm(self) -> Part:
         return self.mixer_norm
 
-    def forward(self, x, ctx, unit, owns_cache=True, normed=None, then=None) -> bool:
+    def forward(self, x, ctx, unit, owns_cache=True, normed=None, then=None):
         xn = ctx.buffer("block.normed", tuple(x.shape), ctx.dtype)
         # the mixer may leave the feed-forward's norm of its result, the feed-forward the next block's entry norm
-        after = (self.ffn_norm, xn) if self._mixer.leaves_norm else None
+        after = (self.ffn_norm, xn, self.ffn) if self._mixer.leaves_norm else None
         if normed is not None:
             left = self._mixer.forward(normed, ctx, unit, x, owns_cache, **({"then": after} if after else {}))
         elif self._mixer.fuses_norm(self.mixer_norm, ctx):
@@ -64,17 +65,17 @@ class PreNormBlock(Block):
             # the mixer reads xn until its last product, whose sum is what writes the norm: a buffer of its own
             mid = ctx.buffer("block.normed_mid", tuple(x.shape), ctx.dtype) if after else None
             if after:
-                after = (self.ffn_norm, mid)
+                after = (self.ffn_norm, mid, self.ffn)
             left = self._mixer.forward(xn, ctx, unit, x, owns_cache, **({"then": after} if after else {}))
             if left:
                 xn = mid
         onward = {"then": then} if then is not None and self.ffn.leaves_norm else {}
-        if left:
-            return bool(self.ffn.forward(xn, ctx, x, **onward))
+        if left:       # True: the rows hold the norm; anything else stands for them
+            return self.ffn.forward(xn if left is True else left, ctx, x, **onward) or False
         if self.ffn.fuses_norm(self.ffn_norm, ctx):
-            return bool(self.ffn.forward(x, ctx, x, norm=self.ffn_norm, **onward))
+            return self.ffn.forward(x, ctx, x, norm=self.ffn_norm, **onward) or False
         self.ffn_norm(x, xn)
-        return bool(self.ffn.forward(xn, ctx, x, **onward))
+        return self.ffn.forward(xn, ctx, x, **onward) or False
 
 
 BLOCKS = {"pre_norm": PreNormBlock}

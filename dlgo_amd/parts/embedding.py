@@ -55,8 +55,14 @@ class OutputHead(Part):
     def fuses_norm(self, norm, ctx) -> bool:
         return isinstance(norm, RMSNorm) and ops.fused_norm_pays(self.weight, ctx.n_tokens)
 
-    def __call__(self, xn: torch.Tensor, out: torch.Tensor, norm=None) -> torch.Tensor:
-        """xn: normed rows (run dtype), or with `norm` the float32 residual rows; out: float32 [rows, vocab]."""
+    def takes_unscaled(self, ctx) -> bool:
+        return ops.streams_few_rows(self.weight, ctx.n_tokens, scaled=True)
+
+    def __call__(self, xn, out: torch.Tensor, norm=None) -> torch.Tensor:
+        """xn: normed rows (run dtype), or what stands for them (see Part.takes_unscaled), or with `norm` the float32
+        residual rows; out: float32 [rows, vocab]."""
+        if isinstance(xn, ops.UnscaledNorm):
+            return ops.gemm_scaled(self.weight, xn, out, ops.EPI_STORE_F32)
         if norm is not None:
             return ops.gemm_rmsnorm(self.weight, xn, norm.weight, norm.eps, out, ops.EPI_STORE_F32)
         return ops.gemm(self.weight, xn, out, ops.EPI_STORE_F32)

@@ -16,8 +16,8 @@ from .norm import RMSNorm
 
 class FeedForward(Part):
     """Interface: forward(xn, ctx, residual) adds the result for the step's rows into `residual`.  One that sets
-    `leaves_norm` also takes then=(norm part, rows) and returns True if it left that norm of the new residual rows
-    in `rows` (see Mixer)."""
+    `leaves_norm` also takes then=(norm part, rows[, the part that will read them]) and returns True if it left that
+    norm of the new residual rows in `rows`, or what it left instead (see Mixer)."""
     leaves_norm = False
 
     def fuses_norm(self, norm, ctx) -> bool:
@@ -59,9 +59,14 @@ class GatedFeedForward(FeedForward):
     def fuses_norm(self, norm, ctx) -> bool:
         return isinstance(norm, RMSNorm) and ops.fused_norm_pays(self.w_gate_up, ctx.n_tokens)
 
-    def forward(self, xn, ctx, residual, norm=None, then=None) -> bool:
-        hid = ctx.buffer("feed_forward.hidden", (xn.shape[0], self.inner), ctx.dtype)
-        if norm is not None:      # xn are the float32 residual rows: the norm rides in the product
+    def takes_unscaled(self, ctx) -> bool:
+        return ops.streams_few_rows(self.w_gate_up, ctx.n_tokens, scaled=True)
+
+    def forward(self, xn, ctx, residual, norm=None, then=None):
+        hid = ctx.buffer("feed_forward.hidden", (residual.shape[0], self.inner), ctx.dtype)
+        if isinstance(xn, ops.UnscaledNorm):   # the norm's factor is applied to the product's sums
+            ops.gemm_scaled(self.w_gate_up, xn, hid, ops.EPI_SWIGLU)
+        elif norm is not None:    # xn are the float32 residual rows: the norm rides in the product
             ops.gemm_rmsnorm(self.w_gate_up, xn, norm.weight, norm.eps, hid, ops.EPI_SWIGLU)
         else:
             ops.gemm(self.w_gate_up, xn, hid, ops.EPI_SWIGLU)

@@ -114,11 +114,11 @@ class DecoderModel:
             nxt = None if last else self.layers[self.order[i + 1].layer][1]
             then = None
             if nxt is not None and nxt.takes_normed:
-                then = (nxt.entry_norm, ctx.buffer(f"model.normed.{i & 1}", tuple(x.shape), ctx.dtype))
+                then = (nxt.entry_norm, ctx.buffer(f"model.normed.{i & 1}", tuple(x.shape), ctx.dtype), nxt.mixer)
             elif last and all_rows_wanted:
-                then = (self.final_norm, ctx.buffer(f"model.normed.{i & 1}", tuple(x.shape), ctx.dtype))
+                then = (self.final_norm, ctx.buffer(f"model.normed.{i & 1}", tuple(x.shape), ctx.dtype), self.head)
             left = block.forward(x, ctx, self.run_unit[i], self.run_owns[i], normed=normed, then=then)
-            normed = then[1] if left else None
+            normed = (then[1] if left is True else left) if left else None     # True: the rows hold the norm
             if last and left:
                 ctx.final_normed = normed
         return x

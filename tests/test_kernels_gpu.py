@@ -120,7 +120,9 @@ def test_head_rmsnorm(dtype, _, rel, heads, kv, hd):
 GEMM_SHAPES = [(200, 37, 96), (130, 5, 40), (64, 1, 64), (388, 130, 352), (34, 8, 160), (512, 257, 128), (6, 3, 8),
                (32790, 20, 2048),      # wide enough for the kernel that gives a block four groups of rows
                # few tokens and weight rows of whole kilobytes (2, 3, 6 and 16 KB in bfloat16): these go through LDS
-               (100, 11, 1024), (8200, 16, 1536), (40, 3, 3072), (72, 1, 8192), (50, 8, 512)]
+               (100, 11, 1024), (8200, 16, 1536), (40, 3, 3072), (72, 1, 8192), (50, 8, 512),
+               # rows of 5, 7 and 28 KB: a wave takes several kilobytes in turn
+               (40, 9, 2560), (24, 16, 3584), (100, 4, 14336)]
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
@@ -259,7 +261,7 @@ def test_gemm_into_the_residual_that_leaves_the_next_norm(dtype, _, rel, n, t, k
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
 @pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5])
-@pytest.mark.parametrize("f,t,k", [(160, 5, 64), (352, 70, 128), (9, 2, 16), (1030, 200, 72), (40, 33, 2056), (8200, 64, 256), (16401, 9, 2048)])
+@pytest.mark.parametrize("f,t,k", [(160, 5, 64), (352, 70, 128), (9, 2, 16), (1030, 200, 72), (40, 33, 2056), (8200, 64, 256), (16401, 9, 2048), (20, 6, 5120)])
 def test_gemm_swiglu(dtype, _, rel, kind, f, t, k):
     ops = _ops()
     if (kind == 1 and t > 8) or (kind == 5 and t > 64):
@@ -307,6 +309,54 @@ def test_gemm_with_fused_rmsnorm(dtype, _, rel, n, t, k, kind):
     ops.gemm_rmsnorm(w, x, nw, eps, hid, ops.EPI_SWIGLU, kind=kind)
     gd, ud = want[:, 0::2], want[:, 1::2]
     close(hid, gd / (1 + torch.exp(-gd)) * ud, tol * 2, "swiglu")
+
+
+@pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("n1,k1,n2,t", [(1024, 1024, 200, 8), (1536, 2048, 132, 1), (2048, 1536, 96, 16), (3072, 1024, 64, 5), (4096, 4096, 40, 3),
+                                        (1024, 8192, 64, 8), (1024, 5120, 32, 3), (2048, 14336, 48, 16), (1024, 2560, 32, 2), (1024, 3584, 32, 9)])
+def test_norm_left_in_parts_and_applied_by_the_next_product(dtype, _, rel, n1, k1, n2, t):
+    """A product that adds into the residual rows leaves the rows times the norm's weights and the sums of squares in
+    shares; the next product multiplies its sums by the factor.  Together: residual += x W1^T; out = rmsnorm(residual) W2^T.
+    The widths are chosen so that both weights have rows of whole KB in both dtypes (n1 is the second one's inner size);
+    the first one's rows go up to 28 KB, which a wave takes in several turns."""
+    ops = _ops()
+    es = torch.tensor([], dtype=dtype).element_size()
+    n1, k1 = n1 * 2 // es, k1 * 2 // es          # the sizes are given for 2-byte elements
+    g = torch.Generator().manual_seed(n1 + t)
+    w1 = (0.3 * torch.randn(n1, k1, generator=g)).to(dtype).to(DEV)
+    w2 = (0.5 * torch.randn(n2, n1, generator=g)).to(dtype).to(DEV)
+    x = torch.randn(t, k1, generator=g).to(dtype).to(DEV)
+    res = (3 * torch.randn(t, n1, generator=g)).to(DEV)
+    nw = (1 + 0.3 * torch.randn(n1, generator=g)).to(DEV)
+    eps = 1e-2
+    assert ops.streams_few_rows(w1, t) and ops.streams_few_rows(w2, t, scaled=True)
+    assert not ops.streams_few_rows(w2[:, :n1 - 8], t) and not ops.streams_few_rows(w1, 17)
+    new_res = res.double() + x.double() @ w1.double().T
+    xn = new_res / torch.sqrt((new_res * new_res).mean(-1, keepdim=True) + eps) * nw.double()
+    want = xn @ w2.double().T
+    tol = 1e-5 if dtype == torch.float32 else 1.5e-2
+    unscaled = torch.empty(t, n1, dtype=dtype, device=DEV)
+    parts = torch.full((16 * ((n1 + 15) // 16) + 7,), float("nan"), device=DEV)
+    left = ops.gemm_accum_leave_norm(w1, x, res, nw, eps, unscaled, parts)
+    close(res, new_res, 1e-5, "residual")
+    assert left.n_parts == (n1 + 15) // 16 and left.width == n1
+    close(left.parts[:t * left.n_parts].view(t, -1).sum(-1), (new_res * new_res).sum(-1), 1e-5, "sum of squares")
+    close(unscaled, new_res * nw.double(), 1e-6 if dtype == torch.float32 else 8e-3, "unscaled rows")
+    for epi, shape, odt in ((ops.EPI_STORE, (t, n2), dtype), (ops.EPI_STORE_F32, (t, n2), torch.float32)):
+        out = torch.empty(shape, dtype=odt, device=DEV)
+        ops.gemm_scaled(w2, left, out, epi)
+        close(out, want, tol, f"epilogue {epi}")
+    acc = torch.randn(t, n2, generator=g).to(DEV)
+    acc0 = acc.clone()
+    ops.gemm_scaled(w2, left, acc, ops.EPI_ACCUM_F32)
+    close(acc, acc0.double() + want, tol, "accumulate")
+    hid = torch.empty(t, n2 // 2, dtype=dtype, device=DEV)
+    ops.gemm_scaled(w2, left, hid, ops.EPI_SWIGLU)
+    gd, ud = want[:, 0::2], want[:, 1::2]
+    close(hid, gd / (1 + torch.exp(-gd)) * ud, tol * 2, "swiglu")
+    with pytest.raises(ops.KernelError, match="whole KB"):
+        ops.gemm_scaled(w2[:, :n1 - 8].contiguous(), ops.UnscaledNorm(unscaled[:, :n1 - 8].contiguous(), parts, left.n_parts, n1 - 8, eps),
+                        torch.empty(t, n2, dtype=dtype, device=DEV))
 
 
 def test_gemm_reference_vectors():
