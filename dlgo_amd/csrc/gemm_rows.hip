@@ -291,12 +291,52 @@ struct NormParts {
   float eps;               // mode 2
 };
 
+// Mode 2's sums of squares: each token's shares are added up by 16 lanes, each its every 16th in order, then across
+// the lanes in a fixed pattern.  ask() issues the loads (in front of W's, so that they are in when W's first are);
+// leave() adds them up and leaves each token's sum in sumsq[16] (shared memory); a barrier has to follow.
+template <int NW, int MODE>
+struct NormShares {
+  static constexpr int TOK_STEP = NW * WAVE / 16;     // tokens that the block takes at a time
+  static constexpr int TOK_TURNS = (16 + TOK_STEP - 1) / TOK_STEP;
+  static constexpr int SHARES = MODE == 2 ? NORM_PARTS_MAX / 16 : 1;
+  float share[TOK_TURNS][SHARES];
+  __device__ __forceinline__ void ask(const NormParts& np, int Tn) {
+    if (MODE != 2) return;
+#pragma unroll
+    for (int turn = 0; turn < TOK_TURNS; ++turn) {
+      const int t = turn * TOK_STEP + (threadIdx.x >> 4);
+      const float* p = np.parts + (size_t)(t < Tn ? t : 0) * np.n_parts;
+#pragma unroll
+      for (int u = 0; u < SHARES; ++u) {
+        const int i = u * 16 + (threadIdx.x & 15);
+        share[turn][u] = t < Tn && i < np.n_parts ? p[i] : 0.f;
+      }
+    }
+  }
+  __device__ __forceinline__ void leave(float* sumsq) const {
+    if (MODE != 2) return;
+#pragma unroll
+    for (int turn = 0; turn < TOK_TURNS; ++turn) {
+      float sh = 0.f;
+#pragma unroll
+      for (int u = 0; u < SHARES; ++u) sh += share[turn][u];
+      sh += __shfl_xor(sh, 1, WAVE);
+      sh += __shfl_xor(sh, 2, WAVE);
+      sh += __shfl_xor(sh, 4, WAVE);
+      sh += __shfl_xor(sh, 8, WAVE);
+      const int t = turn * TOK_STEP + (threadIdx.x >> 4);
+      if ((threadIdx.x & 15) == 0 && t < 16) sumsq[t] = sh;
+    }
+  }
+};
+
 // The end of a streamed product for one group of 16 rows: the waves' partial sums go through LDS (the rows' place, once
 // every wave is done with them, which the caller's barrier has made sure of); wave 0 adds them in wave order and runs the
-// epilogue.  lane: token j = lane % 16, rows 4 G + v of the group.  part_index: where this group's share goes (mode 1).
+// epilogue.  lane: token t_row (the block's token lane % 16), rows 4 G + v of the group.  part_index: where this
+// group's share goes (mode 1).
 template <typename T, int NW, int EPI, int MODE>
 __device__ __forceinline__ void stream_finish(float* red, const f32x4_t& acc, void* __restrict__ Y, int ldy, int N, int n_first,
-                                              bool tok, float sc, const NormParts& np, int part_index) {
+                                              bool tok, float sc, const NormParts& np, int part_index, int t_row) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = lane & 15, G = lane >> 4;
 #pragma unroll
@@ -317,8 +357,8 @@ __device__ __forceinline__ void stream_finish(float* red, const f32x4_t& acc, vo
     // the share of these four columns in the row's sum of squares
     float p = 0.f;
     if (tok) {
-      float* y = (float*)Y + (size_t)j * ldy + n;
-      T* u = (T*)np.unscaled + (size_t)j * np.ld_unscaled + n;
+      float* y = (float*)Y + (size_t)t_row * ldy + n;
+      T* u = (T*)np.unscaled + (size_t)t_row * np.ld_unscaled + n;
 #pragma unroll
       for (int q = 0; q < 4; ++q)
         if (n + q < N) {
@@ -330,9 +370,9 @@ __device__ __forceinline__ void stream_finish(float* red, const f32x4_t& acc, vo
     }
     p += __shfl_xor(p, 16, WAVE);
     p += __shfl_xor(p, 32, WAVE);
-    if (tok && G == 0) np.parts[(size_t)j * np.n_parts + part_index] = p;
+    if (tok && G == 0) np.parts[(size_t)t_row * np.n_parts + part_index] = p;
   } else if (tok) {
-    epilogue4<T, EPI>(Y, ldy, N, j, n, v[0], v[1], v[2], v[3]);
+    epilogue4<T, EPI>(Y, ldy, N, t_row, n, v[0], v[1], v[2], v[3]);
   }
 }
 
@@ -350,36 +390,19 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __rest
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = lane & 15, G = lane >> 4;
   const int n0 = blockIdx.x * 16 * R;          // the block's R groups of 16 rows take the wave's operands of X in turn
-  const int k0 = wave * CH;                    // this wave's part of k
   const bool tok = j < Tn;
   // the lane's operands of X, once for all the groups: token j, the wave's kilobyte of k
   uint4 b[STEPS];
   {
-    const T* xr = (const T*)Xv + (size_t)(tok ? j : 0) * ldx + k0;
+    const T* xr = (const T*)Xv + (size_t)(tok ? j : 0) * ldx + wave * CH + G * EPC;
 #pragma unroll
-    for (int s_ = 0; s_ < STEPS; ++s_) b[s_] = *(const uint4*)(xr + s_ * 4 * EPC + G * EPC);
+    for (int s_ = 0; s_ < STEPS; ++s_) b[s_] = *(const uint4*)(xr + s_ * 4 * EPC);
   }
-  // mode 2: each token's shares of its sum of squares are added up by 16 lanes, each its every 16th in order, then
-  // across the lanes in a fixed pattern.  The loads are asked for here, in front of W's, and used once W's first are in.
-  constexpr int TOK_STEP = NW * WAVE / 16;     // tokens that the block takes at a time
-  constexpr int TOK_TURNS = (16 + TOK_STEP - 1) / TOK_STEP;
-  constexpr int SHARES = MODE == 2 ? NORM_PARTS_MAX / 16 : 1;
   __shared__ float sumsq[16];
-  float share[TOK_TURNS][SHARES];
-  if (MODE == 2) {
-#pragma unroll
-    for (int turn = 0; turn < TOK_TURNS; ++turn) {
-      const int t = turn * TOK_STEP + (threadIdx.x >> 4);
-      const float* p = np.parts + (size_t)(t < Tn ? t : 0) * np.n_parts;
-#pragma unroll
-      for (int u = 0; u < SHARES; ++u) {
-        const int i = u * 16 + (threadIdx.x & 15);
-        share[turn][u] = t < Tn && i < np.n_parts ? p[i] : 0.f;
-      }
-    }
-  }
+  NormShares<NW, MODE> shares;                 // mode 2: asked for here, in front of W's loads
+  shares.ask(np, Tn);
   // load c brings row c's kilobyte of a group; the lane fetches the piece that belongs at its slot.  Rows beyond N repeat the last.
-  const char* base = (const char*)uniform_ptr(W + (size_t)n0 * ldw + k0);
+  const char* base = (const char*)uniform_ptr(W + (size_t)n0 * ldw + wave * CH);
   const uint32_t last_row = (uint32_t)(N - 1 - n0);
   auto issue = [&](int r) {
 #pragma unroll
@@ -413,27 +436,14 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __rest
       for (int s_ = 0; s_ < STEPS; ++s_) Mma16<T>::run(aop[s_], b[s_], acc[r]);
     }
   }
-  if (MODE == 2) {
-#pragma unroll
-    for (int turn = 0; turn < TOK_TURNS; ++turn) {
-      float sh = 0.f;
-#pragma unroll
-      for (int u = 0; u < SHARES; ++u) sh += share[turn][u];
-      sh += __shfl_xor(sh, 1, WAVE);
-      sh += __shfl_xor(sh, 2, WAVE);
-      sh += __shfl_xor(sh, 4, WAVE);
-      sh += __shfl_xor(sh, 8, WAVE);
-      const int t = turn * TOK_STEP + (threadIdx.x >> 4);
-      if ((threadIdx.x & 15) == 0 && t < 16) sumsq[t] = sh;
-    }
-  }
+  shares.leave(sumsq);
   __syncthreads();
   const float sc = MODE == 2 ? 1.0f / sqrtf(sumsq[j] / (float)np.width + np.eps) : 1.f;
   float* red = (float*)lds_raw;                // [NW][16][17]
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     if (r) __syncthreads();                    // wave 0 has read the group before
-    stream_finish<T, NW, EPI, MODE>(red, acc[r], Y, ldy, N, n0 + r * 16, tok, sc, np, blockIdx.x * R + r);
+    stream_finish<T, NW, EPI, MODE>(red, acc[r], Y, ldy, N, n0 + r * 16, tok, sc, np, blockIdx.x * R + r, j);
   }
 }
 
@@ -482,14 +492,19 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_long_kernel(const T* _
 #pragma unroll
     for (int s_ = 0; s_ < STEPS; ++s_) Mma16<T>::run(aop[s_], tok ? b[s_] : make_uint4(0, 0, 0, 0), acc);
   };
+  __shared__ float sumsq[16];
+  NormShares<NW, MODE> shares;
+  shares.ask(np, Tn);
   uint4 b0[STEPS], b1[STEPS];
   ask(0, b0);
   for (int turn = 0; turn < turns; turn += 2) {
     multiply(turn, b0, b1);
     if (turn + 1 < turns) multiply(turn + 1, b1, b0);
   }
+  shares.leave(sumsq);
   __syncthreads();
-  stream_finish<T, NW, EPI, MODE>((float*)lds_raw, acc, Y, ldy, N, n0, tok, 1.f, np, blockIdx.x);
+  const float sc = MODE == 2 ? 1.0f / sqrtf(sumsq[j] / (float)np.width + np.eps) : 1.f;
+  stream_finish<T, NW, EPI, MODE>((float*)lds_raw, acc, Y, ldy, N, n0, tok, sc, np, blockIdx.x, j);
 }
 
 // The same with the RMSNorm of the float32 residual rows riding in the product (see skinny_kernel).  A wave needs the
@@ -623,6 +638,7 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_norm_kernel(const T* _
 // Whether the streaming kernels take a product, and with how many waves: up to 16 tokens and rows of whole kilobytes.
 // Rows of 2, 3, 4, 6 or 8 KB: a wave per kilobyte (a wave keeps 16 KB of LDS; eight of them fill a compute unit's),
 // *turns = 1.  Other lengths, if some number of waves from 8 down to 4 divides them: each wave takes *turns kilobytes.
+// Without `turns` (the kernel that stages the norm's rows in LDS) only the first kind.
 template <typename T>
 static int stream_waves(int Tn, int K, int ldw, int* turns = nullptr) {
   const long long bytes = (long long)K * sizeof(T);
@@ -645,9 +661,12 @@ static const char* launch_skinny_stream(const void* W, const void* X, const floa
                                         int ldw, int ldx, int ldy, int nw, hipStream_t stream, NormParts np = NormParts{},
                                         int turns = 1) {
   const bool is_long = turns > 1 || nw == 5 || nw == 7;
-  // with the norm, done here or left by the product before, a block takes several groups of 16 rows, which share the
-  // work on X (a function of N alone)
-  const int groups = (!NORM && MODE != 2) || is_long ? 1 : (N >= 16384 ? 4 : (N >= 8192 ? 2 : 1));
+  // A block takes up to four groups of 16 rows in turn, which share its operands of X (and the work on the norm): as
+  // many as leave at least 160 blocks, five eighths of the compute units (a function of N alone).  Measured on the
+  // shapes of 1B to 8B Llamas, 1 to 16 tokens: fewer blocks than that cost more than the shared work saves; with more,
+  // four groups are 5 to 25% faster than one on the wide matrices (gate/up, vocabulary) and two on QKV of 5,120 and 6,144 rows.
+  const int blocks1 = (N + 15) / 16;
+  const int groups = is_long ? 1 : (blocks1 >= 4 * 160 ? 4 : (blocks1 >= 2 * 160 ? 2 : 1));
   dim3 g((N + 16 * groups - 1) / (16 * groups));
   // a wave's LDS: 16 KB of W and, with the norm, a kilobyte of column operands per token
   const int lds = nw * (16384 + (NORM ? Tn * 1024 : 0));
@@ -664,7 +683,7 @@ static const char* launch_skinny_stream(const void* W, const void* X, const floa
   } while (0)
 #define STREAM_LONG_GO(NW_)                                                                                                     \
   do {                                                                                                                          \
-    if constexpr (!NORM && MODE != 2) {                                                                                         \
+    if constexpr (!NORM) {                                                                                                      \
       auto kernel = skinny_stream_long_kernel<T, NW_, EPI, MODE>;                                                               \
       STREAM_RAISE(NW_ * 16384, (const void*)kernel);                                                                           \
       hipLaunchKernelGGL(kernel, g, dim3(NW_* WAVE), lds, stream, (const T*)W, X, Y, N, Tn, turns, ldw, ldx, ldy, np);          \
@@ -683,9 +702,9 @@ static const char* launch_skinny_stream(const void* W, const void* X, const floa
       hipLaunchKernelGGL(kernel, g, dim3(NW_* WAVE), lds, stream, (const T*)W, (const float*)X, norm_w, eps, Y, N, Tn, K, ldw,  \
                          ldx, ldy);                                                                                             \
     } else {                                                                                                                    \
-      auto k1 = skinny_stream_kernel<T, NW_, 1, EPI, MODE>;                                                                     \
-      auto k2 = skinny_stream_kernel<T, NW_, MODE == 2 ? 2 : 1, EPI, MODE>;                                                     \
-      auto k4 = skinny_stream_kernel<T, NW_, MODE == 2 ? 4 : 1, EPI, MODE>;                                                     \
+      auto k1 = skinny_stream_kernel<T, NW_, 1, EPI, MODE>;                                                                  \
+      auto k2 = skinny_stream_kernel<T, NW_, 2, EPI, MODE>;                                                  \
+      auto k4 = skinny_stream_kernel<T, NW_, 4, EPI, MODE>;                                                  \
       STREAM_RAISE(NW_ * 16384, (const void*)k1, (const void*)k2, (const void*)k4);                                             \
       auto kernel = groups == 4 ? k4 : (groups == 2 ? k2 : k1);                                                                 \
       hipLaunchKernelGGL(kernel, g, dim3(NW_* WAVE), lds, stream, (const T*)W, X, Y, N, Tn, K, ldw, ldx, ldy, np);              \
@@ -693,6 +712,8 @@ static const char* launch_skinny_stream(const void* W, const void* X, const floa
   } while (0)
   if (is_long) {
     switch (nw) {
+      case 2: STREAM_LONG_GO(2); break;
+      case 3: STREAM_LONG_GO(3); break;
       case 4: STREAM_LONG_GO(4); break;
       case 5: STREAM_LONG_GO(5); break;
       case 6: STREAM_LONG_GO(6); break;
@@ -852,7 +873,7 @@ extern "C" const char* dlgo_gemm_rmsnorm(const void* W, const float* X, const fl
 // scaled: as the consumer (dlgo_gemm_rows_scaled), which takes fewer lengths of rows than the producer.
 extern "C" int dlgo_gemm_rows_streams(int dtype, int Tn, int K, int ldw, int scaled) {
   int turns = 1;
-  return dtype == DLGO_ELEM && stream_waves<elem_t>(Tn, K, ldw, scaled ? nullptr : &turns) > 0 ? 1 : 0;
+  return dtype == DLGO_ELEM && stream_waves<elem_t>(Tn, K, ldw, &turns) > 0 ? 1 : 0;
 }
 
 // residual [T, N] (float32) += X W^T, and for the norm that follows: unscaled [T, N] (run dtype) = new residual * norm_w,
@@ -888,8 +909,9 @@ extern "C" const char* dlgo_gemm_rows_scaled(const void* W, const void* X, void*
                                              hipStream_t stream) {
   DLGO_REQUIRE(dtype == DLGO_ELEM, "gemm_rows: this library is built for dtype code %d, got %d", DLGO_ELEM, dtype);
   DLGO_REQUIRE(N > 0 && Tn >= 0 && K > 0 && ldw >= K && ldx >= K, "gemm_rows_scaled: bad sizes");
-  const int sw = stream_waves<elem_t>(Tn, K, ldw);
-  DLGO_REQUIRE(sw > 0, "gemm_rows_scaled: up to 16 rows and weight rows of 2 to 8 whole KB, got T=%d K=%d", Tn, K);
+  int turns = 1;
+  const int sw = stream_waves<elem_t>(Tn, K, ldw, &turns);
+  DLGO_REQUIRE(sw > 0, "gemm_rows_scaled: up to 16 rows and weight rows of whole KB, got T=%d K=%d", Tn, K);
   const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
   DLGO_REQUIRE(ldw % epc == 0 && ldx % epc == 0 && ((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0,
                "gemm_rows_scaled: W and X must be 16-byte aligned with row strides that keep them so");
@@ -900,7 +922,7 @@ extern "C" const char* dlgo_gemm_rows_scaled(const void* W, const void* X, void*
   if (Tn == 0) return nullptr;
   NormParts np{nullptr, nullptr, 0, const_cast<float*>(parts), n_parts, width, eps};
   const char* err = nullptr;
-#define SCALED_GO(E_) err = launch_skinny_stream<elem_t, E_, false, 2>(W, X, nullptr, 0.f, Y, N, Tn, K, ldw, ldx, ldy, sw, stream, np)
+#define SCALED_GO(E_) err = launch_skinny_stream<elem_t, E_, false, 2>(W, X, nullptr, 0.f, Y, N, Tn, K, ldw, ldx, ldy, sw, stream, np, turns)
   switch (epilogue) {
     case EPI_STORE: SCALED_GO(EPI_STORE); break;
     case EPI_ACCUM_F32: SCALED_GO(EPI_ACCUM_F32); break;
