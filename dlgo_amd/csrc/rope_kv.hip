@@ -137,8 +137,26 @@ __global__ __launch_bounds__(256) void rope_kv_pieces_kernel(T* __restrict__ qkv
                                                              T* __restrict__ cache, long long page_stride, long long v_off,
                                                              int write_kv, int piece_blocks,
                                                              const float* __restrict__ part, int n_parts, long long plane,
-                                                             int part_ld) {
+                                                             int part_ld, int single_tokens) {
   constexpr int E = Piece<T>::E;
+  if ((int)blockIdx.x >= piece_blocks && single_tokens) {
+    // The values of a step of single tokens: every row belongs to another sequence, so nothing of the transposed page
+    // rows is consecutive and a tile would gain nothing: a thread stores the piece it read, element by element.
+    const int per_head = hd / E;
+    const long long idx = (long long)(blockIdx.x - piece_blocks) * 256 + threadIdx.x;
+    if (idx >= (long long)n_tokens * n_kv * per_head) return;
+    const int t = (int)(idx / (n_kv * per_head)), c = (int)(idx % (n_kv * per_head));
+    const int kvh = c / per_head, d0 = (c % per_head) * E;
+    const int pos = positions[t];
+    const int page = page_table[(size_t)slots[tok_seq[t]] * max_pages + pos / PAGE];
+    if (page < 0) return;
+    float x[E];
+    load_piece<T>(qkv, ld, part, n_parts, plane, part_ld, t, (n_heads + n_kv + kvh) * hd + d0, x);
+    T* vcol = cache + v_off + (size_t)page * page_stride + ((size_t)kvh * hd + d0) * PAGE + pos % PAGE;
+#pragma unroll
+    for (int e = 0; e < E; ++e) Elem<T>::store(vcol + (size_t)e * PAGE, x[e]);
+    return;
+  }
   if ((int)blockIdx.x >= piece_blocks) {
     // The values.  A page keeps them transposed ([head size][token]), so a thread that stored its own piece would write
     // single elements a page row apart.  Instead a block takes 64 consecutive rows of the step, one kv head and up to 64
@@ -227,7 +245,7 @@ extern "C" const char* dlgo_rope_kv(void* qkv, int dtype, int n_tokens, int ld, 
                                     const int32_t* positions, const int32_t* tok_seq, const int32_t* slots,
                                     const int32_t* page_table, int max_pages, void* cache, long long page_stride,
                                     long long v_off, int write_kv, const float* part, int n_parts, long long plane, int part_ld,
-                                    hipStream_t stream) {
+                                    int single_tokens, hipStream_t stream) {
   DLGO_REQUIRE(n_tokens >= 0 && n_heads > 0 && n_kv >= 0 && hd > 0, "rope_kv: bad sizes");
   DLGO_REQUIRE(rot >= 0 && rot <= hd && rot % 2 == 0, "rope_kv: rotated width %d must be even and at most head_dim %d", rot, hd);
   DLGO_REQUIRE(ld >= (n_heads + 2 * n_kv) * hd, "rope_kv: row stride %d shorter than the heads it holds", ld);
@@ -246,17 +264,20 @@ extern "C" const char* dlgo_rope_kv(void* qkv, int dtype, int n_tokens, int ld, 
   if (pieces) {
     const long long items = (long long)n_tokens * (n_heads + (write_kv ? n_kv : 0)) * (hd / epc);
     const long long piece_blocks = (items + 255) / 256;
-    const long long value_blocks = write_kv ? (long long)((n_tokens + 63) / 64) * n_kv * ((hd + 63) / 64) : 0;
+    // single_tokens: every row is a sequence of its own (a decode step); the values then go thread by thread
+    const long long value_blocks = !write_kv ? 0
+                                   : single_tokens ? ((long long)n_tokens * n_kv * (hd / epc) + 255) / 256
+                                                   : (long long)((n_tokens + 63) / 64) * n_kv * ((hd + 63) / 64);
     DLGO_REQUIRE(piece_blocks + value_blocks < (1ll << 31), "rope_kv: too many rows at once");
     dim3 g((unsigned)(piece_blocks + value_blocks));
     if (dtype == DLGO_DTYPE_F32)
       hipLaunchKernelGGL(rope_kv_pieces_kernel<float>, g, dim3(256), 0, stream, (float*)qkv, ld, n_tokens, n_heads, n_kv, hd, rot,
                          interleaved, cos_t, sin_t, positions, tok_seq, slots, page_table, max_pages, (float*)cache, page_stride,
-                         v_off, write_kv, (int)piece_blocks, part, n_parts, plane, part_ld);
+                         v_off, write_kv, (int)piece_blocks, part, n_parts, plane, part_ld, single_tokens);
     else if (dtype == DLGO_DTYPE_BF16)
       hipLaunchKernelGGL(rope_kv_pieces_kernel<bf16_t>, g, dim3(256), 0, stream, (bf16_t*)qkv, ld, n_tokens, n_heads, n_kv, hd, rot,
                          interleaved, cos_t, sin_t, positions, tok_seq, slots, page_table, max_pages, (bf16_t*)cache, page_stride,
-                         v_off, write_kv, (int)piece_blocks, part, n_parts, plane, part_ld);
+                         v_off, write_kv, (int)piece_blocks, part, n_parts, plane, part_ld, single_tokens);
     else
       DLGO_FAIL("rope_kv: unknown dtype code %d", dtype);
     DLGO_LAUNCH_CHECK("rope_kv");

@@ -367,10 +367,12 @@ def rope_kv(qkv: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, rot: int,
             cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
             tok_seq: Optional[torch.Tensor], slots: Optional[torch.Tensor], page_table: Optional[torch.Tensor],
             cache: Optional[torch.Tensor], page_stride: int, v_off: int, write_kv: bool = True,
-            unsummed: Optional[UnsummedRows] = None) -> None:
+            unsummed: Optional[UnsummedRows] = None, single_tokens: bool = False) -> None:
     """Rotate the query heads of qkv [T, (H+2KV)*hd] in place; rotate the key heads and copy the value heads
     into the cache page of each token (cache: the first element of this layer's pages).  unsummed: the rows are not
-    in qkv yet but in the runs that gemm_runs left (see rope_takes_unsummed); the rotated queries are written to qkv."""
+    in qkv yet but in the runs that gemm_runs left (see rope_takes_unsummed); the rotated queries are written to qkv.
+    single_tokens: every row is a sequence of its own (a hint for how the transposed values are best stored; the
+    result is the same)."""
     _need(qkv, "qkv rows", dims=2)
     _need(positions, "positions", torch.int32, 1)
     t = qkv.shape[0]
@@ -400,7 +402,8 @@ def rope_kv(qkv: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, rot: int,
     _check(_lib("rope_kv").dlgo_rope_kv(_ptr(qkv), dtype_code(qkv.dtype), t, _rows(qkv, "qkv rows"), n_heads, n_kv, head_dim,
                                         rot, int(interleaved), _ptr(cos), _ptr(sin), table_rows, _ptr(positions),
                                         _ptr(tok_seq), _ptr(slots), _ptr(page_table), max_pages, _ptr(cache),
-                                        ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(write_kv), *part, _stream()))
+                                        ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(write_kv), *part,
+                                        int(single_tokens), _stream()))
 
 
 def rope_takes_unsummed(dtype: torch.dtype, head_dim: int, rot: int) -> bool:

@@ -486,14 +486,17 @@ def test_rope_kv_from_unsummed_runs(dtype, _, rel, H, KV, hd, rot, inter, write)
     cos, sin = torch.from_numpy(np.cos(ang).astype(np.float32)).to(DEV), torch.from_numpy(np.sin(ang).astype(np.float32)).to(DEV)
     slot_t = torch.tensor(slots, dtype=torch.int32, device=DEV)
     got = []
-    for unsummed in (None, ops.UnsummedRows(planes.reshape(-1).to(DEV), 3, T, cols)):
+    # the third way stores the values thread by thread (the arrangement for steps of single tokens): the same pages
+    for unsummed, single in ((None, False), (ops.UnsummedRows(planes.reshape(-1).to(DEV), 3, T, cols), False),
+                             (ops.UnsummedRows(planes.reshape(-1).to(DEV), 3, T, cols), True), (None, True)):
         dq = rows.to(dtype).to(DEV) if unsummed is None else torch.full_like(rows, float("nan")).to(dtype).to(DEV)
         store = storage.clone().to(DEV)
         ops.rope_kv(dq, H, KV if write else 0, hd, rot, inter, cos, sin, positions, tok_seq, slot_t, table.to(DEV),
-                    store[unit_off:], page_stride, v_off, write_kv=write, unsummed=unsummed)
+                    store[unit_off:], page_stride, v_off, write_kv=write, unsummed=unsummed, single_tokens=single)
         got.append((dq[:, :H * hd].cpu(), store.cpu()))
-    assert torch.equal(got[0][0], got[1][0]), "rotated queries"
-    assert torch.equal(torch.nan_to_num(got[0][1].float(), nan=-77.0), torch.nan_to_num(got[1][1].float(), nan=-77.0)), "pages"
+    for other in got[1:]:
+        assert torch.equal(got[0][0], other[0]), "rotated queries"
+        assert torch.equal(torch.nan_to_num(got[0][1].float(), nan=-77.0), torch.nan_to_num(other[1].float(), nan=-77.0)), "pages"
 
 
 def _attention_ref(q, k, v, H, KV, hd, pos_of_q, lo_of_q):
