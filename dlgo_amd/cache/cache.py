@@ -184,6 +184,49 @@ class Cache:
         self.lengths[slot] = 0
         self._free_slots.append(slot)
 
+    def copy_slot(self, src: int, length: Optional[int] = None) -> int:
+        """A new slot that holds what `src` holds below `length` (all of it by default): keys and values are copied page
+        by page into pages of its own, per-sequence state is copied as it is now.  computerex/dlgo: KVCache.Clone
+        (memory/kvcache.go:38-55).  State is not a function of a length, so with state units only the whole sequence
+        can be copied; a windowed group must still hold every page that a token at `length` sees."""
+        self._check_live(src)
+        have = int(self.lengths[src])
+        n = have if length is None else int(length)
+        if n < 0 or n > have:
+            raise CacheError(f"copy_slot: slot {src} holds {have} tokens, {n} asked")
+        if n != have and self.state:
+            raise CacheError("copy_slot: per-sequence state cannot be copied at an earlier length")
+        if not self._free_slots:
+            raise CacheError(f"no free slot: all {self.max_slots} are in use")
+        plans = []
+        for gi, g in enumerate(self.groups):
+            held = self._held[src][gi]
+            last = (n - 1) // PAGE if n > 0 else -1
+            idx = list(range(g.first_needed_page(n), last + 1))
+            missing = [i for i in idx if i not in held]
+            if missing:
+                raise CacheError(f"copy_slot: slot {src} no longer holds pages {missing} that a token at {n} sees")
+            if len(idx) > g.pool.n_free:
+                raise OutOfPages(f"cache full: the copy needs {len(idx)} pages of {PAGE} tokens, {g.pool.n_free} of {g.pool.n_pages} are free")
+            plans.append(idx)
+        dst = self.alloc_slot()
+        for gi, (g, idx) in enumerate(zip(self.groups, plans)):
+            if not idx:
+                continue
+            pages = g.pool.take(len(idx))
+            src_pages = [self._held[src][gi][i] for i in idx]
+            for i, p in zip(idx, pages):
+                self._held[dst][gi][i] = p
+                g.table_host[dst, i] = p
+            g.dirty.add(dst)
+            by_page = g.storage.view(g.pool.n_pages, g.page_stride)
+            by_page[torch.as_tensor(pages, dtype=torch.int64, device=self.device)] = \
+                by_page[torch.as_tensor(src_pages, dtype=torch.int64, device=self.device)]
+        self.lengths[dst] = n
+        for t in self.state.values():
+            t[dst].copy_(t[src])
+        return dst
+
     def _check_live(self, slot: int) -> None:
         if not (0 <= slot < self.max_slots) or not self._live[slot]:
             raise CacheError(f"slot {slot} is not in use")

@@ -155,6 +155,13 @@ class Engine:
             raise EngineError(f"{n} sequences asked, {self.cache.n_free_slots} slots free")
         return [self.cache.alloc_slot() for _ in range(n)]
 
+    def fork(self, slot: int, length: Optional[int] = None) -> int:
+        """A new sequence that starts as a copy of `slot` (its first `length` tokens; all by default) and goes its own
+        way from there: the next step may give the two different tokens."""
+        new = self.cache.copy_slot(slot, length)
+        self.cache.sync_tables()
+        return new
+
     def close(self, slots: Sequence[int]) -> None:
         for s in slots:
             self.cache.free_slot(s)

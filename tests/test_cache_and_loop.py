@@ -103,6 +103,72 @@ def test_groups_by_need_and_window_release():
     assert all(g.pool.n_free == g.pool.n_pages for g in c.groups)
 
 
+def test_copy_of_a_slot_has_pages_of_its_own():
+    """memory/kvcache.go:38-55 (Clone): a deep copy up to a position.  Here: pages of its own with the same content, the
+    same length, the state as it is; nothing shared, so either can go on or be given back without the other noticing."""
+    needs = [[CacheNeed("kv", 2, 16)], [CacheNeed("kv", 2, 16, window=100)], [CacheNeed("kv", 2, 16), CacheNeed("state", state_shape=(3,))]]
+    c = Cache(needs, 64 * PAGE, 32 * PAGE, torch.float32, "cpu", max_slots=4, max_step_tokens=128)
+    a = c.alloc_slot()
+    total = 0
+    for step in [128, 100, 1, 64]:
+        c.reserve([(a, total + step)])
+        c.advance(a, step)
+        total += step
+    for g in c.groups:                                   # every page of the pool tells its own number
+        g.storage.view(g.pool.n_pages, g.page_stride)[:] = torch.arange(g.pool.n_pages, dtype=torch.float32)[:, None]
+    c.state_of(2)[a] = torch.tensor([1.0, 2.0, 3.0])
+    b = c.copy_slot(a)
+    c.check_consistent()
+    assert b != a and c.length(b) == total == 293
+    for gi, g in enumerate(c.groups):
+        pa, pb = c.held_pages(a, gi), c.held_pages(b, gi)
+        assert sorted(pa) == sorted(pb) and not set(pa.values()) & set(pb.values())
+        by_page = g.storage.view(g.pool.n_pages, g.page_stride)
+        for i in pa:
+            assert torch.equal(by_page[pb[i]], by_page[pa[i]]) and by_page[pb[i]][0] == pa[i]
+        assert (g.table_host[b, sorted(pb)] == [pb[i] for i in sorted(pb)]).all()
+    assert torch.equal(c.state_of(2)[b], torch.tensor([1.0, 2.0, 3.0]))
+    # the two go their own ways
+    c.reserve([(b, total + 70)])
+    c.advance(b, 70)
+    assert c.length(a) == total and c.length(b) == total + 70
+    c.free_slot(a)
+    c.check_consistent()
+    assert c.length(b) == total + 70 and len(c.held_pages(b, 0)) == (total + 70 + PAGE - 1) // PAGE
+    c.free_slot(b)
+    assert all(g.pool.n_free == g.pool.n_pages for g in c.groups)
+    # an earlier length: only where nothing depends on what came after it
+    plain = make_cache(n_units=2, max_tokens=8 * PAGE, max_ctx=4 * PAGE)
+    s = plain.alloc_slot()
+    plain.reserve([(s, 150)])
+    plain.advance(s, 150)
+    t = plain.copy_slot(s, 70)
+    assert plain.length(t) == 70 and sorted(plain.held_pages(t)) == [0, 1]
+    with pytest.raises(CacheError, match="holds 150 tokens"):
+        plain.copy_slot(s, 151)
+    u = c.alloc_slot()
+    c.reserve([(u, 10)])
+    c.advance(u, 10)
+    with pytest.raises(CacheError, match="state"):
+        c.copy_slot(u, 5)
+    windowed = Cache([[CacheNeed("kv", 2, 16, window=100)]], 64 * PAGE, 32 * PAGE, torch.float32, "cpu", max_slots=4, max_step_tokens=128)
+    w = windowed.alloc_slot()
+    for step in [128, 128, 128]:
+        windowed.reserve([(w, windowed.length(w) + step)])
+        windowed.advance(w, step)
+    with pytest.raises(CacheError, match="no longer holds"):
+        windowed.copy_slot(w, 100)
+    # no room: nothing changes
+    full = make_cache(n_units=1, max_tokens=4 * PAGE, max_ctx=4 * PAGE, max_slots=3)
+    f = full.alloc_slot()
+    full.reserve([(f, 3 * PAGE)])
+    full.advance(f, 3 * PAGE)
+    with pytest.raises(CacheError, match="cache full"):
+        full.copy_slot(f)
+    full.check_consistent()
+    assert full.live_slots() == [f] and full.groups[0].pool.n_free == 1
+
+
 def test_state_is_zeroed_when_a_slot_is_handed_out():
     c = Cache([[CacheNeed("state", state_shape=(5,), state_dtype=torch.float32)]], PAGE, PAGE, torch.float32, "cpu", max_slots=2)
     s = c.alloc_slot()

@@ -143,6 +143,41 @@ def test_unequal_batches_with_slot_reuse(folders, oracle, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "D"])
+def test_a_forked_sequence_goes_its_own_way(folders, oracle, name, dtype):
+    """memory/kvcache.go:38-55 (Clone): a sequence is copied after its prompt (and one at an earlier length); the copies
+    and the original then take different tokens in the same steps, and each gives the logits of its own whole
+    sequence.  The original is closed half way: the copies hold nothing of it."""
+    from dlgo_amd.engine import Entry
+    raw = CONFIGS[name][0]
+    eng = engine_for(folders[name, dtype], dtype, max_tokens=16 * 64, max_slots=4)
+    prompt, = prompts_for(raw, [70], seed=11)
+    tails = prompts_for(raw, [9, 9, 9], seed=12)
+    (a,) = eng.open(1)
+    eng.step([Entry(a, prompt, [])])
+    b = eng.fork(a)
+    c = eng.fork(a, 33)                       # not at a page's edge: the copy's last page holds tokens it must not see
+    assert (eng.length(a), eng.length(b), eng.length(c)) == (70, 70, 33)
+    seqs = {a: prompt + tails[0], b: prompt + tails[1], c: prompt[:33] + tails[2]}
+    got = {s: [] for s in seqs}
+    live = [a, b, c]
+    for step in range(9):
+        if step == 4:
+            eng.close([a])
+            live.remove(a)
+        out = eng.step([Entry(s, [seqs[s][eng.length(s)]], [0]) for s in live]).cpu().numpy()
+        for r, s in enumerate(live):
+            got[s].append(out[r])
+    eng.cache.check_consistent()
+    for s, rows in got.items():
+        want = oracle(name, dtype, seqs[s])
+        first = len(seqs[s]) - 9
+        assert rel_err(np.stack(rows), want[first:first + len(rows)]) <= TOL[dtype], (name, dtype, s)
+    eng.close([b, c])
+    assert eng.cache.n_free_slots == 4 and all(g.pool.n_free == g.pool.n_pages for g in eng.cache.groups)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_step_cut_into_pieces_and_batch_mates(folders, oracle, dtype):
     """A step with more rows than the workspace holds is cut along the rows; a request's logits do not
     depend on that nor on what else is in the batch."""
