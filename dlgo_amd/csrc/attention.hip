@@ -1543,6 +1543,12 @@ static void decode_plan(int n_pairs, int group, int max_pages_used, bool fused, 
   if (splits > max_pages_used) splits = max_pages_used;
   if (max_pages_used > w * 8 && splits < (max_pages_used + w * 8 - 1) / (w * 8)) splits = (max_pages_used + w * 8 - 1) / (w * 8);
   if (splits > 1 && w > 8 && !through_lds) w = 8;
+  if (through_lds && splits > 1) {
+    // more waves than a sequence can have pages: a wave without a page only adds to the merge.  Halve the waves of a
+    // block (down to 4), then deal the pages to fewer blocks (one sequence at 2,000 to 4,000 tokens: 11.4 -> 10.0 us)
+    while (w > 4 && splits * w > max_pages_used) w >>= 1;
+    if (splits * w > max_pages_used) splits = (max_pages_used + w - 1) / w;
+  }
   *nwv = w;
   *n_splits = splits;
 }
