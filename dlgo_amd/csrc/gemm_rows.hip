@@ -268,17 +268,18 @@ static __device__ __forceinline__ void row_to_lds(const void* base, uint32_t vof
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(base) : "memory");
 }
 typedef uint32_t rows_u32x4_t __attribute__((ext_vector_type(4)));
-
-// What a product may do for the norm that follows it, or take from the product before it (see dlgo_gemm_rows_leave_parts and dlgo_gemm_rows_scaled):
-//   MODE 1 (with the epilogue that adds into the float32 residual rows): beside the new residual rows it leaves
-//     x * norm_w of them in the run dtype, not yet scaled, and each block its 16 columns' share of every row's sum of squares;
-//   MODE 2: its X are such unscaled rows; the shares are added up in a fixed order and the scale 1/sqrt(sum/width + eps)
-//     multiplies the finished sums (it is a scalar per token), before the epilogue.
 static __device__ __forceinline__ uint4 lds_operand(const __attribute__((address_space(3))) char* p) {
   const rows_u32x4_t v = *(const __attribute__((address_space(3))) rows_u32x4_t*)p;
   return make_uint4(v.x, v.y, v.z, v.w);
 }
 
+// What a product may do for the norm that follows it, or take from the product before it (see
+// dlgo_gemm_rows_leave_parts and dlgo_gemm_rows_scaled):
+//   MODE 1 (with the epilogue that adds into the float32 residual rows): beside the new residual rows it leaves
+//     x * norm_w of them in the run dtype, not yet scaled, and each group of 16 columns its share of every row's sum of
+//     squares;
+//   MODE 2: its X are such unscaled rows; the shares are added up in a fixed order and the scale 1/sqrt(sum/width + eps)
+//     multiplies the finished sums (it is a scalar per token), before the epilogue.
 constexpr int NORM_PARTS_MAX = 256;   // most shares of a row's sum of squares (a normed width of 4096)
 
 struct NormParts {
