@@ -232,6 +232,209 @@ __device__ int sample_small(SampleSmall& S, int n, int k, BestIdx top, float tp,
   return pick >= 0 ? S.si[pick] : (top.i < 0 ? 0 : top.i);
 }
 
+// Rows with a small top-k (the reference's default options have 40) need not be walked by one block: whatever survives
+// top-k is among the largest k of its part of the row.  topk_part_kernel: TK_CHUNKS blocks a row; each keeps its part
+// of the row (with temperature and penalty applied) in LDS, finds the part's maximum and, by the same count of
+// distances below it as sample_kernel uses, a set of at most TK_CAP elements that holds the part's k largest (with
+// everything tied at the k-th), and leaves them in the row's scratch.  topk_final_kernel: one block a row gathers the
+// parts' sets, cuts them down the same way against the row's maximum and hands them to sample_small, which makes the
+// exact cuts and the draw.  An element that is missing from a part's set has k larger ones in its own part, so it is
+// below the k-th value of the row: the set that sample_small ends up with is the one sample_kernel would have had.
+// Whatever does not fit (a part with more than TK_CAP elements within its cut, no cut within 255 steps, a row
+// without top-k) is left to sample_kernel: the row's scratch says which rows are done.
+// The row's scratch (floats of its row of `work`): maxima [TK_CHUNKS] as (value, index), counts [TK_CHUNKS] (-1: this
+// part gave up), the done flag, then the parts' values [TK_CHUNKS][TK_CAP] and indices [TK_CHUNKS][TK_CAP].
+#define TK_CHUNKS 32
+#define TK_CAP 128
+#define TK_THREADS 256
+#define TK_CHUNK_MAX 8192                      // floats of a part that LDS takes: rows of up to 262,144
+#define TK_MIN_V 16384
+#define TK_COUNTS (2 * TK_CHUNKS)
+#define TK_DONE (3 * TK_CHUNKS)
+#define TK_VALUES 128
+#define TK_INDICES (TK_VALUES + TK_CHUNKS * TK_CAP)
+#define TK_SCRATCH (TK_INDICES + TK_CHUNKS * TK_CAP)
+
+__global__ __launch_bounds__(TK_THREADS) void topk_part_kernel(const float* __restrict__ logits, int ld, int V,
+                                                               float* __restrict__ work_all,
+                                                               const float* __restrict__ temperature,
+                                                               const int32_t* __restrict__ top_k, const float* __restrict__ penalty,
+                                                               const int32_t* __restrict__ recent, int n_recent,
+                                                               const int32_t* __restrict__ recent_rows,
+                                                               const int32_t* __restrict__ counts) {
+  __shared__ float xs[TK_CHUNK_MAX];
+  __shared__ BestIdx red[TK_THREADS / WAVE];
+  __shared__ int hist[256];
+  __shared__ int limit, n_kept;
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  float* scratch = work_all + (size_t)row * V;
+  int* cnt = (int*)scratch + TK_COUNTS;
+  if (chunk == 0 && threadIdx.x == 0) ((int*)scratch)[TK_DONE] = 0;
+  const float temp = temperature[row];
+  const int k = top_k[row];
+  if (!(temp > 0.f) || k < 1 || k > TK_CAP) {       // not a row for this way
+    if (threadIdx.x == 0) cnt[chunk] = -1;
+    return;
+  }
+  const int per = ((V + TK_CHUNKS - 1) / TK_CHUNKS + 3) & ~3;
+  const int c0 = chunk * per < V ? chunk * per : V, c1 = c0 + per < V ? c0 + per : V;
+  const float* lg = logits + (size_t)row * ld;
+  const float inv_temp = temp == 1.0f ? 1.0f : 1.0f / temp;
+  for (int i = c0 + threadIdx.x; i < c1; i += TK_THREADS) xs[i - c0] = inv_temp != 1.0f ? lg[i] * inv_temp : lg[i];
+  if (threadIdx.x < 256) hist[threadIdx.x] = 0;
+  __syncthreads();
+  // repetition penalty: each distinct recent token once, as in sample_kernel
+  const float pen = penalty[row];
+  const int rr = recent_rows ? recent_rows[row] : row;
+  const int held = counts ? (counts[rr] < n_recent ? counts[rr] : n_recent) : n_recent;
+  if (pen > 1.0f && n_recent > 0) {
+    const int32_t* rc = recent + (size_t)rr * n_recent;
+    for (int t = threadIdx.x; t < held; t += TK_THREADS) {
+      const int tok = rc[t];
+      bool first = tok >= c0 && tok < c1;
+      for (int j = 0; first && j < t; ++j) first = rc[j] != tok;
+      if (first) {
+        const float x = lg[tok] > 0.f ? lg[tok] / pen : lg[tok] * pen;
+        xs[tok - c0] = inv_temp != 1.0f ? x * inv_temp : x;
+      }
+    }
+  }
+  __syncthreads();
+  BestIdx best = {-INFINITY, -1};
+  for (int i = c0 + threadIdx.x; i < c1; i += TK_THREADS) {
+    const float v = xs[i - c0];
+    if (v == v) best = better(best, BestIdx{v, i});
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    BestIdx other;
+    other.v = __shfl_xor(best.v, o, WAVE);
+    other.i = __shfl_xor(best.i, o, WAVE);
+    best = better(best, other);
+  }
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = best;
+  __syncthreads();
+  best = red[0];
+  for (int w = 1; w < TK_THREADS / WAVE; ++w) best = better(best, red[w]);
+  if (best.i < 0) {                               // an empty part, or nothing but NaN: nothing to offer
+    if (threadIdx.x == 0) {
+      cnt[chunk] = 0;
+      ((BestIdx*)scratch)[chunk] = best;
+    }
+    return;
+  }
+  const uint32_t kmax = order_key(best.v);
+  for (int i = c0 + threadIdx.x; i < c1; i += TK_THREADS) {
+    const uint32_t bin = (kmax - order_key(xs[i - c0])) >> 16;
+    if (bin < 255u) atomicAdd(&hist[bin], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    // the distance within which the k largest lie; if they do not lie within 255 steps, everything that does
+    int cum = 0, b = 0;
+    for (; b < 255; ++b) {
+      cum += hist[b];
+      if (cum >= k) break;
+    }
+    limit = cum <= TK_CAP ? (b < 255 ? b : 254) : -1;
+    n_kept = 0;
+  }
+  __syncthreads();
+  if (limit < 0) {
+    if (threadIdx.x == 0) cnt[chunk] = -1;
+    return;
+  }
+  float* cv = scratch + TK_VALUES + chunk * TK_CAP;
+  int* ci = (int*)scratch + TK_INDICES + chunk * TK_CAP;
+  for (int i = c0 + threadIdx.x; i < c1; i += TK_THREADS) {
+    const float x = xs[i - c0];
+    if (((kmax - order_key(x)) >> 16) <= (uint32_t)limit) {
+      const int slot = atomicAdd(&n_kept, 1);
+      cv[slot] = x;
+      ci[slot] = i;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    cnt[chunk] = n_kept;
+    ((BestIdx*)scratch)[chunk] = best;
+  }
+}
+
+__global__ __launch_bounds__(SAMP_THREADS) void topk_final_kernel(int V, float* __restrict__ work_all,
+                                                                  const float* __restrict__ temperature,
+                                                                  const int32_t* __restrict__ top_k, const float* __restrict__ top_p,
+                                                                  const float* __restrict__ min_p, int32_t* __restrict__ recent,
+                                                                  int n_recent, const int32_t* __restrict__ recent_rows,
+                                                                  int32_t* __restrict__ counts, const float* __restrict__ uniform,
+                                                                  int32_t* __restrict__ out) {
+  __shared__ SampleSmall S;
+  __shared__ int hist[256];
+  __shared__ int bstar, part_n[TK_CHUNKS];
+  __shared__ BestIdx top_s;
+  const int row = blockIdx.x;
+  float* scratch = work_all + (size_t)row * V;
+  const float temp = temperature[row];
+  const int k = top_k[row];
+  if (!(temp > 0.f) || k < 1 || k > TK_CAP) return;
+  if (threadIdx.x < TK_CHUNKS) part_n[threadIdx.x] = ((const int*)scratch)[TK_COUNTS + threadIdx.x];
+  if (threadIdx.x < 256) hist[threadIdx.x] = 0;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    BestIdx top = {-INFINITY, -1};
+    bool ok = true;
+    for (int c = 0; c < TK_CHUNKS; ++c) {
+      ok = ok && part_n[c] >= 0;
+      if (part_n[c] > 0) top = better(top, ((const BestIdx*)scratch)[c]);
+    }
+    top_s = top;
+    bstar = ok && top.i >= 0 ? 0 : -2;
+    S.n = 0;
+  }
+  __syncthreads();
+  if (bstar == -2) return;                        // a part gave up, or the row has nothing but NaN
+  const BestIdx top = top_s;
+  const uint32_t kmax = order_key(top.v);
+  const float* cv = scratch + TK_VALUES;
+  const int* ci = (const int*)scratch + TK_INDICES;
+  for (int e = threadIdx.x; e < TK_CHUNKS * TK_CAP; e += SAMP_THREADS)
+    if ((e % TK_CAP) < part_n[e / TK_CAP]) {
+      const uint32_t bin = (kmax - order_key(cv[e])) >> 16;
+      if (bin < 255u) atomicAdd(&hist[bin], 1);
+    }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int cum = 0, b = 0;
+    for (; b < 255; ++b) {
+      cum += hist[b];
+      if (cum >= k) break;
+    }
+    bstar = b < 255 && cum <= SAMP_CAND ? b : -1;
+  }
+  __syncthreads();
+  if (bstar < 0) return;
+  for (int e = threadIdx.x; e < TK_CHUNKS * TK_CAP; e += SAMP_THREADS)
+    if ((e % TK_CAP) < part_n[e / TK_CAP]) {
+      const float x = cv[e];
+      if (((kmax - order_key(x)) >> 16) <= (uint32_t)bstar) {
+        const int slot = atomicAdd(&S.n, 1);
+        S.cv[slot] = x;
+        S.ci[slot] = ci[e];
+      }
+    }
+  __syncthreads();
+  const int pick = sample_small(S, S.n, k, top, top_p[row], min_p[row], uniform[row]);
+  if (threadIdx.x == 0) {
+    out[row] = pick;
+    const int rr = recent_rows ? recent_rows[row] : row;
+    if (counts && n_recent > 0) {
+      recent[(size_t)rr * n_recent + counts[rr] % n_recent] = pick;
+      counts[rr] += 1;
+    }
+    ((int*)scratch)[TK_DONE] = 1;
+  }
+}
+
 __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __restrict__ logits, int ld, int V,
                                                               float* __restrict__ work_all,
                                                               const float* __restrict__ temperature,
@@ -239,7 +442,8 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
                                                               const float* __restrict__ min_p, const float* __restrict__ penalty,
                                                               int32_t* __restrict__ recent, int n_recent,
                                                               const int32_t* __restrict__ recent_rows, int32_t* __restrict__ counts,
-                                                              const float* __restrict__ uniform, int32_t* __restrict__ out) {
+                                                              const float* __restrict__ uniform, int32_t* __restrict__ out,
+                                                              int staged) {
   __shared__ BestIdx redb[SAMP_WAVES];
   __shared__ float red[SAMP_WAVES];
   __shared__ SampleSmall S;
@@ -248,6 +452,8 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
   __shared__ unsigned long long cut_before;
   float* scan = S.scan;
   const int row = blockIdx.x;
+  // staged: the kernels that deal a row to several blocks ran before this one and say which rows they finished
+  if (staged && ((const int*)(work_all + (size_t)row * V))[TK_DONE] != 0) return;
   const float* lg = logits + (size_t)row * ld;
   const float temp = temperature[row];
   if (!(temp > 0.f)) {   // greedy row
@@ -571,8 +777,16 @@ extern "C" const char* dlgo_sample(const float* logits, int ld, int n_rows, int 
   DLGO_REQUIRE(n_recent == 0 || recent, "sample: recent tokens missing");
   DLGO_REQUIRE((recent_rows == nullptr) == (counts == nullptr), "sample: a ring of recent tokens needs both its rows and its counts");
   if (n_rows == 0) return nullptr;
+  // a wide vocabulary: rows with a small top-k are dealt to several blocks first; sample_kernel takes what they leave
+  const int staged = V >= TK_MIN_V && V <= TK_CHUNKS * TK_CHUNK_MAX && V >= TK_SCRATCH && n_rows <= 65535;
+  if (staged) {
+    hipLaunchKernelGGL(topk_part_kernel, dim3(TK_CHUNKS, n_rows), dim3(TK_THREADS), 0, stream, logits, ld, V, work, temperature,
+                       top_k, penalty, recent, n_recent, recent_rows, counts);
+    hipLaunchKernelGGL(topk_final_kernel, dim3(n_rows), dim3(SAMP_THREADS), 0, stream, V, work, temperature, top_k, top_p, min_p,
+                       recent, n_recent, recent_rows, counts, uniform, out);
+  }
   hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMP_THREADS), 0, stream, logits, ld, V, work, temperature, top_k, top_p,
-                     min_p, penalty, recent, n_recent, recent_rows, counts, uniform, out);
+                     min_p, penalty, recent, n_recent, recent_rows, counts, uniform, out, staged);
   DLGO_LAUNCH_CHECK("sample");
   return nullptr;
 }

@@ -26,6 +26,11 @@ class Sampler:
         self._pinned = [torch.empty(max_rows, dtype=torch.int32, pin_memory=True) for _ in range(4)]
         self._pin_next = 0
         self._work: Optional[torch.Tensor] = None
+        # the rows' options go up in one copy from pinned memory that does not wait for the device: a copy from
+        # ordinary memory would hold the host until the step queued before it is done, and the step after it with it
+        self._staging: List[tuple] = []                 # (pinned int32 buffer, event of the copy that last read it)
+        self._staging_next = 0
+        self._options: Optional[torch.Tensor] = None    # the device's copy: 7 rows of int32/float32 bits
         self._rings: Optional[torch.Tensor] = None      # [keys, RECENT] last tokens chosen per key
         self._counts: Optional[torch.Tensor] = None     # [keys] tokens chosen so far per key
 
@@ -43,6 +48,31 @@ class Sampler:
             self._counts, self._rings = counts, rings
         if len(keys):
             self._counts[torch.as_tensor(list(keys), dtype=torch.long)] = 0
+
+    def _upload(self, f: np.ndarray, k: np.ndarray):
+        """f [5, n] float32 and k [2, n] int32 -> their device copies, through one pinned buffer and one copy that the
+        host does not wait for."""
+        n = f.shape[1]
+        if not self._staging:
+            self._staging = [(torch.empty(7 * max(n, self.max_rows), dtype=torch.int32, pin_memory=True), None) for _ in range(4)]
+        i = self._staging_next
+        self._staging_next = (i + 1) % len(self._staging)
+        buf, ev = self._staging[i]
+        if ev is not None:
+            ev.synchronize()
+        if buf.numel() < 7 * n:
+            buf = torch.empty(14 * n, dtype=torch.int32, pin_memory=True)
+        hv = buf.numpy()
+        hv[:5 * n] = f.reshape(-1).view(np.int32)
+        hv[5 * n:7 * n] = k.reshape(-1)
+        if self._options is None or self._options.numel() < 7 * n:
+            self._options = torch.empty(14 * n, dtype=torch.int32, device=self.device)
+        dev = self._options[:7 * n]
+        dev.copy_(buf[:7 * n], non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self._staging[i] = (buf, ev)
+        return dev[:5 * n].view(torch.float32).view(5, n), dev[5 * n:].view(2, n)
 
     def _grow(self, rows: int) -> None:
         if rows > self._out.shape[0]:
@@ -104,8 +134,7 @@ class Sampler:
             if self._counts is None or max(keys) >= self._counts.shape[0]:
                 raise ValueError("sampler: keys that start() was never given")
             k[1] = np.asarray(keys, dtype=np.int32)
-        fd = torch.from_numpy(f).to(self.device)
-        kd = torch.from_numpy(k).to(self.device)
+        fd, kd = self._upload(f, k)
         if rings:       # every choice is recorded, penalty or not: a later row of the request may have one
             ops.sample(logits, self._work, fd[0], kd[0], fd[1], fd[2], fd[3], self._rings, fd[4], out,
                        recent_rows=kd[1], counts=self._counts)

@@ -793,6 +793,59 @@ def test_sample_top_k_in_awkward_rows():
             assert got == want, (c, u)
 
 
+def test_sample_wide_rows_dealt_to_several_blocks():
+    """A wide vocabulary with a small top-k: a row's parts go to blocks of their own first, and whatever they cannot
+    finish falls to the one-block kernel.  Rows of every kind in one call, each with its own options: a plain one, one
+    whose kept values are tied beyond what a part may keep (200 equal values in one part), one whose k-th value lies
+    far below the maximum, ties across parts at the cut, a row without top-k, a greedy row, k at and beyond the limit
+    of this way, a penalised maximum."""
+    import plain_llama as plain
+    ops = _ops()
+    g = torch.Generator().manual_seed(11)
+    v = 128256
+    rows, opts, recents = [], [], []
+
+    def add(r, recent=(), **c):
+        rows.append(r)
+        opts.append(c)
+        recents.append(list(recent))
+    add(torch.randn(v, generator=g) * 2, temp=0.7, top_k=40, top_p=0.9, pen=1.1, recent=[5, 77, 5])
+    r = torch.randn(v, generator=g) * 2
+    r[9000:9200] = 11.0
+    add(r, temp=1.0, top_k=50)
+    r = torch.randn(v, generator=g) * 0.01 - 40.0
+    r[70007] = 30.0
+    add(r, temp=1.0, top_k=5)
+    r = torch.randn(v, generator=g)
+    r[3::4001] = 6.5                         # 33 equal values, one in every part, straddling the cut at k = 20
+    add(r, temp=0.9, top_k=20, top_p=0.95)
+    add(torch.randn(v, generator=g) * 3, temp=0.8)
+    add(torch.randn(v, generator=g) * 3, temp=0.0, top_k=40)
+    add(torch.randn(v, generator=g) * 3, temp=1.2, top_k=128, min_p=0.01)
+    add(torch.randn(v, generator=g) * 3, temp=1.2, top_k=129, top_p=0.99)
+    r = torch.randn(v, generator=g) * 2
+    top = int(r.argmax())
+    add(r, temp=0.5, top_k=3, pen=4.0, recent=[top, int(r.topk(2).indices[1])])
+    n = len(rows)
+    width = max(len(x) for x in recents) or 1
+    rec = torch.full((n, width), -1, dtype=torch.int32)
+    for i, x in enumerate(recents):
+        rec[i, :len(x)] = torch.tensor(x, dtype=torch.int32)
+    lg = torch.stack(rows).to(DEV)
+    col = lambda name, default, dt: torch.tensor([c.get(name, default) for c in opts], dtype=dt, device=DEV)
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    work = torch.empty(n, v, device=DEV)
+    for u in (0.00137, 0.2031, 0.5531, 0.8973, 0.99951):
+        ops.sample(lg, work, col("temp", 1.0, torch.float32), col("top_k", 0, torch.int32), col("top_p", 1.0, torch.float32),
+                   col("min_p", 0.0, torch.float32), col("pen", 1.0, torch.float32), rec.to(DEV),
+                   torch.full((n,), u, dtype=torch.float32, device=DEV), out)
+        got = out.tolist()
+        for i, c in enumerate(opts):
+            want = plain.sample_token(rows[i].double().numpy(), u, c["temp"], c.get("top_k", 0), c.get("top_p", 1.0),
+                                      c.get("min_p", 0.0), c.get("pen", 1.0), recents[i])
+            assert got[i] == want, (i, c, u)
+
+
 def test_sample_reference_behaviour():
     """ops/sampling_test.go: a dominant logit is always drawn (:18-30); temperature 2 halves the logits (:48-57)."""
     logits = torch.zeros(1, 50)
