@@ -147,6 +147,8 @@ class Cache:
             group.pages_per_seq = per_seq       # the most pages one sequence holds of this group at any time
             self.groups.append(group)
 
+        self._stages: list = []          # staging for sync_tables
+        self._stage_next = 0
         self._free_slots = list(range(self.max_slots - 1, -1, -1))
         self._live = np.zeros(self.max_slots, dtype=bool)
         self.lengths = np.zeros(self.max_slots, dtype=np.int64)
@@ -314,19 +316,46 @@ class Cache:
         else:
             self.lengths[slots] += n_tokens
 
+    def _table_stage(self, n_rows: int):
+        """Pinned host buffers (row numbers, rows) that no copy in flight still reads, and their device twins."""
+        if not self._stages:
+            self._stages = [None] * 4
+        i = self._stage_next
+        self._stage_next = (i + 1) % len(self._stages)
+        st = self._stages[i]
+        if st is not None and st[4] is not None:
+            st[4].synchronize()
+        if st is None or st[0].shape[0] < n_rows:
+            cap = max(2 * n_rows, 64)
+            st = [torch.empty(cap, dtype=torch.int64, pin_memory=True),
+                  torch.empty((cap, self.max_pages_per_seq), dtype=torch.int32, pin_memory=True),
+                  torch.empty(cap, dtype=torch.int64, device=self.device),
+                  torch.empty((cap, self.max_pages_per_seq), dtype=torch.int32, device=self.device), None]
+            self._stages[i] = st
+        return st
+
     def sync_tables(self) -> None:
-        """Bring the device page tables up to date (rows of slots that changed)."""
+        """Bring the device page tables up to date (rows of slots that changed).  The rows travel through pinned memory in
+        copies that the host does not wait for: a copy from ordinary memory would hold it until the device has caught up,
+        and a loop that queues a step ahead would lose its lead at every page a sequence begins."""
         for g in self.groups:
             if not g.dirty:
                 continue
             rows = sorted(g.dirty)
             g.dirty.clear()
-            idx = torch.as_tensor(rows, dtype=torch.int64)
-            host = torch.from_numpy(g.table_host[rows])
-            if self.device.type == "cuda":
-                g.table.index_copy_(0, idx.to(self.device), host.to(self.device))
-            else:
-                g.table.index_copy_(0, idx, host)
+            if self.device.type != "cuda":
+                g.table.index_copy_(0, torch.as_tensor(rows, dtype=torch.int64), torch.from_numpy(g.table_host[rows]))
+                continue
+            n = len(rows)
+            st = self._table_stage(n)
+            st[0].numpy()[:n] = rows
+            st[1].numpy()[:n] = g.table_host[rows]
+            st[2][:n].copy_(st[0][:n], non_blocking=True)
+            st[3][:n].copy_(st[1][:n], non_blocking=True)
+            g.table.index_copy_(0, st[2][:n], st[3][:n])
+            ev = torch.cuda.Event()
+            ev.record()
+            st[4] = ev
 
     # -- views for the parts --------------------------------------------------
     def kv_view(self, unit: int) -> "KVView":
