@@ -232,6 +232,46 @@ __device__ int sample_small(SampleSmall& S, int n, int k, BestIdx top, float tp,
   return pick >= 0 ? S.si[pick] : (top.i < 0 ? 0 : top.i);
 }
 
+// The first of the 255 bins of `hist` at which the running count reaches k, found by the block's first wave (four bins
+// a lane, a scan over the lanes, then the lane's own four): *bin = that bin or 255 if none does, *cum = the count up to
+// and including it (all of them if none does).  Every thread of wave 0 must call it; the results are in lane 0.
+__device__ __forceinline__ void first_bin_reaching(const int* hist, int k, int* bin, int* cum) {
+  const int lane = threadIdx.x & 63;
+  int h[4], mine = 0;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    h[q] = 4 * lane + q < 255 ? hist[4 * lane + q] : 0;
+    mine += h[q];
+  }
+  int incl = mine;
+#pragma unroll
+  for (int o = 1; o < WAVE; o <<= 1) {
+    const int y = __shfl_up(incl, o, WAVE);
+    if (lane >= o) incl += y;
+  }
+  const unsigned long long hit = __ballot(incl >= k);
+  const int total = __shfl(incl, WAVE - 1, WAVE);
+  if (!hit) {
+    *bin = 255;
+    *cum = total;
+    return;
+  }
+  const int owner = __ffsll((long long)hit) - 1;
+  int c = __shfl(incl - mine, owner, WAVE), b = 4 * owner;
+  const int h0 = __shfl(h[0], owner, WAVE), h1 = __shfl(h[1], owner, WAVE), h2 = __shfl(h[2], owner, WAVE), h3 = __shfl(h[3], owner, WAVE);
+  const int hs[4] = {h0, h1, h2, h3};
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    c += hs[q];
+    if (c >= k) {
+      b += q;
+      break;
+    }
+  }
+  *bin = b;
+  *cum = c;
+}
+
 // Rows with a small top-k (the reference's default options have 40) need not be walked by one block: whatever survives
 // top-k is among the largest k of its part of the row.  topk_part_kernel: TK_CHUNKS blocks a row; each keeps its part
 // of the row (with temperature and penalty applied) in LDS, finds the part's maximum and, by the same count of
@@ -266,6 +306,7 @@ __global__ __launch_bounds__(TK_THREADS) void topk_part_kernel(const float* __re
   __shared__ BestIdx red[TK_THREADS / WAVE];
   __shared__ int hist[256];
   __shared__ int limit, n_kept;
+  __shared__ int rcs[SAMP_THREADS];               // the row's recent tokens
   const int row = blockIdx.y, chunk = blockIdx.x;
   float* scratch = work_all + (size_t)row * V;
   int* cnt = (int*)scratch + TK_COUNTS;
@@ -280,15 +321,45 @@ __global__ __launch_bounds__(TK_THREADS) void topk_part_kernel(const float* __re
   const int c0 = chunk * per < V ? chunk * per : V, c1 = c0 + per < V ? c0 + per : V;
   const float* lg = logits + (size_t)row * ld;
   const float inv_temp = temp == 1.0f ? 1.0f : 1.0f / temp;
-  for (int i = c0 + threadIdx.x; i < c1; i += TK_THREADS) xs[i - c0] = inv_temp != 1.0f ? lg[i] * inv_temp : lg[i];
+  // the part into LDS, every load on its way before the first is used where the row allows 16-byte loads
+  if ((ld & 3) == 0 && ((uintptr_t)logits & 15) == 0 && ((c1 - c0) & 3) == 0) {
+    const float4* src = (const float4*)(lg + c0);
+    const int n4 = (c1 - c0) >> 2;
+    constexpr int U = TK_CHUNK_MAX / 4 / TK_THREADS;       // 8
+    float4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = u * TK_THREADS + threadIdx.x;
+      v[u] = i < n4 ? src[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = u * TK_THREADS + threadIdx.x;
+      if (i < n4) {
+        float4 x = v[u];
+        if (inv_temp != 1.0f) {
+          x.x *= inv_temp;
+          x.y *= inv_temp;
+          x.z *= inv_temp;
+          x.w *= inv_temp;
+        }
+        ((float4*)xs)[i] = x;
+      }
+    }
+  } else {
+    for (int i = c0 + threadIdx.x; i < c1; i += TK_THREADS) xs[i - c0] = inv_temp != 1.0f ? lg[i] * inv_temp : lg[i];
+  }
   if (threadIdx.x < 256) hist[threadIdx.x] = 0;
-  __syncthreads();
-  // repetition penalty: each distinct recent token once, as in sample_kernel
+  // repetition penalty: each distinct recent token once, as in sample_kernel (the list is looked through in LDS)
   const float pen = penalty[row];
   const int rr = recent_rows ? recent_rows[row] : row;
   const int held = counts ? (counts[rr] < n_recent ? counts[rr] : n_recent) : n_recent;
-  if (pen > 1.0f && n_recent > 0) {
-    const int32_t* rc = recent + (size_t)rr * n_recent;
+  const bool penalised = pen > 1.0f && n_recent > 0;
+  if (penalised)
+    for (int t = threadIdx.x; t < held; t += TK_THREADS) rcs[t] = recent[(size_t)rr * n_recent + t];
+  __syncthreads();
+  if (penalised) {
+    const int* rc = rcs;
     for (int t = threadIdx.x; t < held; t += TK_THREADS) {
       const int tok = rc[t];
       bool first = tok >= c0 && tok < c1;
@@ -329,15 +400,14 @@ __global__ __launch_bounds__(TK_THREADS) void topk_part_kernel(const float* __re
     if (bin < 255u) atomicAdd(&hist[bin], 1);
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
+  if (threadIdx.x < WAVE) {
     // the distance within which the k largest lie; if they do not lie within 255 steps, everything that does
-    int cum = 0, b = 0;
-    for (; b < 255; ++b) {
-      cum += hist[b];
-      if (cum >= k) break;
+    int cum, b;
+    first_bin_reaching(hist, k, &b, &cum);
+    if (threadIdx.x == 0) {
+      limit = cum <= TK_CAP ? (b < 255 ? b : 254) : -1;
+      n_kept = 0;
     }
-    limit = cum <= TK_CAP ? (b < 255 ? b : 254) : -1;
-    n_kept = 0;
   }
   __syncthreads();
   if (limit < 0) {
@@ -377,19 +447,30 @@ __global__ __launch_bounds__(SAMP_THREADS) void topk_final_kernel(int V, float* 
   const float temp = temperature[row];
   const int k = top_k[row];
   if (!(temp > 0.f) || k < 1 || k > TK_CAP) return;
-  if (threadIdx.x < TK_CHUNKS) part_n[threadIdx.x] = ((const int*)scratch)[TK_COUNTS + threadIdx.x];
+  __shared__ BestIdx part_top[TK_CHUNKS];
+  if (threadIdx.x < TK_CHUNKS) {
+    part_n[threadIdx.x] = ((const int*)scratch)[TK_COUNTS + threadIdx.x];
+    part_top[threadIdx.x] = ((const BestIdx*)scratch)[threadIdx.x];
+  }
   if (threadIdx.x < 256) hist[threadIdx.x] = 0;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    BestIdx top = {-INFINITY, -1};
-    bool ok = true;
-    for (int c = 0; c < TK_CHUNKS; ++c) {
-      ok = ok && part_n[c] >= 0;
-      if (part_n[c] > 0) top = better(top, ((const BestIdx*)scratch)[c]);
+  if (threadIdx.x < WAVE) {
+    const int c = threadIdx.x;
+    BestIdx top = c < TK_CHUNKS && part_n[c] > 0 ? part_top[c] : BestIdx{-INFINITY, -1};
+    const bool gave_up = c < TK_CHUNKS && part_n[c] < 0;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      BestIdx other;
+      other.v = __shfl_xor(top.v, o, WAVE);
+      other.i = __shfl_xor(top.i, o, WAVE);
+      top = better(top, other);
     }
-    top_s = top;
-    bstar = ok && top.i >= 0 ? 0 : -2;
-    S.n = 0;
+    const bool ok = __ballot(gave_up) == 0ull;
+    if (threadIdx.x == 0) {
+      top_s = top;
+      bstar = ok && top.i >= 0 ? 0 : -2;
+      S.n = 0;
+    }
   }
   __syncthreads();
   if (bstar == -2) return;                        // a part gave up, or the row has nothing but NaN
@@ -397,30 +478,38 @@ __global__ __launch_bounds__(SAMP_THREADS) void topk_final_kernel(int V, float* 
   const uint32_t kmax = order_key(top.v);
   const float* cv = scratch + TK_VALUES;
   const int* ci = (const int*)scratch + TK_INDICES;
-  for (int e = threadIdx.x; e < TK_CHUNKS * TK_CAP; e += SAMP_THREADS)
-    if ((e % TK_CAP) < part_n[e / TK_CAP]) {
-      const uint32_t bin = (kmax - order_key(cv[e])) >> 16;
+  // the thread's share of what the parts offer, asked for at once: slots threadIdx.x, + 1024, ...
+  constexpr int PER = TK_CHUNKS * TK_CAP / SAMP_THREADS;
+  float mine_v[PER];
+  int mine_i[PER];
+  bool mine[PER];
+#pragma unroll
+  for (int q = 0; q < PER; ++q) {
+    const int e = q * SAMP_THREADS + threadIdx.x;
+    mine[q] = (e % TK_CAP) < part_n[e / TK_CAP];
+    mine_v[q] = mine[q] ? cv[e] : 0.f;
+    mine_i[q] = mine[q] ? ci[e] : 0;
+  }
+#pragma unroll
+  for (int q = 0; q < PER; ++q)
+    if (mine[q]) {
+      const uint32_t bin = (kmax - order_key(mine_v[q])) >> 16;
       if (bin < 255u) atomicAdd(&hist[bin], 1);
     }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int cum = 0, b = 0;
-    for (; b < 255; ++b) {
-      cum += hist[b];
-      if (cum >= k) break;
-    }
-    bstar = b < 255 && cum <= SAMP_CAND ? b : -1;
+  if (threadIdx.x < WAVE) {
+    int cum, b;
+    first_bin_reaching(hist, k, &b, &cum);
+    if (threadIdx.x == 0) bstar = b < 255 && cum <= SAMP_CAND ? b : -1;
   }
   __syncthreads();
   if (bstar < 0) return;
-  for (int e = threadIdx.x; e < TK_CHUNKS * TK_CAP; e += SAMP_THREADS)
-    if ((e % TK_CAP) < part_n[e / TK_CAP]) {
-      const float x = cv[e];
-      if (((kmax - order_key(x)) >> 16) <= (uint32_t)bstar) {
-        const int slot = atomicAdd(&S.n, 1);
-        S.cv[slot] = x;
-        S.ci[slot] = ci[e];
-      }
+#pragma unroll
+  for (int q = 0; q < PER; ++q)
+    if (mine[q] && ((kmax - order_key(mine_v[q])) >> 16) <= (uint32_t)bstar) {
+      const int slot = atomicAdd(&S.n, 1);
+      S.cv[slot] = mine_v[q];
+      S.ci[slot] = mine_i[q];
     }
   __syncthreads();
   const int pick = sample_small(S, S.n, k, top, top_p[row], min_p[row], uniform[row]);
