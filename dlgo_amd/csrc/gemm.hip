@@ -179,10 +179,27 @@ template <int N> static __device__ __forceinline__ void wait_loads() {   // unti
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-template <typename T, int BN, int BT, int WN, int WT, int NS, int EPI>
+// What a tiled product may do for the RMSNorm that follows it, or take from the product before it (the hand-off that
+// gemm_rows.hip's streamed products have, for steps of many rows):
+//   NORM 1 (with the epilogue that adds into the float32 residual rows): beside the new residual rows it leaves them times
+//     the norm's weights in the run dtype, not yet scaled, and for every 32 columns their share of each row's sum of squares;
+//   NORM 2: its X are such unscaled rows; every block adds up the shares of its rows in order and multiplies its sums by
+//     1/sqrt(sum/width + eps) (a scalar per row, so it commutes with the product) before the epilogue.
+struct TileNorm {
+  const float* norm_w;     // NORM 1: the following norm's weights [N]
+  void* unscaled;          // NORM 1: [T, ld_unscaled] in the run dtype
+  int ld_unscaled;
+  float* parts;            // NORM 1: written, NORM 2: read; [T, n_parts]
+  int n_parts;
+  int width;               // NORM 2: the normed width
+  float eps;               // NORM 2
+};
+
+template <typename T, int BN, int BT, int WN, int WT, int NS, int EPI, int NORM = 0>
 __global__ __launch_bounds__(WN* WT* WAVE) void gemm_direct_kernel(const T* __restrict__ W, const T* __restrict__ X,
                                                                      void* __restrict__ Yv, int N, int Tn, int K, int ldw, int ldx,
-                                                                     int ldy, int tiles_t, int nk_split, long long split_stride) {
+                                                                     int ldy, int tiles_t, int nk_split, long long split_stride,
+                                                                     TileNorm tn) {
   constexpr int NW = WN * WT;
   constexpr int EPC = 16 / sizeof(T);
   constexpr int BK = 128 / sizeof(T);
@@ -252,6 +269,34 @@ __global__ __launch_bounds__(WN* WT* WAVE) void gemm_direct_kernel(const T* __re
   for (int s = 0; s < NS - 1; ++s)
     if (s < nk) issue(s, s);
 
+  // NORM 2: the factor of each of the block's rows, while the first tiles are on their way (the loop's barriers stand
+  // between this and the epilogue)
+  __shared__ float row_scale[NORM == 2 ? BT : 1];
+  if (NORM == 2) {
+    for (int r = tid; r < BT; r += NW * WAVE) {
+      const int t = t0 + r < Tn ? t0 + r : Tn - 1;
+      const float* p = tn.parts + (size_t)t * tn.n_parts;
+      float ss = 0.f;
+      int q = 0;
+      if ((tn.n_parts & 3) == 0 && ((uintptr_t)tn.parts & 15) == 0) {
+        // 32 shares at a time, all their loads on the way before the first is added
+        for (; q + 32 <= tn.n_parts; q += 32) {
+          float4 v[8];
+#pragma unroll
+          for (int u = 0; u < 8; ++u) v[u] = *(const float4*)(p + q + 4 * u);
+#pragma unroll
+          for (int u = 0; u < 8; ++u) ss += (v[u].x + v[u].y) + (v[u].z + v[u].w);
+        }
+        for (; q + 4 <= tn.n_parts; q += 4) {
+          const float4 v = *(const float4*)(p + q);
+          ss += (v.x + v.y) + (v.z + v.w);
+        }
+      }
+      for (; q < tn.n_parts; ++q) ss += p[q];
+      row_scale[r] = 1.0f / sqrtf(ss / (float)tn.width + tn.eps);
+    }
+  }
+
   // operands: row lane%32 of a 32-row tile, pieces 2*slab + lane/32, found at slot (lane/32 ^ x) ^ 2*slab
   const int s0 = (lane >> 5) ^ ((lane >> 1) & 7);
   const int rowA = (wn * (BN / WN) + (lane & 31)) * 128, rowB = BN * 128 + (wt * (BT / WT) + (lane & 31)) * 128;
@@ -310,7 +355,14 @@ __global__ __launch_bounds__(WN* WT* WAVE) void gemm_direct_kernel(const T* __re
           for (int q = 0; q < 4; ++q) {
             const int tl = wt * (BT / WT) + j * 32 + (lane & 31);
             const int nl = wn * (BN / WN) + i * 32 + 8 * q + 4 * (lane >> 5);     // four consecutive n of that token
-            const float v0 = acc[i][j][4 * q], v1 = acc[i][j][4 * q + 1], v2 = acc[i][j][4 * q + 2], v3 = acc[i][j][4 * q + 3];
+            float v0 = acc[i][j][4 * q], v1 = acc[i][j][4 * q + 1], v2 = acc[i][j][4 * q + 2], v3 = acc[i][j][4 * q + 3];
+            if (NORM == 2) {
+              const float sc = row_scale[tl];
+              v0 *= sc;
+              v1 *= sc;
+              v2 *= sc;
+              v3 *= sc;
+            }
             if (EPI == EPI_SWIGLU) {
               Elem<T>::store2((T*)(lds + tl * OROW + nl), silu_f<T>(v0) * v1, silu_f<T>(v2) * v3);
             } else {
@@ -342,24 +394,50 @@ __global__ __launch_bounds__(WN* WT* WAVE) void gemm_direct_kernel(const T* __re
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
         const int tt = p * 8 + (lane >> 3), nn = (lane & 7) * 4;
-        const float4 v = *(const float4*)(turn + tt * (GEMM_ROWB / 4) + nn);
+        float4 v = *(const float4*)(turn + tt * (GEMM_ROWB / 4) + nn);
         const int t = t0 + wt * (BT / WT) + j * 32 + tt;
         const int n = n0 + wn * (BN / WN) + i * 32 + nn;
-        if (t < Tn) epilogue4<T, EPI>(Y, ldy, N, t, n, v.x, v.y, v.z, v.w);
+        if (NORM == 2) {
+          const float sc = row_scale[wt * (BT / WT) + j * 32 + tt];
+          v.x *= sc;
+          v.y *= sc;
+          v.z *= sc;
+          v.w *= sc;
+        }
+        if (NORM == 1) {
+          // the eight lanes of a token hold the 32 columns of this tile: the new residual values, their products with
+          // the norm's weights, and the columns' share of the row's sum of squares (N is a multiple of 32 here)
+          float ssq = 0.f;
+          if (t < Tn && n < N) {
+            float* y = (float*)Y + (size_t)t * ldy + n;
+            const float4 old = *(const float4*)y;
+            const float4 r = make_float4(old.x + v.x, old.y + v.y, old.z + v.z, old.w + v.w);
+            *(float4*)y = r;
+            const float4 w4 = *(const float4*)(tn.norm_w + n);
+            Elem<T>::store4((T*)tn.unscaled + (size_t)t * tn.ld_unscaled + n, r.x * w4.x, r.y * w4.y, r.z * w4.z, r.w * w4.w);
+            ssq = fmaf(r.x, r.x, fmaf(r.y, r.y, fmaf(r.z, r.z, r.w * r.w)));
+          }
+          ssq += __shfl_xor(ssq, 1, WAVE);
+          ssq += __shfl_xor(ssq, 2, WAVE);
+          ssq += __shfl_xor(ssq, 4, WAVE);
+          if ((lane & 7) == 0 && t < Tn && n < N) tn.parts[(size_t)t * tn.n_parts + (n >> 5)] = ssq;
+        } else if (t < Tn) {
+          epilogue4<T, EPI>(Y, ldy, N, t, n, v.x, v.y, v.z, v.w);
+        }
       }
       __builtin_amdgcn_wave_barrier();
     }
   }
 }
 
-template <typename T, int BN, int BT, int WN, int WT, int NS, int EPI>
+template <typename T, int BN, int BT, int WN, int WT, int NS, int EPI, int NORM = 0>
 static const char* launch_direct(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy,
-                                 hipStream_t stream, int splits = 1, long long split_stride = 0) {
+                                 hipStream_t stream, int splits = 1, long long split_stride = 0, TileNorm tn = TileNorm{}) {
   const int tiles_t = (Tn + BT - 1) / BT, tiles_n = (N + BN - 1) / BN;
   const int nk_all = K / (int)(128 / sizeof(T)), nk_split = (nk_all + splits - 1) / splits;
   constexpr int smem = NS * (BN + BT) * 128;
   static_assert(smem >= WN * WT * 32 * GEMM_ROWB, "the stages must hold the waves' turning space");
-  auto kernel = gemm_direct_kernel<T, BN, BT, WN, WT, NS, EPI>;
+  auto kernel = gemm_direct_kernel<T, BN, BT, WN, WT, NS, EPI, NORM>;
   static bool raised = false;
   if (smem > 64 * 1024 && !raised) {
     hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -367,7 +445,7 @@ static const char* launch_direct(const void* W, const void* X, void* Y, int N, i
     raised = true;
   }
   hipLaunchKernelGGL(kernel, dim3((unsigned)(tiles_t * tiles_n), (unsigned)((nk_all + nk_split - 1) / nk_split)), dim3(WN * WT * WAVE),
-                     smem, stream, (const T*)W, (const T*)X, Y, N, Tn, K, ldw, ldx, ldy, tiles_t, nk_split, split_stride);
+                     smem, stream, (const T*)W, (const T*)X, Y, N, Tn, K, ldw, ldx, ldy, tiles_t, nk_split, split_stride, tn);
   return nullptr;
 }
 
@@ -537,6 +615,30 @@ static int auto_splits(int N, int Tn, int nk_all, long long part_elems) {
   return splits;
 }
 
+// Which of the kernels that load straight into LDS a product gets when the choice is the library's (20 = 256x256, 21 =
+// 128x128 with two blocks a unit, 22 = 128x128 deeper, 23 = 64x64).  Few rows of X: the weights stream through small
+// tiles, and so does any product of at most two small tiles a compute unit.  Else the large tile when it fills the
+// chip; else two blocks of 128x128 on a unit when there are that many; else one, deeper.  (Measured on the shapes of a
+// 1B Llama.)
+static int direct_kind(int N, int Tn) {
+  const long b256 = (long)((N + 255) / 256) * ((Tn + 255) / 256);
+  const long big = (long)((N + 127) / 128) * ((Tn + 127) / 128);
+  const long small = (long)((N + 63) / 64) * ((Tn + 63) / 64);
+  if (Tn <= 64) return 23;
+  if (Tn <= 128) return N >= 32768 ? 21 : 23;
+  if (small <= 512) return 23;
+  return b256 >= 192 ? 20 : (big > 256 ? 21 : 22);
+}
+
+template <typename T, int EPI, int NORM>
+static const char* launch_direct_norm(int kind, const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy,
+                                      hipStream_t stream, const TileNorm& tn) {
+  if (kind == 20) return launch_direct<T, 256, 256, 4, 4, 2, EPI, NORM>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream, 1, 0, tn);
+  if (kind == 21) return launch_direct<T, 128, 128, 2, 4, 2, EPI, NORM>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream, 1, 0, tn);
+  if (kind == 22) return launch_direct<T, 128, 128, 4, 4, 3, EPI, NORM>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream, 1, 0, tn);
+  return launch_direct<T, 64, 64, 2, 2, 4, EPI, NORM>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream, 1, 0, tn);
+}
+
 template <typename T, int EPI>
 static const char* dispatch(const void* W, const void* X, void* Y, int N, int Tn, int K, int ldw, int ldx, int ldy, int force,
                             int splits, float* part, long long part_elems, hipStream_t stream) {
@@ -556,18 +658,7 @@ static const char* dispatch(const void* W, const void* X, void* Y, int N, int Tn
     DLGO_REQUIRE(splits <= nk_all, "gemm: %d runs of k, but only %d tiles", splits, nk_all);
     return launch_split<T, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, splits, part, stream);
   }
-  if (kind == 0 && direct) {
-    const long b256 = (long)((N + 255) / 256) * ((Tn + 255) / 256);
-    const long big = (long)((N + 127) / 128) * ((Tn + 127) / 128);
-    const long small = (long)((N + 63) / 64) * ((Tn + 63) / 64);
-    // Few rows of X: the weights stream through small tiles, and so does any product of at most two small tiles a compute
-    // unit.  Else the large tile when it fills the chip; else two blocks of 128x128 on a unit when there are that many;
-    // else one, deeper.  (Measured on the shapes of a 1B Llama.)
-    if (Tn <= 64) kind = 23;
-    else if (Tn <= 128) kind = N >= 32768 ? 21 : 23;
-    else if (small <= 512) kind = 23;
-    else if (big >= 128) kind = b256 >= 192 ? 20 : (big > 256 ? 21 : 22);
-  }
+  if (kind == 0 && direct) kind = direct_kind(N, Tn);
   if (kind == 23) return launch_direct<T, 64, 64, 2, 2, 4, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 20) return launch_direct<T, 256, 256, 4, 4, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
   if (kind == 21) return launch_direct<T, 128, 128, 2, 4, 2, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
@@ -685,6 +776,68 @@ extern "C" const char* dlgo_gemm_accum_norm(const void* W, const void* X, float*
   else SUM_NORM(8);
 #undef SUM_NORM
   DLGO_LAUNCH_CHECK("gemm_accum_norm");
+  return nullptr;
+}
+
+// Whether the two entry points below take a product: the tiles that load straight into LDS, every block summing the
+// whole of k (with part_elems floats of scratch at hand dlgo_gemm might share k out instead: then not).  role 1: the
+// product that leaves the norm (N a multiple of 32, up to 8192); role 2: the one that applies it.
+extern "C" int dlgo_gemm_tile_norm_takes(int dtype, int N, int Tn, int K, int ldw, int ldx, int role, long long part_elems) {
+  const size_t elem = dtype == DLGO_DTYPE_F32 ? 4 : 2;
+  if (dtype != DLGO_ELEM || N <= 0 || Tn <= 0 || K <= 0 || !direct_takes(K, ldw, ldx, elem)) return 0;
+  if (auto_splits(N, Tn, K / (int)(128 / elem), part_elems) != 1) return 0;
+  if (role == 1) return N % 32 == 0 && N <= 8192 ? 1 : 0;
+  return role == 2 ? 1 : 0;
+}
+
+// residual [T, N] (float32) += X W^T, and for the RMSNorm that follows: unscaled [T, N] (run dtype) = new residual * norm_w,
+// parts [T, N / 32] = each 32 columns' share of every row's sum of squares (*n_parts = N / 32).  The consumer is
+// dlgo_gemm_tile_scaled (or gemm_rows.hip's dlgo_gemm_rows_scaled) with these parts.
+extern "C" const char* dlgo_gemm_tile_leave(const void* W, const void* X, float* residual, int dtype, int N, int Tn, int K, int ldw,
+                                            int ldx, int ldy, const float* norm_w, void* unscaled, int ld_unscaled, float* parts,
+                                            long long parts_elems, int* n_parts, hipStream_t stream) {
+  DLGO_REQUIRE(dtype == DLGO_ELEM, "gemm: this library is built for dtype code %d, got %d", DLGO_ELEM, dtype);
+  DLGO_REQUIRE(N > 0 && Tn >= 0 && K > 0 && ldw >= K && ldx >= K && ldy >= N && ld_unscaled >= N, "gemm_tile_leave: bad sizes");
+  DLGO_REQUIRE(direct_takes(K, ldw, ldx, sizeof(elem_t)), "gemm_tile_leave: K must be a whole number of 128-byte pieces, got %d", K);
+  const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
+  DLGO_REQUIRE(ldw % epc == 0 && ldx % epc == 0 && ((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0,
+               "gemm_tile_leave: W and X must be 16-byte aligned with row strides that keep them so");
+  DLGO_REQUIRE(N % 32 == 0 && N <= 8192 && ldy % 4 == 0 && ld_unscaled % 4 == 0, "gemm_tile_leave: N a multiple of 32 up to 8192, got %d", N);
+  DLGO_REQUIRE(residual && norm_w && unscaled && parts && n_parts && ((uintptr_t)residual & 15) == 0 && ((uintptr_t)norm_w & 15) == 0 &&
+                   ((uintptr_t)unscaled & 7) == 0 && parts_elems >= (long long)Tn * (N / 32),
+               "gemm_tile_leave: missing or misaligned operand, or scratch too small");
+  *n_parts = N / 32;
+  if (Tn == 0) return nullptr;
+  const TileNorm tn{norm_w, unscaled, ld_unscaled, parts, N / 32, 0, 0.f};
+  const char* err = launch_direct_norm<elem_t, EPI_ACCUM_F32, 1>(direct_kind(N, Tn), W, X, residual, N, Tn, K, ldw, ldx, ldy, stream, tn);
+  if (err) return err;
+  DLGO_LAUNCH_CHECK("gemm_tile_leave");
+  return nullptr;
+}
+
+// Y (epilogue)= scale[t] * (X W^T), X being rows left unscaled with the shares of their sums of squares in parts:
+// scale[t] = 1 / sqrt(sum of the row's parts / width + eps).  Epilogues: store and SwiGLU.
+extern "C" const char* dlgo_gemm_tile_scaled(const void* W, const void* X, void* Y, int dtype, int N, int Tn, int K, int ldw, int ldx,
+                                             int ldy, int epilogue, const float* parts, int n_parts, int width, float eps,
+                                             hipStream_t stream) {
+  DLGO_REQUIRE(dtype == DLGO_ELEM, "gemm: this library is built for dtype code %d, got %d", DLGO_ELEM, dtype);
+  DLGO_REQUIRE(N > 0 && Tn >= 0 && K > 0 && ldw >= K && ldx >= K, "gemm_tile_scaled: bad sizes");
+  DLGO_REQUIRE(direct_takes(K, ldw, ldx, sizeof(elem_t)), "gemm_tile_scaled: K must be a whole number of 128-byte pieces, got %d", K);
+  const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
+  DLGO_REQUIRE(ldw % epc == 0 && ldx % epc == 0 && ((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0,
+               "gemm_tile_scaled: W and X must be 16-byte aligned with row strides that keep them so");
+  DLGO_REQUIRE(parts && n_parts > 0 && width > 0 && eps > 0.f, "gemm_tile_scaled: parts, their number, the width and eps");
+  DLGO_REQUIRE(epilogue == EPI_STORE || epilogue == EPI_SWIGLU, "gemm_tile_scaled: epilogues store and SwiGLU, got %d", epilogue);
+  DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm: SwiGLU epilogue needs an even N and ldy >= N/2");
+  DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm: ldy %d shorter than N %d", ldy, N);
+  if (Tn == 0) return nullptr;
+  const TileNorm tn{nullptr, nullptr, 0, const_cast<float*>(parts), n_parts, width, eps};
+  const int kind = direct_kind(N, Tn);
+  const char* err = epilogue == EPI_STORE
+                        ? launch_direct_norm<elem_t, EPI_STORE, 2>(kind, W, X, Y, N, Tn, K, ldw, ldx, ldy, stream, tn)
+                        : launch_direct_norm<elem_t, EPI_SWIGLU, 2>(kind, W, X, Y, N, Tn, K, ldw, ldx, ldy, stream, tn);
+  if (err) return err;
+  DLGO_LAUNCH_CHECK("gemm_tile_scaled");
   return nullptr;
 }
 

@@ -79,7 +79,7 @@ def _lib(module: str, defines=()):
     lib = _libs.get(key)
     if lib is None:
         lib = build.load(module, defines)
-        for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_accum_norm", "dlgo_gemm_parts", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_gemm_rows_leave_parts", "dlgo_gemm_rows_scaled", "dlgo_attention_rows",
+        for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_accum_norm", "dlgo_gemm_parts", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_gemm_rows_leave_parts", "dlgo_gemm_rows_scaled", "dlgo_gemm_tile_leave", "dlgo_gemm_tile_scaled", "dlgo_attention_rows",
                      "dlgo_attention_prefill", "dlgo_attention_prefill_f32", "dlgo_attention_decode", "dlgo_attention_decode_f32", "dlgo_argmax", "dlgo_sample", "dlgo_bias_add", "dlgo_head_rmsnorm"):
             if hasattr(lib, name):
                 getattr(lib, name).restype = ctypes.c_char_p
@@ -307,8 +307,8 @@ class UnscaledNorm:
 
 
 def streams_few_rows(weight: torch.Tensor, rows: int, scaled: bool = False) -> bool:
-    """Whether gemm_accum_leave_norm (scaled: gemm_scaled) takes this weight with this many rows of x: up to 16 rows and
-    weight rows of whole KB (for gemm_scaled: 2, 3, 4, 6 or 8 of them)."""
+    """Whether the streamed products take this weight with this many rows of x: up to 16 rows and weight rows of whole
+    KB."""
     if weight.dim() != 2 or weight.stride(1) != 1 or not (1 <= rows <= 16):
         return False
     lib = _lib("gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),))
@@ -316,11 +316,32 @@ def streams_few_rows(weight: torch.Tensor, rows: int, scaled: bool = False) -> b
     return bool(lib.dlgo_gemm_rows_streams(dtype_code(weight.dtype), rows, weight.shape[1], weight.stride(0), int(scaled)))
 
 
+def _tiles_take_norm(weight: torch.Tensor, rows: int, role: int) -> bool:
+    """Whether the tiled products leave (role 1) or apply (role 2) a norm for this weight and this many rows: steps of
+    many rows whose product gemm() would give to tiles that sum the whole of k."""
+    if weight.dim() != 2 or weight.stride(1) != 1 or rows <= 16:
+        return False
+    lib = _lib("gemm", (("DLGO_ELEM", dtype_code(weight.dtype)),))
+    lib.dlgo_gemm_tile_norm_takes.restype = ctypes.c_int
+    return bool(lib.dlgo_gemm_tile_norm_takes(dtype_code(weight.dtype), weight.shape[0], rows, weight.shape[1], weight.stride(0),
+                                              weight.shape[1], role, ctypes.c_longlong(GEMM_SPLIT_FLOATS)))
+
+
+def can_leave_unscaled(weight: torch.Tensor, rows: int) -> bool:
+    """Whether gemm_accum_leave_norm takes this weight with this many rows of x (contiguous rows of x assumed)."""
+    return streams_few_rows(weight, rows) or _tiles_take_norm(weight, rows, 1)
+
+
+def can_take_unscaled(weight: torch.Tensor, rows: int) -> bool:
+    """Whether gemm_scaled takes this weight with this many rows (contiguous rows assumed)."""
+    return streams_few_rows(weight, rows, scaled=True) or _tiles_take_norm(weight, rows, 2)
+
+
 def gemm_accum_leave_norm(weight: torch.Tensor, x: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor, eps: float,
                           unscaled: torch.Tensor, parts: torch.Tensor) -> UnscaledNorm:
     """residual += x @ weight.T, and of rmsnorm(residual) * norm_weight of the new rows what UnscaledNorm describes
     (unscaled: [T, N] in the run dtype; parts: float32 scratch of at least T * ceil(N / 16) elements).  For weights
-    and rows that streams_few_rows accepts."""
+    and rows that can_leave_unscaled accepts: few rows go to the streamed product, many to tiles."""
     _need(weight, "gemm weight", dims=2)
     _need(x, "gemm input", weight.dtype, 2)
     _need(residual, "residual rows", torch.float32, 2)
@@ -333,17 +354,20 @@ def gemm_accum_leave_norm(weight: torch.Tensor, x: torch.Tensor, residual: torch
         raise KernelError(f"gemm_accum_leave_norm: x {tuple(x.shape)}, residual {tuple(residual.shape)}, unscaled {tuple(unscaled.shape)} "
                           f"and norm weight {tuple(norm_weight.shape)} do not fit weight {tuple(weight.shape)}")
     n_parts = ctypes.c_int(0)
-    lib = _lib("gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),))
-    _check(lib.dlgo_gemm_rows_leave_parts(_ptr(weight), _ptr(x), _ptr(residual), dtype_code(weight.dtype), n, t, k,
-                                          _rows(weight, "gemm weight"), _rows(x, "gemm input"), _rows(residual, "residual rows"),
-                                          _ptr(norm_weight), _ptr(unscaled), _rows(unscaled, "unscaled rows"), _ptr(parts),
-                                          ctypes.c_longlong(parts.numel()), ctypes.byref(n_parts), _stream()))
+    tiled = t > 16
+    lib = _lib("gemm" if tiled else "gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),))
+    fn = lib.dlgo_gemm_tile_leave if tiled else lib.dlgo_gemm_rows_leave_parts
+    _check(fn(_ptr(weight), _ptr(x), _ptr(residual), dtype_code(weight.dtype), n, t, k,
+              _rows(weight, "gemm weight"), _rows(x, "gemm input"), _rows(residual, "residual rows"),
+              _ptr(norm_weight), _ptr(unscaled), _rows(unscaled, "unscaled rows"), _ptr(parts),
+              ctypes.c_longlong(parts.numel()), ctypes.byref(n_parts), _stream()))
     return UnscaledNorm(unscaled, parts, n_parts.value, n, eps)
 
 
 def gemm_scaled(weight: torch.Tensor, left: UnscaledNorm, out: torch.Tensor, epilogue: int = EPI_STORE) -> torch.Tensor:
     """out (epilogue)= rmsnorm's factor of each row * (left.rows @ weight.T): the product of the normed rows that `left`
-    describes.  Epilogues as gemm(); for weights and rows that streams_few_rows accepts."""
+    describes.  Epilogues as gemm() for few rows, store and SwiGLU for many; for weights and rows that can_take_unscaled
+    accepts."""
     _need(weight, "gemm weight", dims=2)
     x = left.rows
     _need(x, "unscaled rows", weight.dtype, 2)
@@ -356,10 +380,12 @@ def gemm_scaled(weight: torch.Tensor, left: UnscaledNorm, out: torch.Tensor, epi
     cols = n // 2 if epilogue == EPI_SWIGLU else n
     if tuple(out.shape) != (t, cols):
         raise KernelError(f"gemm_scaled: output {tuple(out.shape)}, expected {(t, cols)}")
-    lib = _lib("gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),))
-    _check(lib.dlgo_gemm_rows_scaled(_ptr(weight), _ptr(x), _ptr(out), dtype_code(weight.dtype), n, t, k, _rows(weight, "gemm weight"),
-                                     _rows(x, "unscaled rows"), _rows(out, "gemm output"), epilogue, _ptr(left.parts), left.n_parts,
-                                     left.width, ctypes.c_float(left.eps), _stream()))
+    tiled = t > 16
+    lib = _lib("gemm" if tiled else "gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),))
+    fn = lib.dlgo_gemm_tile_scaled if tiled else lib.dlgo_gemm_rows_scaled
+    _check(fn(_ptr(weight), _ptr(x), _ptr(out), dtype_code(weight.dtype), n, t, k, _rows(weight, "gemm weight"),
+              _rows(x, "unscaled rows"), _rows(out, "gemm output"), epilogue, _ptr(left.parts), left.n_parts,
+              left.width, ctypes.c_float(left.eps), _stream()))
     return out
 
 

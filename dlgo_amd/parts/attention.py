@@ -150,7 +150,7 @@ class Attention(Mixer):
         return isinstance(norm, RMSNorm) and ops.fused_norm_pays(self.w_qkv, ctx.n_tokens)
 
     def takes_unscaled(self, ctx) -> bool:
-        return ops.streams_few_rows(self.w_qkv, ctx.n_tokens, scaled=True)
+        return ops.can_take_unscaled(self.w_qkv, ctx.n_tokens)
 
     def forward(self, xn, ctx, unit, residual, owns_cache=True, norm=None, then=None):
         t = residual.shape[0]
@@ -193,11 +193,19 @@ class Attention(Mixer):
             ops.bias_add(residual, self.b_o)
             return False
         if then is not None and isinstance(then[0], RMSNorm):
-            if len(then) > 2 and then[2] is not None and then[2].takes_unscaled(ctx) and ops.streams_few_rows(self.w_o, t):
+            # the norm left unscaled by a streamed product (few rows); else written whole by the sum of a product whose k
+            # was shared out; else left unscaled by a tiled product (many rows); else not at all
+            unscaled_ok = len(then) > 2 and then[2] is not None and then[2].takes_unscaled(ctx)
+
+            def leave():
                 shares = ctx.scratch("attention.norm_shares", t * ((self.width + 15) // 16), torch.float32)
                 return ops.gemm_accum_leave_norm(self.w_o, out, residual, then[0].weight, then[0].eps, then[1], shares)
+            if unscaled_ok and ops.streams_few_rows(self.w_o, t):
+                return leave()
             if ops.gemm_accum_then_norm(self.w_o, out, residual, split, then[0].weight, then[0].eps, then[1]):
                 return True
+            if unscaled_ok and ops.can_leave_unscaled(self.w_o, t):
+                return leave()
         ops.gemm(self.w_o, out, residual, ops.EPI_ACCUM_F32, scratch=split)
         return False
 

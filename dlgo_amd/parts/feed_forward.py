@@ -60,7 +60,7 @@ class GatedFeedForward(FeedForward):
         return isinstance(norm, RMSNorm) and ops.fused_norm_pays(self.w_gate_up, ctx.n_tokens)
 
     def takes_unscaled(self, ctx) -> bool:
-        return ops.streams_few_rows(self.w_gate_up, ctx.n_tokens, scaled=True)
+        return ops.can_take_unscaled(self.w_gate_up, ctx.n_tokens)
 
     def forward(self, xn, ctx, residual, norm=None, then=None):
         hid = ctx.buffer("feed_forward.hidden", (residual.shape[0], self.inner), ctx.dtype)
@@ -71,8 +71,15 @@ class GatedFeedForward(FeedForward):
         else:
             ops.gemm(self.w_gate_up, xn, hid, ops.EPI_SWIGLU)
         split = ctx.scratch("gemm.split", ops.GEMM_SPLIT_FLOATS, torch.float32)
-        if then is not None and isinstance(then[0], RMSNorm) and ops.gemm_accum_then_norm(
-                self.w_down, hid, residual, split, then[0].weight, then[0].eps, then[1]):
-            return True
+        if then is not None and isinstance(then[0], RMSNorm):
+            if ops.gemm_accum_then_norm(self.w_down, hid, residual, split, then[0].weight, then[0].eps, then[1]):
+                return True
+            # many rows: the tiled product leaves the norm unscaled, if what reads it can apply the factor (with few rows
+            # the split product and its sum above are as fast as the streamed product that would leave it)
+            t = residual.shape[0]
+            if t > 16 and len(then) > 2 and then[2] is not None and then[2].takes_unscaled(ctx) \
+                    and ops.can_leave_unscaled(self.w_down, t):
+                shares = ctx.scratch("feed_forward.norm_shares", t * ((self.width + 15) // 16), torch.float32)
+                return ops.gemm_accum_leave_norm(self.w_down, hid, residual, then[0].weight, then[0].eps, then[1], shares)
         ops.gemm(self.w_down, hid, residual, ops.EPI_ACCUM_F32, scratch=split)
         return False

@@ -359,6 +359,51 @@ def test_norm_left_in_parts_and_applied_by_the_next_product(dtype, _, rel, n1, k
                         torch.empty(t, n2, dtype=dtype, device=DEV))
 
 
+@pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("n1,k1,n2,t", [(256, 128, 136, 17), (2048, 512, 384, 300), (1024, 2048, 1030, 130), (96, 64, 64, 64),
+                                        (4096, 256, 264, 257), (512, 8192, 128, 520)])
+def test_norm_left_and_applied_by_tiled_products(dtype, _, rel, n1, k1, n2, t):
+    """The same hand-off for steps of many rows: the tiled product that adds into the residual leaves the rows times
+    the norm's weights and a share of the sums of squares for every 32 columns; the next tiled product multiplies its
+    sums by each row's factor.  residual += x W1^T; out = rmsnorm(residual) W2^T, plain and through SwiGLU."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(n1 + t)
+    w1 = (0.3 * torch.randn(n1, k1, generator=g)).to(dtype).to(DEV)
+    w2 = (0.5 * torch.randn(n2, n1, generator=g)).to(dtype).to(DEV)
+    x = torch.randn(t, k1, generator=g).to(dtype).to(DEV)
+    res = (3 * torch.randn(t, n1, generator=g)).to(DEV)
+    nw = (1 + 0.3 * torch.randn(n1, generator=g)).to(DEV)
+    eps = 1e-2
+    if not (ops.can_leave_unscaled(w1, t) and ops.can_take_unscaled(w2, t)):
+        pytest.skip("a product of this shape has its k shared out: its ordered sum writes the norm itself")
+    assert not ops.can_leave_unscaled(w1[:n1 - 8], t) and not ops.can_take_unscaled(w2[:, :n1 - 8], t)
+    new_res = res.double() + x.double() @ w1.double().T
+    xn = new_res / torch.sqrt((new_res * new_res).mean(-1, keepdim=True) + eps) * nw.double()
+    want = xn @ w2.double().T
+    tol = 1e-5 if dtype == torch.float32 else 1.5e-2
+    unscaled = torch.empty(t, n1, dtype=dtype, device=DEV)
+    parts = torch.full((t * ((n1 + 15) // 16) + 7,), float("nan"), device=DEV)
+    left = ops.gemm_accum_leave_norm(w1, x, res, nw, eps, unscaled, parts)
+    close(res, new_res, 1e-5, "residual")
+    assert left.n_parts == n1 // 32 and left.width == n1
+    close(left.parts[:t * left.n_parts].view(t, -1).sum(-1), (new_res * new_res).sum(-1), 1e-5, "sum of squares")
+    close(unscaled, new_res * nw.double(), 1e-5 if dtype == torch.float32 else 8e-3, "unscaled rows")
+    out = torch.empty(t, n2, dtype=dtype, device=DEV)
+    ops.gemm_scaled(w2, left, out)
+    close(out, want, tol, "store")
+    hid = torch.empty(t, n2 // 2, dtype=dtype, device=DEV)
+    ops.gemm_scaled(w2, left, hid, ops.EPI_SWIGLU)
+    gd, ud = want[:, 0::2], want[:, 1::2]
+    close(hid, gd / (1 + torch.exp(-gd)) * ud, tol * 2, "swiglu")
+    # into a part of wider rows, from a part of the weight's rows (as the attention's QKV product does)
+    wide = torch.full((t, n2 + 16), 7.0, dtype=dtype, device=DEV)
+    ops.gemm_scaled(w2[:n2 - 8], left, wide[:, :n2 - 8])
+    close(wide[:, :n2 - 8], want[:, :n2 - 8], tol, "store into a part of the rows")
+    assert (wide[:, n2 - 8:] == 7.0).all()
+    with pytest.raises(ops.KernelError):
+        ops.gemm_scaled(w2, left, torch.empty(t, n2, device=DEV), ops.EPI_STORE_F32)
+
+
 def test_gemm_reference_vectors():
     """blas/blas_test.go:21-64: identity, [[1,2],[3,4]]·[1,1] = [3,7], batch layout out[p*rows + r]."""
     ops = _ops()
