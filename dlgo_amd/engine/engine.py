@@ -81,7 +81,7 @@ class _PromptGraph:
 class Engine:
     def __init__(self, model, dtype="bfloat16", device="cuda:0", max_tokens: int = 8192, max_ctx: Optional[int] = None,
                  max_slots: Optional[int] = None, max_step_tokens: int = 8192, logits_rows: int = 1024,
-                 use_graphs: bool = True, graph_max_batch: int = 128, prompt_graph_max_tokens: int = 1024,
+                 use_graphs: bool = True, graph_max_batch: int = 128, prompt_graph_max_tokens: int = 4096,
                  prompt_graph_limit: int = 32):
         """`model` holds its weights already (see from_folder / from_random).  use_graphs: steps of single tokens are
         recorded per batch size, and steps of fresh prompts of up to prompt_graph_max_tokens rows per shape (the
@@ -272,8 +272,9 @@ class Engine:
         # Fresh prompts of a shape seen before: the launches depend on the rows per sequence and the wanted places only,
         # so the step is recorded the second time the shape comes and replayed from then on.
         shape = None
+        # (a recording keeps its logits: not where those would be more than 64 MB)
         if (self.use_graphs and sink is None and n_out and total <= min(self.max_step_tokens, self.prompt_graph_max_tokens)
-                and not any(starts)):
+                and n_out * self.vocab * 4 <= (64 << 20) and not any(starts)):
             shape = (tuple(q_lens), tuple(wanted))
         out = None
         if sink is None and (shape is None or shape not in self._prompt_graphs):
