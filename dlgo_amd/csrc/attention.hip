@@ -60,6 +60,18 @@ template <> struct Vec16<bf16_t> {
   }
 };
 
+// The blocks a decode step gives the pages of a (sequence, kv head): the grid has `most`.  A sequence uses them all, or,
+// where the grid is sized for the longest sequence the launch allows (chunk > 0), as many as give each block about
+// `chunk` pages, at least `least`.  The blocks used share the sequence's pages evenly; the others return at once.
+struct SplitPlan {
+  int most, least, chunk;
+};
+__device__ __forceinline__ int splits_used(const SplitPlan& sp, int n_pages) {
+  if (sp.chunk <= 0) return sp.most;
+  const int by_pages = (n_pages + sp.chunk / 2) / sp.chunk;
+  return by_pages < sp.least ? sp.least : (by_pages > sp.most ? sp.most : by_pages);
+}
+
 template <typename T>
 __global__ __launch_bounds__(WAVE) void attn_rows_kernel(const T* __restrict__ q, int ldq, T* __restrict__ out, int ldo,
                                                          const int32_t* __restrict__ positions,
@@ -619,20 +631,23 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, float* __restrict__ part,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, const int32_t* __restrict__ page_table,
     int max_pages, bf16_t* __restrict__ cache, long long page_stride, long long v_off, int n_heads, int group,
-    int head_blocks, int n_splits, int window, float scale_log2e, const float* __restrict__ cos_t,
+    int head_blocks, SplitPlan sp, int window, float scale_log2e, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int rot, int interleaved, int new_kv, int k_col, int v_col) {
   constexpr int HD = HEAD_DIM;
   constexpr int KS = (HD + 31) / 32;   // k steps of K Q^T (16x16x32)
   constexpr int DT = HD / 16;          // 16-row tiles of the output's head dimension
   constexpr int LS = HD + 2;           // floats a wave leaves in LDS per head: values, max, sum
   extern __shared__ float lds[];
-  const int split = blockIdx.x, seq = blockIdx.z;
-  const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
+  // the split is the slowest index: the blocks of a short sequence that have pages are then neighbours in launch order,
+  // which is dealt round to the XCDs, and not every fourth or eighth block on the same few of them
+  const int split = blockIdx.z, seq = blockIdx.y;
+  const int kvh = blockIdx.x / head_blocks, hb = blockIdx.x % head_blocks;
   const int pos = positions[seq];
   const int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
   // the pages that hold keys of this token are dealt evenly to the splits
   const int first_pg = lo / PAGE, last_pg = pos / PAGE;
-  const int span = (last_pg - first_pg + n_splits) / n_splits;
+  const int n_splits = sp.most, used = splits_used(sp, last_pg - first_pg + 1);
+  const int span = (last_pg - first_pg + used) / used;
   const int pg0 = first_pg + split * span;
   const int pg1 = pg0 + span - 1 < last_pg ? pg0 + span - 1 : last_pg;
   if (pg0 > pg1) return;               // the whole block: fewer pages than splits
@@ -927,7 +942,7 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_lds_kernel(
     const bf16_t* __restrict__ q, int ldq, bf16_t* __restrict__ out, int ldo, float* __restrict__ part,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, const int32_t* __restrict__ page_table,
     int max_pages, bf16_t* __restrict__ cache, long long page_stride, long long v_off, int n_heads, int group,
-    int head_blocks, int n_splits, int window, float scale_log2e, const float* __restrict__ cos_t,
+    int head_blocks, SplitPlan sp, int window, float scale_log2e, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, int rot, int interleaved, int new_kv, int k_col, int v_col) {
   constexpr int HD = HEAD_DIM;
   constexpr int KS = (HD + 31) / 32;   // k steps of K Q^T (16x16x32)
@@ -939,12 +954,13 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_lds_kernel(
   using KSw = SlotSwizzle<KSLOTS>;
   using VSw = SlotSwizzle<8>;
   extern __shared__ __attribute__((aligned(16))) float lds[];
-  const int split = blockIdx.x, seq = blockIdx.z;
-  const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
+  const int split = blockIdx.z, seq = blockIdx.y;         // as attn_decode_kernel
+  const int kvh = blockIdx.x / head_blocks, hb = blockIdx.x % head_blocks;
   const int pos = positions[seq];
   const int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
   const int first_pg = lo / PAGE, last_pg = pos / PAGE;
-  const int span = (last_pg - first_pg + n_splits) / n_splits;
+  const int n_splits = sp.most, used = splits_used(sp, last_pg - first_pg + 1);
+  const int span = (last_pg - first_pg + used) / used;
   const int pg0 = first_pg + split * span;
   const int pg1 = pg0 + span - 1 < last_pg ? pg0 + span - 1 : last_pg;
   if (pg0 > pg1) return;               // the whole block: fewer pages than splits
@@ -1199,19 +1215,20 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_f32_kernel(
     const float* __restrict__ q, int ldq, float* __restrict__ out, int ldo, float* __restrict__ part,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, const int32_t* __restrict__ page_table,
     int max_pages, const float* __restrict__ cache, long long page_stride, long long v_off, int n_heads, int group,
-    int head_blocks, int n_splits, int window, float scale) {
+    int head_blocks, SplitPlan sp, int window, float scale) {
   constexpr int HD = HEAD_DIM;
   constexpr int KC = HD / 16;          // 16-element chunks of the head
   constexpr int DT = HD / 16;          // 16-row tiles of the output's head dimension
   constexpr int KT = HD <= 64 ? 4 : 2; // 16-key tiles held at once
   constexpr int LS = HD + 2;           // floats a wave leaves in LDS per head: values, max, sum
   extern __shared__ float lds[];
-  const int split = blockIdx.x, seq = blockIdx.z;
-  const int kvh = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
+  const int split = blockIdx.z, seq = blockIdx.y;         // as attn_decode_kernel
+  const int kvh = blockIdx.x / head_blocks, hb = blockIdx.x % head_blocks;
   const int pos = positions[seq];
   const int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
   const int first_pg = lo / PAGE, last_pg = pos / PAGE;
-  const int span = (last_pg - first_pg + n_splits) / n_splits;
+  const int n_splits = sp.most, used = splits_used(sp, last_pg - first_pg + 1);
+  const int span = (last_pg - first_pg + used) / used;
   const int pg0 = first_pg + split * span;
   const int pg1 = pg0 + span - 1 < last_pg ? pg0 + span - 1 : last_pg;
   if (pg0 > pg1) return;               // the whole block: fewer pages than splits
@@ -1372,11 +1389,11 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_f32_kernel(
 template <typename TO, bool NATURAL>
 __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restrict__ part, TO* __restrict__ out, int ldo,
                                                             const int32_t* __restrict__ positions, int n_heads,
-                                                            int n_splits, int window) {
+                                                            SplitPlan sp, int window) {
   constexpr int HD = HEAD_DIM;
   constexpr int PS = HD + 4;
   constexpr int ND = (HD + WAVE - 1) / WAVE;           // elements of the head per lane
-  const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const int seq = blockIdx.x, head = blockIdx.y, lane = threadIdx.x, n_splits = sp.most;
   const float* base = part + (size_t)(seq * n_heads + head) * n_splits * PS;
   const int pos = positions[seq];
   float M = -INFINITY, L = 0.f, acc[ND];
@@ -1396,7 +1413,8 @@ __global__ __launch_bounds__(WAVE) void attn_combine_kernel(const float* __restr
     if (c0 == 0) {
       const int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
       const int n_pages = pos / PAGE - lo / PAGE + 1;
-      const int span = (n_pages - 1 + n_splits) / n_splits;
+      const int used = splits_used(sp, n_pages);
+      const int span = (n_pages - 1 + used) / used;
       s1 = (n_pages - 1) / span;                     // the last split that was given pages
     }
     float M_new = M;
@@ -1459,10 +1477,10 @@ extern "C" const char* dlgo_attention_rows(const void* q, int ldq, void* out, in
   if (n_splits > 1) {     // the rows are the "sequences" of the combine: one position each
     if (dtype == DLGO_DTYPE_F32)
       hipLaunchKernelGGL((attn_combine_kernel<float, true>), dim3(n_tokens, n_heads), dim3(WAVE), 0, stream, part, (float*)out, ldo,
-                         positions, n_heads, n_splits, window);
+                         positions, n_heads, SplitPlan{n_splits, n_splits, 0}, window);
     else
       hipLaunchKernelGGL((attn_combine_kernel<bf16_t, true>), dim3(n_tokens, n_heads), dim3(WAVE), 0, stream, part, (bf16_t*)out, ldo,
-                         positions, n_heads, n_splits, window);
+                         positions, n_heads, SplitPlan{n_splits, n_splits, 0}, window);
     DLGO_LAUNCH_CHECK("attention_combine");
   }
   return nullptr;
@@ -1528,7 +1546,7 @@ extern "C" const char* dlgo_attention_prefill_f32(const void* q, int ldq, void* 
 // max_pages_used bounds the pages of any sequence of the step (a recorded
 // launch passes the context's bound).  part: float32 scratch, used when the pages are split over several
 // blocks: n_seq * n_heads * n_splits * (hd + 4) with n_splits = dlgo_attention_decode_splits(...).
-static void decode_plan(int n_pairs, int group, int max_pages_used, bool fused, bool through_lds, int* nwv, int* n_splits) {
+static void decode_plan(int n_pairs, int group, int max_pages_used, bool fused, bool through_lds, int* nwv, SplitPlan* plan) {
   const int heads_here = group < 16 ? group : 16;
   const int per_wave = heads_here * (HEAD_DIM + 2) * 4;      // bytes of LDS a wave needs for the merge
   // the registers a wave needs grow with the head size (a page's keys and values are held at once), and a block
@@ -1541,7 +1559,13 @@ static void decode_plan(int n_pairs, int group, int max_pages_used, bool fused, 
   // enough blocks to fill the chip: with few (sequence, kv head) pairs each pair's pages go to several blocks
   int splits = n_pairs >= 256 ? 1 : (256 + n_pairs - 1) / n_pairs;
   if (splits > max_pages_used) splits = max_pages_used;
-  if (max_pages_used > w * 8 && splits < (max_pages_used + w * 8 - 1) / (w * 8)) splits = (max_pages_used + w * 8 - 1) / (w * 8);
+  const int to_fill = splits;
+  // and enough that a block has at most sixteen pages a wave, so that one long sequence among short ones is not the
+  // step's tail.  These are blocks for the longest sequence the launch allows, which for a recorded step is the longest
+  // the cache allows: a shorter sequence uses fewer of them (splits_used)
+  const int long_pages = w * 16;
+  if (max_pages_used > long_pages && splits < (max_pages_used + long_pages - 1) / long_pages)
+    splits = (max_pages_used + long_pages - 1) / long_pages;
   if (splits > 1 && w > 8 && !through_lds) w = 8;
   if (through_lds && splits > 1) {
     // more waves than a sequence can have pages: a wave without a page only adds to the merge.  Halve the waves of a
@@ -1550,15 +1574,18 @@ static void decode_plan(int n_pairs, int group, int max_pages_used, bool fused, 
     if (splits * w > max_pages_used) splits = (max_pages_used + w - 1) / w;
   }
   *nwv = w;
-  *n_splits = splits;
+  plan->most = splits;
+  plan->least = to_fill < splits ? to_fill : splits;
+  plan->chunk = splits > to_fill ? w * 16 : 0;
 }
 
 // variant: 0 or 2 = the pages go through LDS, 1 = they are read straight into the operands' registers
 extern "C" int dlgo_attention_decode_splits(int n_seq, int n_heads, int n_kv, int max_pages_used, int fused, int variant) {
-  int nwv, n_splits;
+  int nwv;
+  SplitPlan plan;
   const int group = n_heads / n_kv;
-  decode_plan(n_seq * n_kv * ((group + 15) / 16), group, max_pages_used, fused != 0, variant != 1, &nwv, &n_splits);
-  return n_splits;
+  decode_plan(n_seq * n_kv * ((group + 15) / 16), group, max_pages_used, fused != 0, variant != 1, &nwv, &plan);
+  return plan.most;
 }
 
 extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, int ldo, float* part, long long part_elems,
@@ -1581,21 +1608,23 @@ extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, 
                "attention: operands must be 16-byte aligned");
   const int group = n_heads / n_kv;
   const int head_blocks = (group + 15) / 16;
-  int nwv, n_splits;
+  int nwv;
+  SplitPlan plan;
   const bool fused = cos_t != nullptr || new_kv;
   const bool through_lds = variant != 1;
-  decode_plan(n_seq * n_kv * head_blocks, group, max_pages_used, fused, through_lds, &nwv, &n_splits);
+  decode_plan(n_seq * n_kv * head_blocks, group, max_pages_used, fused, through_lds, &nwv, &plan);
+  const int n_splits = plan.most;
   DLGO_REQUIRE(n_splits == 1 || (part && part_elems >= (long long)n_seq * n_heads * n_splits * (HEAD_DIM + 4)),
                "attention: scratch for partial results too small");
-  DLGO_REQUIRE((long long)n_kv * head_blocks <= 65535 && n_seq <= 65535 && n_heads <= 65535, "attention: grid too large");
+  DLGO_REQUIRE((long long)n_kv * head_blocks <= 65535 && n_seq <= 65535 && n_heads <= 65535 && n_splits <= 65535, "attention: grid too large");
   if (n_seq == 0) return nullptr;
   const int heads_here = group < 16 ? group : 16;
   const size_t smem = (size_t)nwv * heads_here * (HEAD_DIM + 2) * 4;
-  dim3 grid(n_splits, n_kv * head_blocks, n_seq);
+  dim3 grid(n_kv * head_blocks, n_seq, n_splits);
 #define DECODE_GO(W_, F_)                                                                                                      \
   hipLaunchKernelGGL((attn_decode_kernel<W_, F_>), grid, dim3(W_ * WAVE), smem, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo,  \
                      part, positions, slots, page_table, max_pages, (bf16_t*)cache, page_stride, v_off, n_heads, group,        \
-                     head_blocks, n_splits, window, scale * LOG2E, cos_t, sin_t, rot, interleaved, new_kv,                    \
+                     head_blocks, plan, window, scale * LOG2E, cos_t, sin_t, rot, interleaved, new_kv,                    \
                      n_heads * head_dim, (n_heads + n_kv) * head_dim)
   if (through_lds) {
     const size_t pages = (size_t)nwv * 2 * PAGE * HEAD_DIM * 2;       // a page's keys and values of one kv head for every wave
@@ -1611,7 +1640,7 @@ extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, 
     }                                                                                                                          \
     hipLaunchKernelGGL(kernel, grid, dim3(W_* WAVE), lds_bytes, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo, part,        \
                        positions, slots, page_table, max_pages, (bf16_t*)cache, page_stride, v_off, n_heads, group,            \
-                       head_blocks, n_splits, window, scale* LOG2E, cos_t, sin_t, rot, interleaved, new_kv,                    \
+                       head_blocks, plan, window, scale* LOG2E, cos_t, sin_t, rot, interleaved, new_kv,                    \
                        n_heads* head_dim, (n_heads + n_kv) * head_dim);                                                        \
   } while (0)
     if (fused) {
@@ -1642,7 +1671,7 @@ extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, 
   DLGO_LAUNCH_CHECK("attention_decode");
   if (n_splits > 1) {
     hipLaunchKernelGGL((attn_combine_kernel<bf16_t, false>), dim3(n_seq, n_heads), dim3(WAVE), 0, stream, part, (bf16_t*)out, ldo,
-                       positions, n_heads, n_splits, window);
+                       positions, n_heads, plan, window);
     DLGO_LAUNCH_CHECK("attention_combine");
   }
   return nullptr;
@@ -1665,20 +1694,22 @@ extern "C" const char* dlgo_attention_decode_f32(const void* q, int ldq, void* o
   DLGO_REQUIRE(window >= 0, "attention: bad window");
   const int group = n_heads / n_kv;
   const int head_blocks = (group + 15) / 16;
-  int nwv, n_splits;
-  decode_plan(n_seq * n_kv * head_blocks, group, max_pages_used, false, false, &nwv, &n_splits);
+  int nwv;
+  SplitPlan plan;
+  decode_plan(n_seq * n_kv * head_blocks, group, max_pages_used, false, false, &nwv, &plan);
+  const int n_splits = plan.most;
   if (nwv > 8) nwv = 8;                // a wave holds 128 registers of keys and values: two waves to a SIMD
   DLGO_REQUIRE(n_splits == 1 || (part && part_elems >= (long long)n_seq * n_heads * n_splits * (HEAD_DIM + 4)),
                "attention: scratch for partial results too small");
-  DLGO_REQUIRE((long long)n_kv * head_blocks <= 65535 && n_seq <= 65535 && n_heads <= 65535, "attention: grid too large");
+  DLGO_REQUIRE((long long)n_kv * head_blocks <= 65535 && n_seq <= 65535 && n_heads <= 65535 && n_splits <= 65535, "attention: grid too large");
   if (n_seq == 0) return nullptr;
   const int heads_here = group < 16 ? group : 16;
   const size_t smem = (size_t)nwv * heads_here * (HEAD_DIM + 2) * 4;
-  dim3 grid(n_splits, n_kv * head_blocks, n_seq);
+  dim3 grid(n_kv * head_blocks, n_seq, n_splits);
 #define DECODE_GO(W_)                                                                                                         \
   hipLaunchKernelGGL((attn_decode_f32_kernel<W_>), grid, dim3(W_ * WAVE), smem, stream, (const float*)q, ldq, (float*)out, ldo, \
                      part, positions, slots, page_table, max_pages, (const float*)cache, page_stride, v_off, n_heads, group,  \
-                     head_blocks, n_splits, window, scale)
+                     head_blocks, plan, window, scale)
   if (nwv == 8) DECODE_GO(8);
   else if (nwv == 4) DECODE_GO(4);
   else if (nwv == 2) DECODE_GO(2);
@@ -1687,7 +1718,7 @@ extern "C" const char* dlgo_attention_decode_f32(const void* q, int ldq, void* o
   DLGO_LAUNCH_CHECK("attention_decode_f32");
   if (n_splits > 1) {
     hipLaunchKernelGGL((attn_combine_kernel<float, true>), dim3(n_seq, n_heads), dim3(WAVE), 0, stream, part, (float*)out, ldo,
-                       positions, n_heads, n_splits, window);
+                       positions, n_heads, plan, window);
     DLGO_LAUNCH_CHECK("attention_combine");
   }
   return nullptr;

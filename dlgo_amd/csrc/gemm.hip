@@ -596,7 +596,7 @@ static const char* launch_tiled(const void* W, const void* X, void* Y, int N, in
 
 // In how many runs a product shares its k tiles out when the choice is the kernel's (64x64 tiles).  Few rows of X and
 // few tiles of output: a block for every compute unit, of at least eight k tiles.  More rows (a short prompt) and a long
-// inner size: about two blocks a unit, at most four runs.  (Measured on the shapes of 1B and 8B Llamas.)
+// inner size: about two blocks a unit, at most four runs.  (Measured on the shapes of 1B, 3B and 8B Llamas.)
 static int auto_splits(int N, int Tn, int nk_all, long long part_elems) {
   const long small = (long)((N + 63) / 64) * ((Tn + 63) / 64);
   int splits = 1;
@@ -605,7 +605,13 @@ static int auto_splits(int N, int Tn, int nk_all, long long part_elems) {
       splits = (int)(256 / small);
       if (splits > nk_all / 8) splits = nk_all / 8;
     } else if (small <= 128 && nk_all >= 32) {
-      splits = 2;                                             // half the units would idle otherwise
+      // half the units would idle otherwise: two runs, or with one tile of rows up to four, as many as make the rounds
+      // of 256 blocks times a block's k tiles least (more runs where that is equal: two blocks share a unit well)
+      long best = 0;
+      for (int s = 2; s <= (Tn <= 64 ? 4 : 2); ++s) {
+        const long cost = ((small * s + 255) / 256) * ((nk_all + s - 1) / s);
+        if (s == 2 || cost <= best) { best = cost; splits = s; }
+      }
     }
   } else if (small <= 256 && nk_all >= 128) {
     splits = (int)(512 / small);

@@ -149,16 +149,16 @@ def _streams_rows(weight: torch.Tensor, t: int, kind: int, has_scratch: bool, sp
     # k in 128-byte pieces, if it is a whole number of them (what the kernels that load tiles straight into LDS take)
     piece = 128 // weight.element_size()
     nk = k // piece if k % piece == 0 else 0
-    can_split = has_scratch and splits != 1 and nk >= 32 and n <= 4096
+    can_split = has_scratch and splits != 1 and nk >= 32
     if kind != GEMM_AUTO or splits > 1:
         return kind in (GEMM_STREAM, 5, 6, 7, 8, 9, 10, 11)
     if t <= GEMM_FEW_ROWS_WIDE:         # measured on the shapes of a 1B Llama: a long inner size is better split,
         row_kb = k * weight.element_size() / 1024.0
         if t <= 8 and n >= GEMM_VERY_WIDE and row_kb in (2.0, 3.0, 4.0, 6.0, 8.0):
             return True                 # a vocabulary of rows that go through LDS whole: streamed faster than tiled
-        return not (can_split and nk >= 64) and not (n >= GEMM_VERY_WIDE and nk > 0)   # else a vocabulary is better tiled
-    if t <= GEMM_FEW_ROWS:
-        return n < 16384 and not (can_split and (nk >= 64 or t >= 24)) and (t <= 40 or nk == 0)
+        return not (can_split and n <= 4096 and nk >= 64) and not (n >= GEMM_VERY_WIDE and nk > 0)   # else a vocabulary is better tiled
+    if t <= GEMM_FEW_ROWS:              # measured on the shapes of 1B, 3B and 8B Llamas: up to 128 tiles of 64x64 split k
+        return n < 16384 and not (can_split and n <= 8192 and (nk >= 48 or t >= 24)) and (t <= 40 or nk == 0)
     return False
 
 

@@ -689,18 +689,31 @@ def test_attention_finds_a_far_key_and_respects_the_window_edge(dtype, _, rel, k
     assert not torch.allclose(run([4], [449], 149)[0, :hd], v[300, :hd].float(), atol=0.2)
 
 
+def _wider(table, bound):
+    """The page table with room for sequences of `bound` pages (a recorded step's launch is sized for the longest
+    sequence the cache allows, whatever the sequences hold)."""
+    if bound is None:
+        return table
+    wide = torch.full((table.shape[0], bound), -1, dtype=table.dtype)
+    wide[:, :table.shape[1]] = table
+    return wide
+
+
+@pytest.mark.parametrize("bound", [None, 3000])
 @pytest.mark.parametrize("variant", [0, 1])
 @pytest.mark.parametrize("H,KV,hd,rot,inter,window", [(4, 2, 16, 16, False, 0), (32, 8, 64, 64, False, 0), (6, 3, 48, 32, True, 0),
                                                        (40, 2, 32, 32, False, 0), (8, 8, 128, 128, True, 50), (4, 1, 80, 0, False, 0),
                                                        (6, 2, 80, 48, False, 0), (2, 1, 256, 256, False, 0)])
-def test_decode_attention_that_rotates_and_stores_by_itself(H, KV, hd, rot, inter, window, variant):
+def test_decode_attention_that_rotates_and_stores_by_itself(H, KV, hd, rot, inter, window, variant, bound):
     """One row per sequence: the split kernel given unrotated [q | k | v] rows against the two-kernel way
-    (rotate and store, then attend): the same output, the same cache afterwards."""
+    (rotate and store, then attend): the same output, the same cache afterwards.  Also with a launch sized for
+    sequences of 3,000 pages, of whose blocks a short sequence uses a few."""
     ops = _ops()
     from dlgo_amd.parts import rotary_frequencies
     dtype = torch.bfloat16
     lens = [70, 3, 129, 64, 65, 1, 2000]
     table, slots, storage, page_stride, unit_off, v_off = _paged_setup(dtype, lens, KV, hd, seed=rot + hd)
+    table = _wider(table, bound)
     g = torch.Generator().manual_seed(H + hd)
     for i, n in enumerate(lens):                       # what the sequences hold before this step
         if n > 1:
@@ -733,6 +746,87 @@ def test_decode_attention_that_rotates_and_stores_by_itself(H, KV, hd, rot, inte
         caches.append(store.cpu())
     assert torch.equal(caches[0], caches[1])
     assert torch.allclose(outs[0], outs[1], atol=1e-6, rtol=0)
+
+
+def _fill_pages(storage, table, slot, k, v, KV, hd, page_stride, unit_off, v_off):
+    """_fill_cache a page at a time."""
+    from dlgo_amd.cache import PAGE
+    for pg in range((k.shape[0] + PAGE - 1) // PAGE):
+        p0, p1 = pg * PAGE, min(k.shape[0], (pg + 1) * PAGE)
+        base = int(table[slot, pg]) * page_stride + unit_off
+        for kvh in range(KV):
+            o = base + kvh * PAGE * hd
+            storage[o:o + (p1 - p0) * hd] = k[p0:p1, kvh * hd:(kvh + 1) * hd].reshape(-1)
+            ov = base + v_off + kvh * hd * PAGE
+            storage[ov:ov + hd * PAGE].view(hd, PAGE)[:, :p1 - p0] = v[p0:p1, kvh * hd:(kvh + 1) * hd].T
+
+
+@pytest.mark.parametrize("kernel", ["bfloat16", "bfloat16 registers", "float32"])
+@pytest.mark.parametrize("H,KV,hd,bound,lens", [
+    # 288 (sequence, kv head) pairs fill the chip by themselves: a sequence gets a second block from about 12,000 tokens
+    (8, 8, 64, 400, [12500, 8200, 4097, 64, 65, 1] + [3 + 7 * i for i in range(30)]),
+    # ten pairs: every sequence is dealt to 26 blocks, the longest to more of the 47 the launch holds
+    (4, 2, 128, 3000, [9000, 300, 1, 2049, 130]),
+    # 64 pairs: four blocks each, ten for the sequence of 40,000 tokens
+    (4, 2, 128, 3000, [40000, 77, 9000] + [5 + 11 * i for i in range(29)]),
+])
+def test_decode_attention_of_short_sequences_in_a_launch_sized_for_long_ones(H, KV, hd, bound, lens, kernel):
+    """A recorded decode step is launched with blocks for the longest sequence the cache allows; a sequence uses as many
+    of them as its own pages call for.  A page that falls between two blocks' shares, or is read by both, would be lost
+    among thousands of random keys, so each sequence holds marked keys (the first and last of its pages, of the first
+    and last page, of the pages where a share may end), each answering to a query along one axis so strongly that the
+    output is that key's value."""
+    ops = _ops()
+    from dlgo_amd.cache import PAGE
+    dtype = torch.float32 if kernel == "float32" else torch.bfloat16
+    table, slots, storage, page_stride, unit_off, v_off = _paged_setup(dtype, lens, KV, hd, seed=hd + len(lens))
+    table = _wider(table, bound)
+    g = torch.Generator().manual_seed(bound)
+    n_marks = 16
+    marks, values = [], []
+    for i, length in enumerate(lens):
+        pages = (length + PAGE - 1) // PAGE
+        cand = [0, PAGE - 1, PAGE, length - 1, length - 2, (pages - 1) * PAGE, (pages - 1) * PAGE - 1]
+        for used in (2, 3, 4, 5, 6, 7, 8, 26, 27, 30):
+            span = (pages + used - 1) // used
+            cand += [span * PAGE - 1, span * PAGE, 2 * span * PAGE - 1, 2 * span * PAGE, (used - 1) * span * PAGE]
+        mine = []
+        for c in cand:
+            if 0 <= c < length and c not in mine:
+                mine.append(c)
+        mine = (mine * n_marks)[:n_marks] if len(mine) < n_marks else mine[:n_marks]
+        k = (0.05 * torch.randn(length, KV * hd, generator=g)).to(dtype)
+        v = torch.randn(length, KV * hd, generator=g).to(dtype)
+        for axis, t in enumerate(mine):
+            if mine.index(t) == axis:               # a position marked twice answers to its first axis
+                for kvh in range(KV):
+                    k[t, kvh * hd:(kvh + 1) * hd] = 0
+                    k[t, kvh * hd + axis] = 60.0
+        _fill_pages(storage, table, slots[i], k, v, KV, hd, page_stride, unit_off, v_off)
+        marks.append(mine)
+        values.append(v.float())
+    dev = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    n = len(lens)
+    store = storage.to(DEV)
+    positions, tok_seq, dslots, dtable = dev([x - 1 for x in lens]), dev(list(range(n))), dev(slots), table.to(DEV)
+    g_heads = H // KV
+    for axis in range(n_marks):
+        q = torch.zeros(n, H, hd)
+        q[:, :, axis] = 60.0
+        q = q.reshape(n, H * hd).to(dtype).to(DEV)
+        out = torch.full((n, H * hd), float("nan"), dtype=dtype, device=DEV)
+        ops.attention(q, out, H, KV, hd, positions, tok_seq, dslots, dtable, store[unit_off:], page_stride, v_off,
+                      q_lens=[1] * n, start_pos=[x - 1 for x in lens], kernel="split", max_pages_used=bound,
+                      split_variant=1 if kernel == "bfloat16 registers" else 0)
+        got = out.float().cpu().view(n, H, hd)
+        for i in range(n):
+            t = marks[i][axis]
+            if marks[i].index(t) != axis:           # a short sequence has fewer marks than axes
+                continue
+            for h in range(H):
+                kvh = h // g_heads
+                assert torch.allclose(got[i, h], values[i][t, kvh * hd:(kvh + 1) * hd], atol=2e-2), \
+                    f"sequence {i} of {lens[i]} tokens, key {t}, head {h}"
 
 
 def test_attention_reference_vectors():
