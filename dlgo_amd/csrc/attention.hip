@@ -880,8 +880,8 @@ static __device__ __forceinline__ void page_to_lds(const void* base, uint32_t vo
 
 // what rotated8 reads, separated from what it computes, so that the loads can stand in front of a page's loads
 struct Rot8In {
-  uint4 x, p;
-  float4 c0, c1, s0, s1;
+  uint4 x, p = {};
+  float4 c0 = {}, c1 = {}, s0 = {}, s1 = {};
 };
 __device__ __forceinline__ Rot8In rot8_load(const bf16_t* __restrict__ vec, int d0, const float* __restrict__ cs,
                                             const float* __restrict__ sn, int rot, int interleaved) {

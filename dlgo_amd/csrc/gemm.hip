@@ -201,7 +201,6 @@ __global__ __launch_bounds__(WN* WT* WAVE) void gemm_direct_kernel(const T* __re
                                                                      int ldy, int tiles_t, int nk_split, long long split_stride,
                                                                      TileNorm tn) {
   constexpr int NW = WN * WT;
-  constexpr int EPC = 16 / sizeof(T);
   constexpr int BK = 128 / sizeof(T);
   constexpr int MI = BN / WN / 32, NJ = BT / WT / 32;
   constexpr int LA = BN / 8 / NW, LB = BT / 8 / NW;     // loads (8 rows of 128 bytes each) per wave and stage
