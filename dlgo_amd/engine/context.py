@@ -18,9 +18,18 @@ class Workspace:
         self.max_rows = max_rows
         self._bufs: Dict[Tuple[str, int, torch.dtype], torch.Tensor] = {}
         self._retired: List[torch.Tensor] = []
+        self._views: Dict[str, Tuple[tuple, torch.dtype, torch.Tensor]] = {}    # name -> the last (shape, dtype, view) handed out
 
     def get(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
-        rows, cols = int(shape[0]), int(np.prod(shape[1:], dtype=np.int64)) if len(shape) > 1 else 1
+        # the layers of a step ask for the same rows one after the other: the view made for the first serves the rest
+        # (views keep no state of their own, and the buffer under them never moves)
+        last = self._views.get(name)
+        if last is not None and last[0] == shape and last[1] is dtype:
+            return last[2]
+        rows = int(shape[0])
+        cols = 1
+        for n in shape[1:]:
+            cols *= int(n)
         if rows > self.max_rows:
             raise RuntimeError(f"workspace {name}: {rows} rows asked, room for {self.max_rows}")
         key = (name, cols, dtype)
@@ -28,7 +37,9 @@ class Workspace:
         if buf is None:
             buf = torch.empty((self.max_rows, cols), dtype=dtype, device=self.device)
             self._bufs[key] = buf
-        return buf[:rows].view(rows, *shape[1:]) if len(shape) > 1 else buf[:rows, 0]
+        view = buf[:rows].view(rows, *shape[1:]) if len(shape) > 1 else buf[:rows, 0]
+        self._views[name] = (tuple(shape), dtype, view)
+        return view
 
     def flat(self, name: str, n: int, dtype: torch.dtype, zero: bool = False) -> torch.Tensor:
         """A flat scratch buffer of at least n elements (zero-filled when made, if asked).  When a larger one

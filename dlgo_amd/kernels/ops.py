@@ -39,10 +39,14 @@ def dtype_code(dtype: torch.dtype) -> int:
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)    # the handle without a Stream object around it
 
 
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)              # the current device without torch.cuda's start-up check
+
+
 def _stream() -> ctypes.c_void_p:
-    """torch's current stream on the current device, as the launches take it."""
-    if _raw_stream is not None:
-        return ctypes.c_void_p(_raw_stream(torch.cuda.current_device()))
+    """torch's current stream on the current device, as the launches take it (asked at every launch: a recording has
+    a stream of its own)."""
+    if _raw_stream is not None and _raw_device is not None:
+        return ctypes.c_void_p(_raw_stream(_raw_device()))
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
@@ -61,9 +65,10 @@ def _need(t: torch.Tensor, name: str, dtype: Optional[torch.dtype] = None, dims:
 
 def _rows(t: torch.Tensor, name: str) -> int:
     """Row stride (elements) of a 2-d tensor whose rows are contiguous."""
-    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
-        raise KernelError(f"{name}: expected rows that are contiguous in memory, found shape {tuple(t.shape)} strides {t.stride()}")
-    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+    strides = t.stride()
+    if len(strides) != 2 or (strides[1] != 1 and t.shape[1] > 1):
+        raise KernelError(f"{name}: expected rows that are contiguous in memory, found shape {tuple(t.shape)} strides {strides}")
+    return strides[0] if t.shape[0] > 1 else max(strides[0], t.shape[1])
 
 
 def _check(err: Optional[bytes]) -> None:
