@@ -183,7 +183,10 @@ def test_gemm_direct_to_lds(dtype, _, rel, kind, n, t, k):
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
 @pytest.mark.parametrize("n,t,k,splits", [(130, 20, 512, 2), (64, 64, 2048, 5), (257, 33, 1024, 8), (2048, 64, 8192, 0), (300, 17, 4096, 0),
-                                          (96, 40, 640, 3)])
+                                          (96, 40, 640, 3),
+                                          # 96 and 80 tiles of output: between a half and a whole round of the chip, where
+                                          # the number of runs is chosen by rounds times tiles of k (four and three here)
+                                          (6144, 32, 4096, 0), (5120, 17, 3072, 0)])
 def test_gemm_with_split_inner_size(dtype, _, rel, n, t, k, splits):
     """The inner size shared out over blocks whose sums are added in a fixed order: every epilogue, runs that do not
     divide the tiles evenly, and twice the same bits."""
