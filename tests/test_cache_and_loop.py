@@ -178,6 +178,31 @@ def test_state_is_zeroed_when_a_slot_is_handed_out():
     assert t == s and torch.equal(c.state_of(0)[t], torch.zeros(5))
 
 
+def test_workspace_buffers_keep_their_place():
+    """A step's scratch rows: a buffer per (name, width, type) that never moves, so that a recorded step can be
+    replayed; the view made for one layer serves the next one that asks for the same rows, and other rows or another
+    width get views of their own."""
+    from dlgo_amd.engine.context import Workspace
+    ws = Workspace(torch.device("cpu"), 16)
+    a = ws.get("rows", (5, 8), torch.float32)
+    assert tuple(a.shape) == (5, 8) and ws.get("rows", (5, 8), torch.float32) is a
+    b = ws.get("rows", (7, 8), torch.float32)
+    assert tuple(b.shape) == (7, 8) and b.data_ptr() == a.data_ptr()          # more rows of the same buffer
+    c = ws.get("rows", (5, 4, 2), torch.float32)
+    assert tuple(c.shape) == (5, 4, 2) and c.data_ptr() == a.data_ptr()       # the same width, seen as 4 x 2
+    d = ws.get("rows", (5, 6), torch.float32)
+    e = ws.get("rows", (5, 8), torch.bfloat16)
+    assert len({a.data_ptr(), d.data_ptr(), e.data_ptr()}) == 3              # another width, another type: other buffers
+    a.fill_(3.0)
+    assert float(ws.get("rows", (5, 8), torch.float32)[4, 7]) == 3.0          # and the first one is still where it was
+    assert tuple(ws.get("flags", (9,), torch.int32).shape) == (9,)
+    with pytest.raises(RuntimeError, match="room for 16"):
+        ws.get("rows", (17, 8), torch.float32)
+    f1 = ws.flat("runs", 100, torch.float32)
+    assert ws.flat("runs", 50, torch.float32) is f1 and ws.flat("runs", 200, torch.float32).numel() >= 200
+    assert ws.bytes() > 0
+
+
 def test_random_traffic_keeps_the_books():
     rng = random.Random(0)
     c = make_cache(n_units=3, max_tokens=40 * PAGE, max_ctx=10 * PAGE, max_slots=6,
