@@ -43,7 +43,7 @@ template <typename F>
 __device__ __forceinline__ void for_each_element(const float* __restrict__ row, int V, bool vec, F f) {
   if (vec) {
     const float4* r4 = (const float4*)row;
-#pragma unroll 4
+#pragma unroll 8
     for (int i = threadIdx.x; i < V / 4; i += SAMP_THREADS) {
       const float4 x = r4[i];
       f(4 * i, x.x);
@@ -555,7 +555,7 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
   // temperature for all, then the repetition penalty (which comes first in the pipeline) redone for the few it touches
   const bool vec = (V & 3) == 0 && (ld & 3) == 0 && ((uintptr_t)logits & 15) == 0 && ((uintptr_t)work_all & 15) == 0;
   if (vec) {
-#pragma unroll 4
+#pragma unroll 8
     for (int i = threadIdx.x; i < V / 4; i += SAMP_THREADS) {
       float4 x = ((const float4*)lg)[i];
       if (inv_temp != 1.0f) {
@@ -740,13 +740,20 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
 #pragma unroll
     for (int c = 0; c < 4; ++c) ev[c] = expf(x[c] - top.v);
   };
+  // The totals of the 256-element pieces are kept (where the row is not too long for that), so that the wave that
+  // holds the target goes straight to the piece that reaches it instead of walking its run from the start.
+  float* piece_total = S.sv;            // sv, si, se and skey lie together and are free by now: 4 * SAMP_CAND floats
+  const int pieces = seg / (4 * WAVE);  // of a wave's run
+  const bool keep = pieces * SAMP_WAVES <= 4 * SAMP_CAND;
   float running = 0.f;
-#pragma unroll 2
+#pragma unroll 4
   for (int b = w0; b < w1; b += 4 * WAVE) {
     float ev[4];
     four(b + 4 * lane, ev);
     const float mine = ((ev[0] + ev[1]) + ev[2]) + ev[3];
-    running += __shfl(scan64(mine), WAVE - 1, WAVE);
+    const float total = __shfl(scan64(mine), WAVE - 1, WAVE);
+    running += total;
+    if (keep && lane == 0) piece_total[wave * pieces + (b - w0) / (4 * WAVE)] = total;
   }
   if (lane == 0) scan[wave] = running;
   if (threadIdx.x == 0) chosen = -1;
@@ -773,6 +780,37 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
   if (wave == holder) {
     float cum = before;
     int pick = -1, last = -1;
+    if (keep) {
+      // the first piece whose end reaches the target, by the same sums in the same order as the walk below makes them.
+      // (A walk from the start could stop a piece earlier, at a lane whose sum rounds above its piece's total: a draw
+      // within rounding of an edge either way.  If the piece found holds no such element after all, or none reaches
+      // the target, the walk from the start decides as it always did.)
+      float c = before;
+      int p = 0;
+      const int n_mine = (w1 - w0 + 4 * WAVE - 1) / (4 * WAVE);
+      for (; p < n_mine; ++p) {
+        const float t = piece_total[wave * pieces + p];
+        if (c + t >= target) break;
+        c += t;
+      }
+      if (p < n_mine) {
+        float ev[4];
+        const int i0 = w0 + p * 4 * WAVE + 4 * lane;
+        four(i0, ev);
+        const float s1 = ev[0], s2 = s1 + ev[1], s3 = s2 + ev[2], s4 = s3 + ev[3];
+        const float incl = scan64(s4);
+        float excl = __shfl_up(incl, 1, WAVE);
+        if (lane == 0) excl = 0.f;
+        const float base = c + excl;
+        const float sums[4] = {s1, s2, s3, s4};
+        int mine_pick = -1;
+#pragma unroll
+        for (int e = 3; e >= 0; --e)
+          if (ev[e] > 0.f && base + sums[e] >= target) mine_pick = i0 + e;
+        const unsigned long long hit = __ballot(mine_pick >= 0);
+        if (hit) pick = __shfl(mine_pick, __ffsll((long long)hit) - 1, WAVE);
+      }
+    }
     for (int b = w0; b < w1 && pick < 0; b += 4 * WAVE) {
       float ev[4];
       const int i0 = b + 4 * lane;
