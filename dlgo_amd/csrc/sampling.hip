@@ -56,11 +56,8 @@ __device__ __forceinline__ void for_each_element(const float* __restrict__ row, 
   }
 }
 
-__device__ BestIdx block_argmax(const float* row, int V, BestIdx* red, bool vec = false) {
-  BestIdx best = {-INFINITY, -1};
-  for_each_element(row, V, vec, [&](int i, float v) {
-    if (v == v) best = better(best, BestIdx{v, i});
-  });
+// the best of what the block's threads have each found
+__device__ BestIdx block_best(BestIdx best, BestIdx* red) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) {
     BestIdx other;
@@ -74,6 +71,14 @@ __device__ BestIdx block_argmax(const float* row, int V, BestIdx* red, bool vec 
   BestIdx r = red[0];
   for (int w = 1; w < SAMP_WAVES; ++w) r = better(r, red[w]);
   return r;
+}
+
+__device__ BestIdx block_argmax(const float* row, int V, BestIdx* red, bool vec = false) {
+  BestIdx best = {-INFINITY, -1};
+  for_each_element(row, V, vec, [&](int i, float v) {
+    if (v == v) best = better(best, BestIdx{v, i});
+  });
+  return block_best(best, red);
 }
 
 __device__ float block_sum_f(float v, float* red) {
@@ -537,7 +542,7 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
   __shared__ float red[SAMP_WAVES];
   __shared__ SampleSmall S;
   __shared__ int hist[256];
-  __shared__ int chosen, bstar, cut_bin;
+  __shared__ int chosen, bstar, cut_bin, again;
   __shared__ unsigned long long cut_before;
   float* scan = S.scan;
   const int row = blockIdx.x;
@@ -552,8 +557,14 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
   }
   float* work = work_all + (size_t)row * V;
   const float inv_temp = temp == 1.0f ? 1.0f : 1.0f / temp;
-  // temperature for all, then the repetition penalty (which comes first in the pipeline) redone for the few it touches
+  // temperature for all, then the repetition penalty (which comes first in the pipeline) redone for the few it touches.
+  // The largest element is looked for on the way: the penalty only lowers values, so it stands unless it is one of the
+  // penalised tokens itself, and then the row is searched again.
   const bool vec = (V & 3) == 0 && (ld & 3) == 0 && ((uintptr_t)logits & 15) == 0 && ((uintptr_t)work_all & 15) == 0;
+  BestIdx seen = {-INFINITY, -1};
+  auto look = [&](int i, float x) {
+    if (x == x) seen = better(seen, BestIdx{x, i});
+  };
   if (vec) {
 #pragma unroll 8
     for (int i = threadIdx.x; i < V / 4; i += SAMP_THREADS) {
@@ -565,11 +576,20 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
         x.w *= inv_temp;
       }
       ((float4*)work)[i] = x;
+      look(4 * i, x.x);
+      look(4 * i + 1, x.y);
+      look(4 * i + 2, x.z);
+      look(4 * i + 3, x.w);
     }
   } else {
-    for (int i = threadIdx.x; i < V; i += SAMP_THREADS) work[i] = inv_temp != 1.0f ? lg[i] * inv_temp : lg[i];
+    for (int i = threadIdx.x; i < V; i += SAMP_THREADS) {
+      const float x = inv_temp != 1.0f ? lg[i] * inv_temp : lg[i];
+      work[i] = x;
+      look(i, x);
+    }
   }
-  __syncthreads();
+  if (threadIdx.x == 0) again = 0;
+  BestIdx top = block_best(seen, redb);      // (its barriers also put the row in place for the reads below)
   // repetition penalty: each distinct recent token once
   // The recent tokens of this row: row `rr` of the table, all n_recent entries (-1 where empty), or with `counts` a
   // ring that holds the last min(counts[rr], n_recent) tokens, to which the token chosen here is added at the end.
@@ -591,10 +611,11 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
     if (first) {
       const float x = lg[tok] > 0.f ? lg[tok] / pen : lg[tok] * pen;
       work[tok] = inv_temp != 1.0f ? x * inv_temp : x;
+      if (tok == top.i) again = 1;
     }
   }
   __syncthreads();
-  BestIdx top = block_argmax(work, V, redb, vec);
+  if (again) top = block_argmax(work, V, redb, vec);
   const int k = top_k[row];
   const float tp = top_p[row], mp = min_p[row];
   // top-k: everything below the k-th largest value is masked; ties at it stay
@@ -891,13 +912,14 @@ extern "C" const char* dlgo_argmax_noalloc(const float* logits, int ld, int n_ro
   return nullptr;
 }
 
-// work: [n_rows, V] float32 scratch.  recent: a table of token ids with n_recent columns.  Without counts, row r of
+// work: [n_rows, V] float32 scratch.  small_top_k: 1 unless the caller knows the rows' options and none has a top-k of
+// 1 to 128 (the result is the same either way).  recent: a table of token ids with n_recent columns.  Without counts, row r of
 // it holds row r's recent tokens, -1 where empty.  With recent_rows and counts, row recent_rows[r] of it is a ring of the
 // last tokens chosen for that key, counts[key] the number chosen so far; the kernel adds the token it chooses.
 extern "C" const char* dlgo_sample(const float* logits, int ld, int n_rows, int V, float* work,
                                    const float* temperature, const int32_t* top_k, const float* top_p, const float* min_p,
                                    const float* penalty, int32_t* recent, int n_recent, const int32_t* recent_rows,
-                                   int32_t* counts, const float* uniform, int32_t* out, hipStream_t stream) {
+                                   int32_t* counts, const float* uniform, int32_t* out, int small_top_k, hipStream_t stream) {
   DLGO_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "sample: bad sizes rows=%d V=%d ld=%d", n_rows, V, ld);
   DLGO_REQUIRE(n_recent >= 0 && n_recent <= SAMP_THREADS, "sample: at most %d recent tokens, got %d", SAMP_THREADS, n_recent);
   DLGO_REQUIRE(work && temperature && top_k && top_p && min_p && penalty && uniform && out, "sample: missing argument");
@@ -905,7 +927,8 @@ extern "C" const char* dlgo_sample(const float* logits, int ld, int n_rows, int 
   DLGO_REQUIRE((recent_rows == nullptr) == (counts == nullptr), "sample: a ring of recent tokens needs both its rows and its counts");
   if (n_rows == 0) return nullptr;
   // a wide vocabulary: rows with a small top-k are dealt to several blocks first; sample_kernel takes what they leave
-  const int staged = V >= TK_MIN_V && V <= TK_CHUNKS * TK_CHUNK_MAX && V >= TK_SCRATCH && n_rows <= 65535;
+  // (small_top_k: 0 = the caller knows that no row has a top-k of 1 to TK_CAP, so the two kernels would find nothing to do)
+  const int staged = small_top_k != 0 && V >= TK_MIN_V && V <= TK_CHUNKS * TK_CHUNK_MAX && V >= TK_SCRATCH && n_rows <= 65535;
   if (staged) {
     hipLaunchKernelGGL(topk_part_kernel, dim3(TK_CHUNKS, n_rows), dim3(TK_THREADS), 0, stream, logits, ld, V, work, temperature,
                        top_k, penalty, recent, n_recent, recent_rows, counts);

@@ -135,9 +135,10 @@ class Sampler:
                 raise ValueError("sampler: keys that start() was never given")
             k[1] = np.asarray(keys, dtype=np.int32)
         fd, kd = self._upload(f, k)
+        small_top_k = any(not c.greedy and 1 <= c.top_k <= 128 for c in configs)     # else two kernels need not be launched
         if rings:       # every choice is recorded, penalty or not: a later row of the request may have one
             ops.sample(logits, self._work, fd[0], kd[0], fd[1], fd[2], fd[3], self._rings, fd[4], out,
-                       recent_rows=kd[1], counts=self._counts)
+                       recent_rows=kd[1], counts=self._counts, small_top_k=small_top_k)
             return out
         rec = None
         if recent is not None and penalised:
@@ -146,5 +147,5 @@ class Sampler:
                 toks = list(toks)[-RECENT:]
                 r[i, :len(toks)] = toks
             rec = torch.from_numpy(r).to(self.device)
-        ops.sample(logits, self._work, fd[0], kd[0], fd[1], fd[2], fd[3], rec, fd[4], out)
+        ops.sample(logits, self._work, fd[0], kd[0], fd[1], fd[2], fd[3], rec, fd[4], out, small_top_k=small_top_k)
         return out

@@ -986,6 +986,13 @@ def test_sample_wide_rows_dealt_to_several_blocks():
             want = plain.sample_token(rows[i].double().numpy(), u, c["temp"], c.get("top_k", 0), c.get("top_p", 1.0),
                                       c.get("min_p", 0.0), c.get("pen", 1.0), recents[i])
             assert got[i] == want, (i, c, u)
+        # a caller that knows no row has a small top-k may say so, and two kernels are not launched: the same tokens
+        # (said of rows that do have one, it costs time only: the one-block kernel takes them)
+        again = torch.empty_like(out)
+        ops.sample(lg, work, col("temp", 1.0, torch.float32), col("top_k", 0, torch.int32), col("top_p", 1.0, torch.float32),
+                   col("min_p", 0.0, torch.float32), col("pen", 1.0, torch.float32), rec.to(DEV),
+                   torch.full((n,), u, dtype=torch.float32, device=DEV), again, small_top_k=False)
+        assert again.tolist() == got, u
 
 
 def test_sample_reference_behaviour():
