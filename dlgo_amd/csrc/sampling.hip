@@ -285,10 +285,13 @@ __device__ __forceinline__ void first_bin_reaching(const int* hist, int k, int* 
 // parts' sets, cuts them down the same way against the row's maximum and hands them to sample_small, which makes the
 // exact cuts and the draw.  An element that is missing from a part's set has k larger ones in its own part, so it is
 // below the k-th value of the row: the set that sample_small ends up with is the one sample_kernel would have had.
-// Whatever does not fit (a part with more than TK_CAP elements within its cut, no cut within 255 steps, a row
-// without top-k) is left to sample_kernel: the row's scratch says which rows are done.
+// A row that nothing cuts (no top-k, top-p or min-p) goes the same way with sums in place of candidates: see
+// whole_row_draw.  Whatever does not fit (a part with more than TK_CAP elements within its cut, no cut within 255
+// steps, a row with a top-p or min-p cut but no top-k) is left to sample_kernel: the row's scratch says which rows
+// are done.
 // The row's scratch (floats of its row of `work`): maxima [TK_CHUNKS] as (value, index), counts [TK_CHUNKS] (-1: this
-// part gave up), the done flag, then the parts' values [TK_CHUNKS][TK_CAP] and indices [TK_CHUNKS][TK_CAP].
+// part gave up), the done flag, then the parts' values [TK_CHUNKS][TK_CAP] and indices [TK_CHUNKS][TK_CAP] (for a row
+// that nothing cuts: counts = the part's pieces of 256, values = their masses).
 #define TK_CHUNKS 32
 #define TK_CAP 128
 #define TK_THREADS 256
@@ -300,10 +303,20 @@ __device__ __forceinline__ void first_bin_reaching(const int* hist, int k, int* 
 #define TK_INDICES (TK_VALUES + TK_CHUNKS * TK_CAP)
 #define TK_SCRATCH (TK_INDICES + TK_CHUNKS * TK_CAP)
 
+// the elements of a part of a row (the last part may be shorter)
+__device__ __forceinline__ int part_length(int V) { return ((V + TK_CHUNKS - 1) / TK_CHUNKS + 3) & ~3; }
+
+// A row that is drawn from as it is, but for temperature and penalty: no top-k, top-p or min-p cuts anything.  Such a
+// row needs no candidates, only sums, and those the parts can make as well.
+__device__ __forceinline__ bool whole_row_draw(float temp, int k, float tp, float mp, int V) {
+  return temp > 0.f && (k <= 0 || k >= V) && !(tp < 1.0f) && !(mp > 0.f);
+}
+
 __global__ __launch_bounds__(TK_THREADS) void topk_part_kernel(const float* __restrict__ logits, int ld, int V,
                                                                float* __restrict__ work_all,
                                                                const float* __restrict__ temperature,
-                                                               const int32_t* __restrict__ top_k, const float* __restrict__ penalty,
+                                                               const int32_t* __restrict__ top_k, const float* __restrict__ top_p,
+                                                               const float* __restrict__ min_p, const float* __restrict__ penalty,
                                                                const int32_t* __restrict__ recent, int n_recent,
                                                                const int32_t* __restrict__ recent_rows,
                                                                const int32_t* __restrict__ counts) {
@@ -318,11 +331,12 @@ __global__ __launch_bounds__(TK_THREADS) void topk_part_kernel(const float* __re
   if (chunk == 0 && threadIdx.x == 0) ((int*)scratch)[TK_DONE] = 0;
   const float temp = temperature[row];
   const int k = top_k[row];
-  if (!(temp > 0.f) || k < 1 || k > TK_CAP) {       // not a row for this way
+  const bool whole = whole_row_draw(temp, k, top_p[row], min_p[row], V);
+  if (!whole && (!(temp > 0.f) || k < 1 || k > TK_CAP)) {       // not a row for this way
     if (threadIdx.x == 0) cnt[chunk] = -1;
     return;
   }
-  const int per = ((V + TK_CHUNKS - 1) / TK_CHUNKS + 3) & ~3;
+  const int per = part_length(V);
   const int c0 = chunk * per < V ? chunk * per : V, c1 = c0 + per < V ? c0 + per : V;
   const float* lg = logits + (size_t)row * ld;
   const float inv_temp = temp == 1.0f ? 1.0f : 1.0f / temp;
@@ -399,6 +413,32 @@ __global__ __launch_bounds__(TK_THREADS) void topk_part_kernel(const float* __re
     }
     return;
   }
+  if (whole) {
+    // no cut at all: what the draw needs of this part is its mass, exp(x - the part's maximum) added up in pieces of
+    // 256 elements (a lane four neighbours, then the lanes in a fixed order); topk_final_kernel scales the parts to the
+    // row's maximum, finds the piece that reaches the target and walks that piece alone
+    float* mass = scratch + TK_VALUES + chunk * TK_CAP;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n_pieces = (c1 - c0 + 4 * WAVE - 1) / (4 * WAVE);
+    for (int pc = wave; pc < n_pieces; pc += TK_THREADS / WAVE) {
+      const int j0 = pc * 4 * WAVE + 4 * lane;
+      float ev[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float below = j0 + e < c1 - c0 ? xs[j0 + e] - best.v : -INFINITY;
+        ev[e] = below == below ? expf(below) : 0.f;        // (a part of nothing but -inf has no mass: -inf - -inf is no number)
+      }
+      float sum = ((ev[0] + ev[1]) + ev[2]) + ev[3];
+#pragma unroll
+      for (int o = 1; o < WAVE; o <<= 1) sum += __shfl_xor(sum, o, WAVE);
+      if (lane == 0) mass[pc] = sum;
+    }
+    if (threadIdx.x == 0) {
+      cnt[chunk] = n_pieces;
+      ((BestIdx*)scratch)[chunk] = best;
+    }
+    return;
+  }
   const uint32_t kmax = order_key(best.v);
   for (int i = c0 + threadIdx.x; i < c1; i += TK_THREADS) {
     const uint32_t bin = (kmax - order_key(xs[i - c0])) >> 16;
@@ -436,10 +476,12 @@ __global__ __launch_bounds__(TK_THREADS) void topk_part_kernel(const float* __re
   }
 }
 
-__global__ __launch_bounds__(SAMP_THREADS) void topk_final_kernel(int V, float* __restrict__ work_all,
+__global__ __launch_bounds__(SAMP_THREADS) void topk_final_kernel(const float* __restrict__ logits, int ld, int V,
+                                                                  float* __restrict__ work_all,
                                                                   const float* __restrict__ temperature,
                                                                   const int32_t* __restrict__ top_k, const float* __restrict__ top_p,
-                                                                  const float* __restrict__ min_p, int32_t* __restrict__ recent,
+                                                                  const float* __restrict__ min_p, const float* __restrict__ penalty,
+                                                                  int32_t* __restrict__ recent,
                                                                   int n_recent, const int32_t* __restrict__ recent_rows,
                                                                   int32_t* __restrict__ counts, const float* __restrict__ uniform,
                                                                   int32_t* __restrict__ out) {
@@ -451,7 +493,8 @@ __global__ __launch_bounds__(SAMP_THREADS) void topk_final_kernel(int V, float* 
   float* scratch = work_all + (size_t)row * V;
   const float temp = temperature[row];
   const int k = top_k[row];
-  if (!(temp > 0.f) || k < 1 || k > TK_CAP) return;
+  const bool whole = whole_row_draw(temp, k, top_p[row], min_p[row], V);
+  if (!whole && (!(temp > 0.f) || k < 1 || k > TK_CAP)) return;
   __shared__ BestIdx part_top[TK_CHUNKS];
   if (threadIdx.x < TK_CHUNKS) {
     part_n[threadIdx.x] = ((const int*)scratch)[TK_COUNTS + threadIdx.x];
@@ -480,6 +523,114 @@ __global__ __launch_bounds__(SAMP_THREADS) void topk_final_kernel(int V, float* 
   __syncthreads();
   if (bstar == -2) return;                        // a part gave up, or the row has nothing but NaN
   const BestIdx top = top_s;
+  if (whole) {
+    // The draw over the whole row from the parts' masses: one wave.  Cumulative sums in index order: the parts (each
+    // scaled from its own maximum to the row's), within the part that reaches the target its pieces of 256, within
+    // that piece its elements, taken from the logits again with temperature and penalty as the part applied them.
+    // Where rounding leaves a level without an element that reaches the target, the last one with any weight is taken
+    // (as sample_kernel does); a level with no weight at all leaves the row to sample_kernel.
+    if (threadIdx.x >= WAVE) return;
+    const int lane = threadIdx.x;
+    auto scan64 = [&](float x) {          // inclusive, lanes in order
+#pragma unroll
+      for (int o = 1; o < WAVE; o <<= 1) {
+        const float y = __shfl_up(x, o, WAVE);
+        if (lane >= o) x += y;
+      }
+      return x;
+    };
+    auto first_reaching = [&](float weight, float incl, float before, float target, int* at, float* excl_at) {
+      const unsigned long long hit = __ballot(weight > 0.f && before + incl >= target);
+      const unsigned long long any = __ballot(weight > 0.f);
+      if (!any) return false;
+      *at = hit ? __ffsll((long long)hit) - 1 : 63 - __clzll(any);
+      float excl = __shfl_up(incl, 1, WAVE);
+      if (lane == 0) excl = 0.f;
+      *excl_at = __shfl(excl, *at, WAVE);
+      return true;
+    };
+    const int n_mine = lane < TK_CHUNKS ? part_n[lane] : 0;
+    const float scale = n_mine > 0 ? expf(part_top[lane].v - top.v) : 0.f;
+    float part_mass = 0.f;
+    {
+      const float* mass = scratch + TK_VALUES + (lane < TK_CHUNKS ? lane : 0) * TK_CAP;
+      for (int pc = 0; pc < n_mine; ++pc) part_mass += mass[pc] * scale;
+    }
+    const float part_incl = scan64(part_mass);
+    const float Z = __shfl(part_incl, WAVE - 1, WAVE);
+    const float target = uniform[row] * Z;
+    int c_at, p_at;
+    float before, more;
+    if (!first_reaching(part_mass, part_incl, 0.f, target, &c_at, &before)) return;
+    const int n_pieces = __shfl(n_mine, c_at, WAVE);
+    const float scale_at = __shfl(scale, c_at, WAVE);
+    const float piece_mass = lane < n_pieces ? (scratch + TK_VALUES + c_at * TK_CAP)[lane] * scale_at : 0.f;
+    if (!first_reaching(piece_mass, scan64(piece_mass), before, target, &p_at, &more)) return;
+    before += more;
+    // the piece's elements
+    const int per = part_length(V);
+    const int c0 = c_at * per, c1 = c0 + per < V ? c0 + per : V;
+    const int i0 = c0 + p_at * 4 * WAVE + 4 * lane;
+    const float* lg = logits + (size_t)row * ld;
+    const float inv_temp = temp == 1.0f ? 1.0f : 1.0f / temp;
+    const float pen = penalty[row];
+    const int rr = recent_rows ? recent_rows[row] : row;
+    const int held = counts ? (counts[rr] < n_recent ? counts[rr] : n_recent) : n_recent;
+    const int32_t* rc = recent + (size_t)rr * n_recent;
+    // which of the piece's elements are recent tokens: the list 64 at a time, a lane each, and passed round
+    bool listed[4] = {false, false, false, false};
+    if (pen > 1.0f && n_recent > 0) {
+      const int piece0 = c0 + p_at * 4 * WAVE;
+      for (int t0 = 0; t0 < held; t0 += WAVE) {
+        const int mine_tok = t0 + lane < held ? rc[t0 + lane] : -1;
+        const int m = held - t0 < WAVE ? held - t0 : WAVE;
+        for (int t = 0; t < m; ++t) {
+          const int tok = __shfl(mine_tok, t, WAVE);
+          if ((unsigned)(tok - piece0) < (unsigned)(4 * WAVE)) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) listed[e] = listed[e] || tok == i0 + e;
+          }
+        }
+      }
+    }
+    float ev[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      ev[e] = 0.f;
+      if (i0 + e < c1) {
+        float x = lg[i0 + e];
+        if (listed[e]) x = x > 0.f ? x / pen : x * pen;
+        if (inv_temp != 1.0f) x *= inv_temp;
+        ev[e] = expf(x - top.v);
+      }
+    }
+    const float s1 = ev[0], s2 = s1 + ev[1], s3 = s2 + ev[2], s4 = s3 + ev[3];
+    const float incl = scan64(s4);
+    float excl = __shfl_up(incl, 1, WAVE);
+    if (lane == 0) excl = 0.f;
+    const float base = before + excl;
+    const float sums[4] = {s1, s2, s3, s4};
+    int mine_pick = -1, mine_last = -1;
+#pragma unroll
+    for (int e = 3; e >= 0; --e)
+      if (ev[e] > 0.f) {
+        if (mine_last < 0) mine_last = i0 + e;
+        if (base + sums[e] >= target) mine_pick = i0 + e;
+      }
+    const unsigned long long hit = __ballot(mine_pick >= 0);
+    const unsigned long long any = __ballot(mine_last >= 0);
+    if (!any) return;
+    const int pick = hit ? __shfl(mine_pick, __ffsll((long long)hit) - 1, WAVE) : __shfl(mine_last, 63 - __clzll(any), WAVE);
+    if (lane == 0) {
+      out[row] = pick;
+      if (counts && n_recent > 0) {
+        recent[(size_t)rr * n_recent + counts[rr] % n_recent] = pick;
+        counts[rr] += 1;
+      }
+      ((int*)scratch)[TK_DONE] = 1;
+    }
+    return;
+  }
   const uint32_t kmax = order_key(top.v);
   const float* cv = scratch + TK_VALUES;
   const int* ci = (const int*)scratch + TK_INDICES;
@@ -912,28 +1063,30 @@ extern "C" const char* dlgo_argmax_noalloc(const float* logits, int ld, int n_ro
   return nullptr;
 }
 
-// work: [n_rows, V] float32 scratch.  small_top_k: 1 unless the caller knows the rows' options and none has a top-k of
-// 1 to 128 (the result is the same either way).  recent: a table of token ids with n_recent columns.  Without counts, row r of
+// work: [n_rows, V] float32 scratch.  dealt_rows: 1 unless the caller knows the rows' options and none is of a kind that
+// several blocks share (a top-k of 1 to 128, or no cut at all); a row is drawn from the same distribution either way,
+// and a row with a top-k gets the same token.  recent: a table of token ids with n_recent columns.  Without counts, row r of
 // it holds row r's recent tokens, -1 where empty.  With recent_rows and counts, row recent_rows[r] of it is a ring of the
 // last tokens chosen for that key, counts[key] the number chosen so far; the kernel adds the token it chooses.
 extern "C" const char* dlgo_sample(const float* logits, int ld, int n_rows, int V, float* work,
                                    const float* temperature, const int32_t* top_k, const float* top_p, const float* min_p,
                                    const float* penalty, int32_t* recent, int n_recent, const int32_t* recent_rows,
-                                   int32_t* counts, const float* uniform, int32_t* out, int small_top_k, hipStream_t stream) {
+                                   int32_t* counts, const float* uniform, int32_t* out, int dealt_rows, hipStream_t stream) {
   DLGO_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "sample: bad sizes rows=%d V=%d ld=%d", n_rows, V, ld);
   DLGO_REQUIRE(n_recent >= 0 && n_recent <= SAMP_THREADS, "sample: at most %d recent tokens, got %d", SAMP_THREADS, n_recent);
   DLGO_REQUIRE(work && temperature && top_k && top_p && min_p && penalty && uniform && out, "sample: missing argument");
   DLGO_REQUIRE(n_recent == 0 || recent, "sample: recent tokens missing");
   DLGO_REQUIRE((recent_rows == nullptr) == (counts == nullptr), "sample: a ring of recent tokens needs both its rows and its counts");
   if (n_rows == 0) return nullptr;
-  // a wide vocabulary: rows with a small top-k are dealt to several blocks first; sample_kernel takes what they leave
-  // (small_top_k: 0 = the caller knows that no row has a top-k of 1 to TK_CAP, so the two kernels would find nothing to do)
-  const int staged = small_top_k != 0 && V >= TK_MIN_V && V <= TK_CHUNKS * TK_CHUNK_MAX && V >= TK_SCRATCH && n_rows <= 65535;
+  // a wide vocabulary: rows with a small top-k, and rows that nothing cuts, are dealt to several blocks first;
+  // sample_kernel takes what they leave
+  // (dealt_rows: 0 = the caller knows that no row is one the two kernels take, so they would find nothing to do)
+  const int staged = dealt_rows != 0 && V >= TK_MIN_V && V <= TK_CHUNKS * TK_CHUNK_MAX && V >= TK_SCRATCH && n_rows <= 65535;
   if (staged) {
     hipLaunchKernelGGL(topk_part_kernel, dim3(TK_CHUNKS, n_rows), dim3(TK_THREADS), 0, stream, logits, ld, V, work, temperature,
-                       top_k, penalty, recent, n_recent, recent_rows, counts);
-    hipLaunchKernelGGL(topk_final_kernel, dim3(n_rows), dim3(SAMP_THREADS), 0, stream, V, work, temperature, top_k, top_p, min_p,
-                       recent, n_recent, recent_rows, counts, uniform, out);
+                       top_k, top_p, min_p, penalty, recent, n_recent, recent_rows, counts);
+    hipLaunchKernelGGL(topk_final_kernel, dim3(n_rows), dim3(SAMP_THREADS), 0, stream, logits, ld, V, work, temperature, top_k,
+                       top_p, min_p, penalty, recent, n_recent, recent_rows, counts, uniform, out);
   }
   hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMP_THREADS), 0, stream, logits, ld, V, work, temperature, top_k, top_p,
                      min_p, penalty, recent, n_recent, recent_rows, counts, uniform, out, staged);

@@ -621,12 +621,13 @@ def argmax(logits: torch.Tensor, out: torch.Tensor, scratch: Optional[torch.Tens
 def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
            top_p: torch.Tensor, min_p: torch.Tensor, penalty: torch.Tensor, recent: Optional[torch.Tensor],
            uniform: torch.Tensor, out: torch.Tensor, recent_rows: Optional[torch.Tensor] = None,
-           counts: Optional[torch.Tensor] = None, small_top_k: bool = True) -> torch.Tensor:
+           counts: Optional[torch.Tensor] = None, dealt_rows: bool = True) -> torch.Tensor:
     """One token per row of float32 logits, each row with its own options.  work: float32 scratch [rows, vocab].  recent [rows, w]: the row's recent tokens
     (-1 where empty) for the repetition penalty.  With recent_rows [rows] and counts: recent is a table of rings, row
     recent_rows[r] of it belongs to row r and holds its last min(counts, w) tokens; the chosen token is added to it.
-    small_top_k=False: the caller, who has the options on the host, knows that no row has a top-k of 1 to 128; the
-    kernels that deal such rows to several blocks are then not launched (the tokens chosen are the same)."""
+    dealt_rows=False: the caller, who has the options on the host, knows that no row is of a kind that several blocks
+    share over a wide vocabulary (a top-k of 1 to 128, or no top-k, top-p or min-p at all); the kernels for those are
+    then not launched."""
     _need(logits, "logits", torch.float32, 2)
     n, v = logits.shape
     for name, t, dt in (("temperature", temperature, torch.float32), ("top_k", top_k, torch.int32),
@@ -654,6 +655,6 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, 
             raise KernelError("sample: recent_rows has one entry per row of logits, counts one per row of the table")
     _check(_lib("sampling").dlgo_sample(_ptr(logits), _rows(logits, "logits"), n, v, _ptr(work), _ptr(temperature),
                                         _ptr(top_k), _ptr(top_p), _ptr(min_p), _ptr(penalty), _ptr(recent), n_recent,
-                                        _ptr(recent_rows), _ptr(counts), _ptr(uniform), _ptr(out), int(bool(small_top_k)),
+                                        _ptr(recent_rows), _ptr(counts), _ptr(uniform), _ptr(out), int(bool(dealt_rows)),
                                         _stream()))
     return out

@@ -135,10 +135,12 @@ class Sampler:
                 raise ValueError("sampler: keys that start() was never given")
             k[1] = np.asarray(keys, dtype=np.int32)
         fd, kd = self._upload(f, k)
-        small_top_k = any(not c.greedy and 1 <= c.top_k <= 128 for c in configs)     # else two kernels need not be launched
+        # rows that several blocks share: a small top-k, or no cut at all; without one, two kernels need not be launched
+        dealt_rows = any(not c.greedy and (1 <= c.top_k <= 128 or (not 0 < c.top_k < self.vocab and c.top_p >= 1.0 and c.min_p <= 0.0))
+                         for c in configs)
         if rings:       # every choice is recorded, penalty or not: a later row of the request may have one
             ops.sample(logits, self._work, fd[0], kd[0], fd[1], fd[2], fd[3], self._rings, fd[4], out,
-                       recent_rows=kd[1], counts=self._counts, small_top_k=small_top_k)
+                       recent_rows=kd[1], counts=self._counts, dealt_rows=dealt_rows)
             return out
         rec = None
         if recent is not None and penalised:
@@ -147,5 +149,5 @@ class Sampler:
                 toks = list(toks)[-RECENT:]
                 r[i, :len(toks)] = toks
             rec = torch.from_numpy(r).to(self.device)
-        ops.sample(logits, self._work, fd[0], kd[0], fd[1], fd[2], fd[3], rec, fd[4], out, small_top_k=small_top_k)
+        ops.sample(logits, self._work, fd[0], kd[0], fd[1], fd[2], fd[3], rec, fd[4], out, dealt_rows=dealt_rows)
         return out

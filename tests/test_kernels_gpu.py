@@ -991,8 +991,63 @@ def test_sample_wide_rows_dealt_to_several_blocks():
         again = torch.empty_like(out)
         ops.sample(lg, work, col("temp", 1.0, torch.float32), col("top_k", 0, torch.int32), col("top_p", 1.0, torch.float32),
                    col("min_p", 0.0, torch.float32), col("pen", 1.0, torch.float32), rec.to(DEV),
-                   torch.full((n,), u, dtype=torch.float32, device=DEV), again, small_top_k=False)
+                   torch.full((n,), u, dtype=torch.float32, device=DEV), again, dealt_rows=False)
         assert again.tolist() == got, u
+
+
+@pytest.mark.parametrize("v", [20011, 128256])
+def test_sample_whole_rows_from_the_masses_of_their_parts(v):
+    """A wide row that no top-k, top-p or min-p cuts is drawn from by the parts' sums: each part's mass from its own
+    maximum, scaled to the row's, then the piece of 256 that reaches the target, then its elements.  Random rows are
+    compared with the plain pipeline; rows whose mass sits in three far-apart tokens say exactly which token a draw
+    must give: by position in the row (first, middle and last part, the last element of a part, the very last element),
+    with one of them penalised away, and with half the row masked."""
+    import plain_llama as plain
+    ops = _ops()
+    g = torch.Generator().manual_seed(v)
+    per = ((v + 31) // 32 + 3) & ~3                      # a part's elements
+    rows, opts, recents, expect = [], [], [], []
+
+    def add(r, recent=(), expect_by_u=None, **c):
+        rows.append(r)
+        opts.append(c)
+        recents.append(list(recent))
+        expect.append(expect_by_u)
+    add(torch.randn(v, generator=g) * 2, temp=0.8)
+    add(torch.randn(v, generator=g) * 3, temp=1.3, pen=1.5, recent=[7, 7, 100, v - 1])
+    add(torch.randn(v, generator=g) * 2, temp=1.0, top_k=v + 3)            # a top-k that cuts nothing
+    spikes = [5, 17 * per - 1, v - 1]                    # first part; the last element of a part; the last of the row
+    r = torch.randn(v, generator=g) * 0.01 - 30.0
+    r[spikes] = 20.0
+    add(r, temp=1.0, expect_by_u={0.2: spikes[0], 0.5: spikes[1], 0.9: spikes[2], 0.999: spikes[2], 0.001: spikes[0]})
+    add(r.clone(), temp=2.0, pen=4.0, recent=[spikes[1], 3],              # the middle one penalised: 20 -> 5, e^-7.5 of the others
+        expect_by_u={0.2: spikes[0], 0.45: spikes[0], 0.55: spikes[2], 0.9: spikes[2]})
+    r = torch.randn(v, generator=g)
+    r[torch.randperm(v, generator=g)[: v // 2]] = float("-inf")
+    r[per * 9: per * 10] = float("-inf")                 # and a whole part
+    add(r, temp=0.7)
+    n = len(rows)
+    width = max(len(x) for x in recents) or 1
+    rec = torch.full((n, width), -1, dtype=torch.int32)
+    for i, x in enumerate(recents):
+        rec[i, :len(x)] = torch.tensor(x, dtype=torch.int32)
+    lg = torch.stack(rows).to(DEV)
+    col = lambda name, default, dt: torch.tensor([c.get(name, default) for c in opts], dtype=dt, device=DEV)
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    work = torch.empty(n, v, device=DEV)
+    for u in (0.001, 0.2, 0.45, 0.5, 0.55, 0.9, 0.999):
+        ops.sample(lg, work, col("temp", 1.0, torch.float32), col("top_k", 0, torch.int32), col("top_p", 1.0, torch.float32),
+                   col("min_p", 0.0, torch.float32), col("pen", 1.0, torch.float32), rec.to(DEV),
+                   torch.full((n,), u, dtype=torch.float32, device=DEV), out)
+        got = out.tolist()
+        for i, c in enumerate(opts):
+            if expect[i] is not None:
+                if u in expect[i]:
+                    assert got[i] == expect[i][u], (i, c, u)
+                continue
+            want = plain.sample_token(rows[i].double().numpy(), u, c["temp"], c.get("top_k", 0), 1.0, 0.0, c.get("pen", 1.0), recents[i])
+            assert got[i] == want, (i, c, u)
+            assert rows[i][got[i]] > float("-inf")
 
 
 def test_sample_reference_behaviour():
