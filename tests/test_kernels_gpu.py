@@ -1026,6 +1026,12 @@ def test_sample_whole_rows_from_the_masses_of_their_parts(v):
     r[torch.randperm(v, generator=g)[: v // 2]] = float("-inf")
     r[per * 9: per * 10] = float("-inf")                 # and a whole part
     add(r, temp=0.7)
+    # two tokens hold the mass, neighbours in one piece of 256, and the first of them is penalised away: the walk
+    # through the piece has to know that too, or every draw would stop at the first
+    r = torch.randn(v, generator=g) * 0.01 - 30.0
+    near = 5 * per + 300
+    r[[near, near + 3]] = 20.0
+    add(r, temp=2.0, pen=4.0, recent=[11, near], expect_by_u={u: near + 3 for u in (0.001, 0.2, 0.45, 0.5, 0.55, 0.9, 0.999)})
     n = len(rows)
     width = max(len(x) for x in recents) or 1
     rec = torch.full((n, width), -1, dtype=torch.int32)
