@@ -285,10 +285,10 @@ __device__ __forceinline__ void first_bin_reaching(const int* hist, int k, int* 
 // parts' sets, cuts them down the same way against the row's maximum and hands them to sample_small, which makes the
 // exact cuts and the draw.  An element that is missing from a part's set has k larger ones in its own part, so it is
 // below the k-th value of the row: the set that sample_small ends up with is the one sample_kernel would have had.
-// A row that nothing cuts (no top-k, top-p or min-p) goes the same way with sums in place of candidates: see
-// whole_row_draw.  Whatever does not fit (a part with more than TK_CAP elements within its cut, no cut within 255
-// steps, a row with a top-p or min-p cut but no top-k) is left to sample_kernel: the row's scratch says which rows
-// are done.
+// A row that nothing cuts (no top-k, top-p or min-p) goes the same way with sums in place of candidates (see
+// whole_row_draw), and a row whose only cut is min-p with the elements near its parts' maxima as candidates (see
+// min_p_row).  Whatever does not fit (a part with more than TK_CAP elements within its cut, no cut within 255 steps,
+// a row with top-p but no top-k) is left to sample_kernel: the row's scratch says which rows are done.
 // The row's scratch (floats of its row of `work`): maxima [TK_CHUNKS] as (value, index), counts [TK_CHUNKS] (-1: this
 // part gave up), the done flag, then the parts' values [TK_CHUNKS][TK_CAP] and indices [TK_CHUNKS][TK_CAP] (for a row
 // that nothing cuts: counts = the part's pieces of 256, values = their masses).
@@ -312,6 +312,12 @@ __device__ __forceinline__ bool whole_row_draw(float temp, int k, float tp, floa
   return temp > 0.f && (k <= 0 || k >= V) && !(tp < 1.0f) && !(mp > 0.f);
 }
 
+// A row whose only cut is min-p: what stays lies within log(min_p) of the row's maximum, so within that of its
+// part's maximum, and a part can offer those elements as it offers the largest k.
+__device__ __forceinline__ bool min_p_row(float temp, int k, float tp, float mp, int V) {
+  return temp > 0.f && (k <= 0 || k >= V) && !(tp < 1.0f) && mp > 0.f;
+}
+
 __global__ __launch_bounds__(TK_THREADS) void topk_part_kernel(const float* __restrict__ logits, int ld, int V,
                                                                float* __restrict__ work_all,
                                                                const float* __restrict__ temperature,
@@ -332,7 +338,8 @@ __global__ __launch_bounds__(TK_THREADS) void topk_part_kernel(const float* __re
   const float temp = temperature[row];
   const int k = top_k[row];
   const bool whole = whole_row_draw(temp, k, top_p[row], min_p[row], V);
-  if (!whole && (!(temp > 0.f) || k < 1 || k > TK_CAP)) {       // not a row for this way
+  const bool by_min_p = min_p_row(temp, k, top_p[row], min_p[row], V);
+  if (!whole && !by_min_p && (!(temp > 0.f) || k < 1 || k > TK_CAP)) {       // not a row for this way
     if (threadIdx.x == 0) cnt[chunk] = -1;
     return;
   }
@@ -439,6 +446,13 @@ __global__ __launch_bounds__(TK_THREADS) void topk_part_kernel(const float* __re
     }
     return;
   }
+  if (by_min_p && best.v == -INFINITY) {          // a part of nothing but -inf offers nothing
+    if (threadIdx.x == 0) {
+      cnt[chunk] = 0;
+      ((BestIdx*)scratch)[chunk] = best;
+    }
+    return;
+  }
   const uint32_t kmax = order_key(best.v);
   for (int i = c0 + threadIdx.x; i < c1; i += TK_THREADS) {
     const uint32_t bin = (kmax - order_key(xs[i - c0])) >> 16;
@@ -446,11 +460,15 @@ __global__ __launch_bounds__(TK_THREADS) void topk_part_kernel(const float* __re
   }
   __syncthreads();
   if (threadIdx.x < WAVE) {
-    // the distance within which the k largest lie; if they do not lie within 255 steps, everything that does
+    // the distance within which the k largest lie; if they do not lie within 255 steps, everything that does.
+    // A row cut by min-p alone: the part cannot know the cut, which hangs on the row's maximum, so it offers its
+    // largest elements, as many whole steps of distance as TK_CAP elements fill.  What it does not offer is smaller
+    // than all it offers, so topk_final_kernel can tell whether anything that stays may be missing.
     int cum, b;
-    first_bin_reaching(hist, k, &b, &cum);
+    first_bin_reaching(hist, by_min_p ? TK_CAP + 1 : k, &b, &cum);
     if (threadIdx.x == 0) {
-      limit = cum <= TK_CAP ? (b < 255 ? b : 254) : -1;
+      if (by_min_p) limit = b < 255 ? b - 1 : 254;
+      else limit = cum <= TK_CAP ? (b < 255 ? b : 254) : -1;
       n_kept = 0;
     }
   }
@@ -494,7 +512,8 @@ __global__ __launch_bounds__(SAMP_THREADS) void topk_final_kernel(const float* _
   const float temp = temperature[row];
   const int k = top_k[row];
   const bool whole = whole_row_draw(temp, k, top_p[row], min_p[row], V);
-  if (!whole && (!(temp > 0.f) || k < 1 || k > TK_CAP)) return;
+  const bool by_min_p = min_p_row(temp, k, top_p[row], min_p[row], V);
+  if (!whole && !by_min_p && (!(temp > 0.f) || k < 1 || k > TK_CAP)) return;
   __shared__ BestIdx part_top[TK_CHUNKS];
   if (threadIdx.x < TK_CHUNKS) {
     part_n[threadIdx.x] = ((const int*)scratch)[TK_COUNTS + threadIdx.x];
@@ -646,29 +665,57 @@ __global__ __launch_bounds__(SAMP_THREADS) void topk_final_kernel(const float* _
     mine_v[q] = mine[q] ? cv[e] : 0.f;
     mine_i[q] = mine[q] ? ci[e] : 0;
   }
+  if (by_min_p) {
+    // Of what the parts offer, what the cut against the row's maximum leaves (sample_small makes the same cut again),
+    // if sample_small has room for it.  A part's offer is complete above its smallest element: if that one stays too,
+    // smaller ones that the part kept to itself might, and the row is left to sample_kernel.
+    const float cut = top.v + logf(min_p[row]);
+    uint32_t* least = (uint32_t*)hist;                 // the parts' smallest offers, as ordered keys
+    if (threadIdx.x < TK_CHUNKS) least[threadIdx.x] = 0xffffffffu;
+    __syncthreads();
 #pragma unroll
-  for (int q = 0; q < PER; ++q)
-    if (mine[q]) {
-      const uint32_t bin = (kmax - order_key(mine_v[q])) >> 16;
-      if (bin < 255u) atomicAdd(&hist[bin], 1);
+    for (int q = 0; q < PER; ++q)
+      if (mine[q]) atomicMin(&least[(q * SAMP_THREADS + threadIdx.x) / TK_CAP], order_key(mine_v[q]));
+    __syncthreads();
+    bool complete = true;
+    for (int c = 0; c < TK_CHUNKS; ++c) complete = complete && (part_n[c] == 0 || least[c] < order_key(cut));
+    if (!complete) return;
+#pragma unroll
+    for (int q = 0; q < PER; ++q)
+      if (mine[q] && !(mine_v[q] < cut)) {
+        const int slot = atomicAdd(&S.n, 1);
+        if (slot < SAMP_CAND) {
+          S.cv[slot] = mine_v[q];
+          S.ci[slot] = mine_i[q];
+        }
+      }
+    __syncthreads();
+    if (S.n > SAMP_CAND) return;
+  } else {
+#pragma unroll
+    for (int q = 0; q < PER; ++q)
+      if (mine[q]) {
+        const uint32_t bin = (kmax - order_key(mine_v[q])) >> 16;
+        if (bin < 255u) atomicAdd(&hist[bin], 1);
+      }
+    __syncthreads();
+    if (threadIdx.x < WAVE) {
+      int cum, b;
+      first_bin_reaching(hist, k, &b, &cum);
+      if (threadIdx.x == 0) bstar = b < 255 && cum <= SAMP_CAND ? b : -1;
     }
-  __syncthreads();
-  if (threadIdx.x < WAVE) {
-    int cum, b;
-    first_bin_reaching(hist, k, &b, &cum);
-    if (threadIdx.x == 0) bstar = b < 255 && cum <= SAMP_CAND ? b : -1;
+    __syncthreads();
+    if (bstar < 0) return;
+#pragma unroll
+    for (int q = 0; q < PER; ++q)
+      if (mine[q] && ((kmax - order_key(mine_v[q])) >> 16) <= (uint32_t)bstar) {
+        const int slot = atomicAdd(&S.n, 1);
+        S.cv[slot] = mine_v[q];
+        S.ci[slot] = mine_i[q];
+      }
   }
   __syncthreads();
-  if (bstar < 0) return;
-#pragma unroll
-  for (int q = 0; q < PER; ++q)
-    if (mine[q] && ((kmax - order_key(mine_v[q])) >> 16) <= (uint32_t)bstar) {
-      const int slot = atomicAdd(&S.n, 1);
-      S.cv[slot] = mine_v[q];
-      S.ci[slot] = mine_i[q];
-    }
-  __syncthreads();
-  const int pick = sample_small(S, S.n, k, top, top_p[row], min_p[row], uniform[row]);
+  const int pick = sample_small(S, S.n, by_min_p ? 0x7fffffff : k, top, top_p[row], min_p[row], uniform[row]);
   if (threadIdx.x == 0) {
     out[row] = pick;
     const int rr = recent_rows ? recent_rows[row] : row;
@@ -1064,7 +1111,7 @@ extern "C" const char* dlgo_argmax_noalloc(const float* logits, int ld, int n_ro
 }
 
 // work: [n_rows, V] float32 scratch.  dealt_rows: 1 unless the caller knows the rows' options and none is of a kind that
-// several blocks share (a top-k of 1 to 128, or no cut at all); a row is drawn from the same distribution either way,
+// several blocks share (a top-k of 1 to 128, or neither top-k nor top-p); a row is drawn from the same distribution either way,
 // and a row with a top-k gets the same token.  recent: a table of token ids with n_recent columns.  Without counts, row r of
 // it holds row r's recent tokens, -1 where empty.  With recent_rows and counts, row recent_rows[r] of it is a ring of the
 // last tokens chosen for that key, counts[key] the number chosen so far; the kernel adds the token it chooses.

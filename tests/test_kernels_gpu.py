@@ -1056,6 +1056,63 @@ def test_sample_whole_rows_from_the_masses_of_their_parts(v):
             assert rows[i][got[i]] > float("-inf")
 
 
+@pytest.mark.parametrize("v", [20011, 128256])
+def test_sample_rows_cut_by_min_p_alone(v):
+    """A wide row whose only cut is min-p: each part offers what lies within log(min_p) of its own maximum, which
+    holds everything within that of the row's.  Against the plain pipeline: random rows with loose and tight cuts, a
+    row with so loose a cut that the parts give up (the one-block kernel takes it), the survivors all in one part,
+    the largest element penalised below the cut, a masked part; and a row whose survivors are known, one in the first
+    part and one in the last, so that a draw says which."""
+    import plain_llama as plain
+    ops = _ops()
+    g = torch.Generator().manual_seed(v + 1)
+    per = ((v + 31) // 32 + 3) & ~3
+    rows, opts, recents, expect = [], [], [], []
+
+    def add(r, recent=(), expect_by_u=None, **c):
+        rows.append(r)
+        opts.append(c)
+        recents.append(list(recent))
+        expect.append(expect_by_u)
+    add(torch.randn(v, generator=g) * 2, temp=0.8, min_p=0.05)
+    add(torch.randn(v, generator=g) * 2, temp=1.0, min_p=0.5)
+    add(torch.randn(v, generator=g) * 2, temp=1.5, min_p=1e-6)                 # nearly everything stays: too much to offer
+    r = torch.randn(v, generator=g) * 0.5
+    r[3 * per + 10: 3 * per + 90] += 9.0                                       # 80 survivors, all in one part
+    add(r, temp=1.0, min_p=0.01)
+    r = torch.randn(v, generator=g) * 2
+    top = int(r.argmax())
+    add(r, temp=0.7, min_p=0.2, pen=8.0, recent=[top])                         # the maximum falls, the cut with it
+    r = torch.randn(v, generator=g) * 2
+    r[per * 20: per * 21] = float("-inf")
+    add(r, temp=0.9, min_p=0.1, top_k=v)
+    r = torch.randn(v, generator=g) * 0.01 - 30.0
+    r[7] = 20.0
+    r[v - 2] = 20.0 + math.log(3.0)                                            # three times the weight of the other
+    add(r, temp=1.0, min_p=0.1, expect_by_u={0.1: 7, 0.24: 7, 0.26: v - 2, 0.9: v - 2})
+    n = len(rows)
+    width = max(len(x) for x in recents) or 1
+    rec = torch.full((n, width), -1, dtype=torch.int32)
+    for i, x in enumerate(recents):
+        rec[i, :len(x)] = torch.tensor(x, dtype=torch.int32)
+    lg = torch.stack(rows).to(DEV)
+    col = lambda name, default, dt: torch.tensor([c.get(name, default) for c in opts], dtype=dt, device=DEV)
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    work = torch.empty(n, v, device=DEV)
+    for u in (0.003, 0.1, 0.24, 0.26, 0.61, 0.9, 0.997):
+        ops.sample(lg, work, col("temp", 1.0, torch.float32), col("top_k", 0, torch.int32), col("top_p", 1.0, torch.float32),
+                   col("min_p", 0.0, torch.float32), col("pen", 1.0, torch.float32), rec.to(DEV),
+                   torch.full((n,), u, dtype=torch.float32, device=DEV), out)
+        got = out.tolist()
+        for i, c in enumerate(opts):
+            if expect[i] is not None:
+                if u in expect[i]:
+                    assert got[i] == expect[i][u], (i, c, u)
+                continue
+            want = plain.sample_token(rows[i].double().numpy(), u, c["temp"], c.get("top_k", 0), 1.0, c["min_p"], c.get("pen", 1.0), recents[i])
+            assert got[i] == want, (i, c, u)
+
+
 def test_sample_reference_behaviour():
     """ops/sampling_test.go: a dominant logit is always drawn (:18-30); temperature 2 halves the logits (:48-57)."""
     logits = torch.zeros(1, 50)
