@@ -1080,6 +1080,9 @@ def test_sample_rows_cut_by_min_p_alone(v):
     r = torch.randn(v, generator=g) * 0.5
     r[3 * per + 10: 3 * per + 90] += 9.0                                       # 80 survivors, all in one part
     add(r, temp=1.0, min_p=0.01)
+    r = torch.randn(v, generator=g) * 0.5
+    r[6 * per + 10: 6 * per + 310] += 9.0                                      # 300 in one part: more than a part may offer,
+    add(r, temp=1.0, min_p=0.01)                                               # and the row must not be drawn from the 128
     r = torch.randn(v, generator=g) * 2
     top = int(r.argmax())
     add(r, temp=0.7, min_p=0.2, pen=8.0, recent=[top])                         # the maximum falls, the cut with it
