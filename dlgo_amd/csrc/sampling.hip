@@ -864,6 +864,10 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
       if (order_key(work[i]) < tau) work[i] = -INFINITY;
     __syncthreads();
   }
+  // What top-p and min-p cut is not written into the row: the draw, which is all that reads the row after them, leaves
+  // out what lies below the two cuts as it goes (a pass over the row costs one compute unit 11 us and more).
+  uint32_t cut_key = 0u;                 // top-p: elements whose ordered key is below this are out
+  float cut_value = -INFINITY;           // min-p: elements below this are out
   // top-p: smallest set, by falling probability, whose mass reaches p
   if (tp < 1.0f) {
     // The cut is the largest value tau with mass({x >= tau}) >= p * (all the mass).  Masses are exp(x - max) in fixed
@@ -920,18 +924,10 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
       need -= cut_before;
       __syncthreads();
     }
-    const uint32_t tau = kmax - prefix;
-    for (int i = threadIdx.x; i < V; i += SAMP_THREADS)
-      if (order_key(work[i]) < tau) work[i] = -INFINITY;
-    __syncthreads();
+    cut_key = kmax - prefix;
   }
   // min-p: probability below min_p * (largest probability) is masked
-  if (mp > 0.f) {
-    const float cut = top.v + logf(mp);
-    for (int i = threadIdx.x; i < V; i += SAMP_THREADS)
-      if (work[i] < cut) work[i] = -INFINITY;
-    __syncthreads();
-  }
+  if (mp > 0.f) cut_value = top.v + logf(mp);
   // softmax and inverse-CDF draw, cumulative sums in index order.  Each wave owns a run of the row and walks it 256
   // elements at a time (four to a lane), adding them up within the lane and then by a scan over the lanes; the waves'
   // totals, added in wave order, tell which wave holds the target, and that wave walks its run once more, with the
@@ -947,7 +943,8 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
     }
     return x;
   };
-  auto four = [&](int i, float* ev) {   // exp(work - top) of elements i..i+3 of the wave's run, 0 beyond it
+  const bool any_cut = cut_key != 0u || cut_value > -INFINITY;
+  auto four = [&](int i, float* ev) {   // exp(work - top) of elements i..i+3 of the wave's run, 0 beyond it and below the cuts
     float x[4];
     if (vec && i + 3 < w1) {
       const float4 v4 = *(const float4*)(work + i);
@@ -955,6 +952,11 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
     } else {
 #pragma unroll
       for (int c = 0; c < 4; ++c) x[c] = i + c < w1 ? work[i + c] : -INFINITY;
+    }
+    if (any_cut) {
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        if (order_key(x[c]) < cut_key || x[c] < cut_value) x[c] = -INFINITY;
     }
 #pragma unroll
     for (int c = 0; c < 4; ++c) ev[c] = expf(x[c] - top.v);
