@@ -136,27 +136,53 @@ __global__ __launch_bounds__(WAVE) void argmax_final_kernel(const BestIdx* __res
   if (threadIdx.x == 0) out[blockIdx.x] = best.i < 0 ? 0 : best.i;
 }
 
-// Largest key tau with |{i : key_i >= tau}| >= need, by bisection on the key's bits (top-k).
-__device__ uint32_t bisect_threshold(const float* work, int V, float need, float* red, bool vec = false) {
-  uint32_t prefix = 0;
-  for (int bit = 31; bit >= 0; --bit) {
-    const uint32_t cand = prefix | (1u << bit);
-    float part = 0.f;
-    if (vec) {
-#pragma unroll 4
-      for (int i = threadIdx.x; i < V / 4; i += SAMP_THREADS) {
-        const float4 w4 = ((const float4*)work)[i];
-        if (order_key(w4.x) >= cand) part += 1.0f;
-        if (order_key(w4.y) >= cand) part += 1.0f;
-        if (order_key(w4.z) >= cand) part += 1.0f;
-        if (order_key(w4.w) >= cand) part += 1.0f;
+// Largest key tau with |{i : key_i >= tau}| >= need (top-k), found 11, 11 and 10 bits of the key at a time, each time
+// from a count of the elements by those bits: three passes over the row.  hist: 2048 ints of LDS; at: two ints of LDS.
+// Called by the whole block.
+__device__ uint32_t radix_threshold(const float* work, int V, int need, int* hist, int* at, bool vec) {
+  uint32_t prefix = 0;              // the key's upper bits, as far as they are known
+  for (int level = 0; level < 3; ++level) {
+    const int shift = level == 0 ? 21 : (level == 1 ? 10 : 0), bits = level == 2 ? 10 : 11;
+    for (int b = threadIdx.x; b < 2048; b += SAMP_THREADS) hist[b] = 0;
+    __syncthreads();
+    for_each_element(work, V, vec, [&](int, float x) {
+      const uint32_t key = order_key(x);
+      if (level == 0 || (key >> (shift + bits)) == prefix) atomicAdd(&hist[(key >> shift) & ((1u << bits) - 1u)], 1);
+    });
+    __syncthreads();
+    if (threadIdx.x < WAVE) {
+      // the highest bin from which upwards `need` elements lie: a lane adds up 32 neighbouring bins, the lanes are
+      // added from the top, and the lane in whose bins the count is reached walks them down
+      const int lane = threadIdx.x;
+      int mine = 0;
+      for (int q = 0; q < 32; ++q) mine += hist[32 * lane + q];
+      int from_top = mine;          // this lane's bins and all above
+#pragma unroll
+      for (int o = 1; o < WAVE; o <<= 1) {
+        const int y = __shfl_down(from_top, o, WAVE);
+        if (lane + o < WAVE) from_top += y;
       }
-    } else {
-      for (int i = threadIdx.x; i < V; i += SAMP_THREADS)
-        if (order_key(work[i]) >= cand) part += 1.0f;
+      const unsigned long long reached = __ballot(from_top >= need);
+      // (not reached at all: fewer elements than asked for share the prefix, which cannot be: the level above counted
+      // them; at the first level it means fewer than `need` elements in the row, and every element stays)
+      const int owner = reached ? 63 - __clzll(reached) : 0;
+      if (lane == owner) {
+        int above = from_top - mine, bin = 32 * lane;
+        for (int q = 31; q >= 0; --q) {
+          if (above + hist[32 * lane + q] >= need || q == 0) {
+            bin = 32 * lane + q;
+            break;
+          }
+          above += hist[32 * lane + q];
+        }
+        at[0] = bin;
+        at[1] = above;
+      }
     }
-    const float total = block_sum_f(part, red);
-    if (total >= need) prefix = cand;
+    __syncthreads();
+    prefix = (prefix << bits) | (uint32_t)at[0];
+    need -= at[1];
+    __syncthreads();
   }
   return prefix;
 }
@@ -287,8 +313,9 @@ __device__ __forceinline__ void first_bin_reaching(const int* hist, int k, int* 
 // below the k-th value of the row: the set that sample_small ends up with is the one sample_kernel would have had.
 // A row that nothing cuts (no top-k, top-p or min-p) goes the same way with sums in place of candidates (see
 // whole_row_draw), and a row whose only cut is min-p with the elements near its parts' maxima as candidates (see
-// min_p_row).  Whatever does not fit (a part with more than TK_CAP elements within its cut, no cut within 255 steps,
-// a row with top-p but no top-k) is left to sample_kernel: the row's scratch says which rows are done.
+// min_p_row), as has a row with a top-k between TK_CAP and SAMP_CAND (see large_top_k).  Whatever does not fit (a part
+// with more than TK_CAP elements within its cut, no cut within 255 steps, a row with top-p but no top-k, a larger
+// top-k still) is left to sample_kernel: the row's scratch says which rows are done.
 // The row's scratch (floats of its row of `work`): maxima [TK_CHUNKS] as (value, index), counts [TK_CHUNKS] (-1: this
 // part gave up), the done flag, then the parts' values [TK_CHUNKS][TK_CAP] and indices [TK_CHUNKS][TK_CAP] (for a row
 // that nothing cuts: counts = the part's pieces of 256, values = their masses).
@@ -318,6 +345,11 @@ __device__ __forceinline__ bool min_p_row(float temp, int k, float tp, float mp,
   return temp > 0.f && (k <= 0 || k >= V) && !(tp < 1.0f) && mp > 0.f;
 }
 
+// A top-k of more than TK_CAP and at most SAMP_CAND: a part cannot offer its largest k, but it can offer its largest
+// TK_CAP as for min_p_row, and topk_final_kernel can tell whether the row's largest k lie among what it was offered
+// (each part's smallest offer falls below them).
+__device__ __forceinline__ bool large_top_k(float temp, int k, int V) { return temp > 0.f && k > TK_CAP && k <= SAMP_CAND && k < V; }
+
 __global__ __launch_bounds__(TK_THREADS) void topk_part_kernel(const float* __restrict__ logits, int ld, int V,
                                                                float* __restrict__ work_all,
                                                                const float* __restrict__ temperature,
@@ -338,7 +370,8 @@ __global__ __launch_bounds__(TK_THREADS) void topk_part_kernel(const float* __re
   const float temp = temperature[row];
   const int k = top_k[row];
   const bool whole = whole_row_draw(temp, k, top_p[row], min_p[row], V);
-  const bool by_min_p = min_p_row(temp, k, top_p[row], min_p[row], V);
+  // (the part's largest elements are what it offers of a row cut by min-p alone and of a row with a large top-k)
+  const bool by_min_p = min_p_row(temp, k, top_p[row], min_p[row], V) || large_top_k(temp, k, V);
   if (!whole && !by_min_p && (!(temp > 0.f) || k < 1 || k > TK_CAP)) {       // not a row for this way
     if (threadIdx.x == 0) cnt[chunk] = -1;
     return;
@@ -513,8 +546,11 @@ __global__ __launch_bounds__(SAMP_THREADS) void topk_final_kernel(const float* _
   const int k = top_k[row];
   const bool whole = whole_row_draw(temp, k, top_p[row], min_p[row], V);
   const bool by_min_p = min_p_row(temp, k, top_p[row], min_p[row], V);
-  if (!whole && !by_min_p && (!(temp > 0.f) || k < 1 || k > TK_CAP)) return;
+  const bool big_k = large_top_k(temp, k, V);
+  if (!whole && !by_min_p && !big_k && (!(temp > 0.f) || k < 1 || k > TK_CAP)) return;
   __shared__ BestIdx part_top[TK_CHUNKS];
+  __shared__ uint32_t least[TK_CHUNKS];             // the parts' smallest offers, as ordered keys
+  if (threadIdx.x < TK_CHUNKS) least[threadIdx.x] = 0xffffffffu;
   if (threadIdx.x < TK_CHUNKS) {
     part_n[threadIdx.x] = ((const int*)scratch)[TK_COUNTS + threadIdx.x];
     part_top[threadIdx.x] = ((const BestIdx*)scratch)[threadIdx.x];
@@ -670,9 +706,6 @@ __global__ __launch_bounds__(SAMP_THREADS) void topk_final_kernel(const float* _
     // if sample_small has room for it.  A part's offer is complete above its smallest element: if that one stays too,
     // smaller ones that the part kept to itself might, and the row is left to sample_kernel.
     const float cut = top.v + logf(min_p[row]);
-    uint32_t* least = (uint32_t*)hist;                 // the parts' smallest offers, as ordered keys
-    if (threadIdx.x < TK_CHUNKS) least[threadIdx.x] = 0xffffffffu;
-    __syncthreads();
 #pragma unroll
     for (int q = 0; q < PER; ++q)
       if (mine[q]) atomicMin(&least[(q * SAMP_THREADS + threadIdx.x) / TK_CAP], order_key(mine_v[q]));
@@ -697,6 +730,7 @@ __global__ __launch_bounds__(SAMP_THREADS) void topk_final_kernel(const float* _
       if (mine[q]) {
         const uint32_t bin = (kmax - order_key(mine_v[q])) >> 16;
         if (bin < 255u) atomicAdd(&hist[bin], 1);
+        if (big_k) atomicMin(&least[(q * SAMP_THREADS + threadIdx.x) / TK_CAP], order_key(mine_v[q]));
       }
     __syncthreads();
     if (threadIdx.x < WAVE) {
@@ -706,6 +740,13 @@ __global__ __launch_bounds__(SAMP_THREADS) void topk_final_kernel(const float* _
     }
     __syncthreads();
     if (bstar < 0) return;
+    if (big_k) {
+      // the parts offered their largest TK_CAP, not their largest k: everything within the cut's distance is here only
+      // if each part's smallest offer lies farther from the maximum than that
+      bool complete = true;
+      for (int c = 0; c < TK_CHUNKS; ++c) complete = complete && (part_n[c] == 0 || ((kmax - least[c]) >> 16) > (uint32_t)bstar);
+      if (!complete) return;
+    }
 #pragma unroll
     for (int q = 0; q < PER; ++q)
       if (mine[q] && ((kmax - order_key(mine_v[q])) >> 16) <= (uint32_t)bstar) {
@@ -858,8 +899,9 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
       if (threadIdx.x == 0) finish(pick);
       return;
     }
-    // many equal values at the cut, or the k-th value far below the maximum: the cut by bisection over the whole row
-    const uint32_t tau = bisect_threshold(work, V, (float)k, red, vec);
+    // many equal values at the cut, or the k-th value far below the maximum: the cut from counts over the whole row
+    __shared__ int cut_at[2];
+    const uint32_t tau = radix_threshold(work, V, k, (int*)S.sv, cut_at, vec);
     for (int i = threadIdx.x; i < V; i += SAMP_THREADS)
       if (order_key(work[i]) < tau) work[i] = -INFINITY;
     __syncthreads();
@@ -1113,7 +1155,7 @@ extern "C" const char* dlgo_argmax_noalloc(const float* logits, int ld, int n_ro
 }
 
 // work: [n_rows, V] float32 scratch.  dealt_rows: 1 unless the caller knows the rows' options and none is of a kind that
-// several blocks share (a top-k of 1 to 128, or neither top-k nor top-p); a row is drawn from the same distribution either way,
+// several blocks share (a top-k of 1 to 1,024, or neither top-k nor top-p); a row is drawn from the same distribution either way,
 // and a row with a top-k gets the same token.  recent: a table of token ids with n_recent columns.  Without counts, row r of
 // it holds row r's recent tokens, -1 where empty.  With recent_rows and counts, row recent_rows[r] of it is a ring of the
 // last tokens chosen for that key, counts[key] the number chosen so far; the kernel adds the token it chooses.

@@ -626,7 +626,7 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, 
     (-1 where empty) for the repetition penalty.  With recent_rows [rows] and counts: recent is a table of rings, row
     recent_rows[r] of it belongs to row r and holds its last min(counts, w) tokens; the chosen token is added to it.
     dealt_rows=False: the caller, who has the options on the host, knows that no row is of a kind that several blocks
-    share over a wide vocabulary (a top-k of 1 to 128, or neither top-k nor top-p); the kernels for those are
+    share over a wide vocabulary (a top-k of 1 to 1,024, or neither top-k nor top-p); the kernels for those are
     then not launched."""
     _need(logits, "logits", torch.float32, 2)
     n, v = logits.shape

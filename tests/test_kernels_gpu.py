@@ -965,6 +965,14 @@ def test_sample_wide_rows_dealt_to_several_blocks():
     add(torch.randn(v, generator=g) * 3, temp=0.0, top_k=40)
     add(torch.randn(v, generator=g) * 3, temp=1.2, top_k=128, min_p=0.01)
     add(torch.randn(v, generator=g) * 3, temp=1.2, top_k=129, top_p=0.99)
+    # a top-k beyond what a part may offer: the parts offer their largest 128 and the last block checks that the row's
+    # largest k are among them; they are not where one part holds 300 of the largest 400, and not beyond 1,024
+    add(torch.randn(v, generator=g) * 3, temp=0.9, top_k=500)
+    add(torch.randn(v, generator=g) * 3, temp=1.0, top_k=1000, min_p=0.001)
+    add(torch.randn(v, generator=g) * 3, temp=1.0, top_k=1025)
+    r = torch.randn(v, generator=g)
+    r[4008 * 7 + 5: 4008 * 7 + 305] += 8.0
+    add(r, temp=1.5, top_k=400)
     r = torch.randn(v, generator=g) * 2
     top = int(r.argmax())
     add(r, temp=0.5, top_k=3, pen=4.0, recent=[top, int(r.topk(2).indices[1])])
