@@ -81,16 +81,6 @@ __device__ BestIdx block_argmax(const float* row, int V, BestIdx* red, bool vec 
   return block_best(best, red);
 }
 
-__device__ float block_sum_f(float v, float* red) {
-  v = wave_sum(v);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
-  __syncthreads();
-  float t = 0.f;
-  for (int w = 0; w < SAMP_WAVES; ++w) t += red[w];
-  return t;
-}
-
 // argmax in two stages, so that a few rows still fill the chip: ARGMAX_CHUNKS blocks per row each find the
 // best of their part of the row, then one wave per row picks among them (larger value, then smaller index).
 #define ARGMAX_CHUNKS 64
@@ -778,7 +768,6 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
                                                               const float* __restrict__ uniform, int32_t* __restrict__ out,
                                                               int staged) {
   __shared__ BestIdx redb[SAMP_WAVES];
-  __shared__ float red[SAMP_WAVES];
   __shared__ SampleSmall S;
   __shared__ int hist[256];
   __shared__ int chosen, bstar, cut_bin, again;
