@@ -135,7 +135,8 @@ class Sampler:
                 raise ValueError("sampler: keys that start() was never given")
             k[1] = np.asarray(keys, dtype=np.int32)
         fd, kd = self._upload(f, k)
-        # rows that several blocks share: a top-k of up to 1,024, or neither top-k nor top-p; without one, two kernels need not be launched
+        # rows that several blocks share: a top-k of up to 1,024, or neither top-k nor top-p; without one, two kernels need not be
+        # launched (a hint only: which rows those kernels take they decide themselves, from the options on the device)
         dealt_rows = any(not c.greedy and (1 <= c.top_k <= 1024 or (not 0 < c.top_k < self.vocab and c.top_p >= 1.0))
                          for c in configs)
         if rings:       # every choice is recorded, penalty or not: a later row of the request may have one
