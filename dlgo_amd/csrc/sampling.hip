@@ -779,7 +779,7 @@ __global__ __launch_bounds__(SAMP_THREADS) void sample_kernel(const float* __res
   const float* lg = logits + (size_t)row * ld;
   const float temp = temperature[row];
   if (!(temp > 0.f)) {   // greedy row
-    const BestIdx b = block_argmax(lg, V, redb);
+    const BestIdx b = block_argmax(lg, V, redb, (V & 3) == 0 && (ld & 3) == 0 && ((uintptr_t)logits & 15) == 0);
     if (threadIdx.x == 0) out[row] = b.i < 0 ? 0 : b.i;
     return;
   }
