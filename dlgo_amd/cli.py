@@ -36,6 +36,8 @@ def main(argv=None) -> int:
     ap.add_argument("--write-random", metavar="CONFIG_JSON",
                     help="write a model folder with random weights for this config.json into MODEL_DIR, then exit")
     ap.add_argument("--weight-seed", type=int, default=0, help="seed of --write-random")
+    ap.add_argument("--weight-std", type=float, default=None,
+                    help="standard deviation of --write-random's matrices (default: the configuration's initializer_range)")
     ap.add_argument("--info", action="store_true", help="print the model's description and exit")
     args = ap.parse_args(argv)
     if args.model is None:
@@ -54,7 +56,11 @@ def main(argv=None) -> int:
         from . import models  # noqa: F401
         from .config import load_config
         from .weights import write_random_model
-        write_random_model(load_config(args.write_random), args.weight_seed, args.model)
+        try:
+            write_random_model(load_config(args.write_random), args.weight_seed, args.model, std=args.weight_std)
+        except Exception as e:
+            print(f"Error writing model: {e}" + (" (--weight-std)" if "initializer_range" in str(e) else ""), file=sys.stderr)
+            return 1
         print(f"wrote {args.model}")
         return 0
 

@@ -491,6 +491,21 @@ def test_command_line_checks_like_the_reference(capsys):
     assert main(["--temp", "-0.1", "x"]) == 1 and "--temp must be >= 0" in capsys.readouterr().err
 
 
+def test_command_line_writes_a_random_model_or_says_why_not(tmp_path, capsys):
+    import json
+    from conftest import TINY_A
+    from dlgo_amd.cli import main
+    from dlgo_amd.config import load_config
+    raw = {k: v for k, v in TINY_A.items() if k != "initializer_range"}
+    (tmp_path / "c.json").write_text(json.dumps(raw))
+    out = str(tmp_path / "m")
+    assert main(["--write-random", str(tmp_path / "c.json"), out]) == 1
+    assert "initializer_range" in capsys.readouterr().err          # no width of the weights in the file: one line, no traceback
+    assert main(["--write-random", str(tmp_path / "c.json"), out, "--weight-std", "0.05", "--weight-seed", "3"]) == 0
+    assert load_config(out).hidden_size == raw["hidden_size"] and (tmp_path / "m" / "model.safetensors").exists()
+    assert main(["--write-random", str(tmp_path / "nope.json"), out]) == 1 and "no such file" in capsys.readouterr().err
+
+
 def test_engine_refuses_to_run_without_a_gpu(tmp_path):
     if torch.cuda.is_available():
         pytest.skip("a GPU is present")
