@@ -64,10 +64,14 @@ def main(argv=None) -> int:
         print(f"wrote {args.model}")
         return 0
 
-    prompts = [_ids(p) for p in args.prompt_ids]
-    if args.prompts_file:
-        with open(args.prompts_file) as f:
-            prompts += [_ids(line) for line in f if line.strip()]
+    try:
+        prompts = [_ids(p) for p in args.prompt_ids]
+        if args.prompts_file:
+            with open(args.prompts_file) as f:
+                prompts += [_ids(line) for line in f if line.strip()]
+    except (OSError, ValueError) as e:
+        print(f"Error reading prompts (token ids separated by commas or spaces): {e}", file=sys.stderr)
+        return 1
     from . import (with_greedy, with_ignore_eos, with_max_tokens, with_min_p, with_repetition_penalty, with_seed,
                    with_temperature, with_top_k, with_top_p)
     from .api import load_llm
@@ -88,7 +92,11 @@ def main(argv=None) -> int:
         opts.append(with_greedy())
     if args.ignore_eos:
         opts.append(with_ignore_eos())
-    results = llm.generate(prompts, *opts)
+    try:
+        results = llm.generate(prompts, *opts)
+    except Exception as e:
+        print(f"Error generating: {e}", file=sys.stderr)
+        return 1
     for i, r in enumerate(results):
         print(json.dumps({"request": i, "tokens": r.tokens, "finish_reason": r.finish_reason}))
     print(f"[{results[0]}]")

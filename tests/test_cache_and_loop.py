@@ -489,6 +489,8 @@ def test_command_line_checks_like_the_reference(capsys):
     assert main(["--ctx", "0", "x"]) == 1 and "--ctx must be > 0" in capsys.readouterr().err
     assert main(["--max-tokens", "0", "x"]) == 1 and "--max-tokens must be > 0" in capsys.readouterr().err
     assert main(["--temp", "-0.1", "x"]) == 1 and "--temp must be >= 0" in capsys.readouterr().err
+    assert main(["x", "--prompt-ids", "1,b,3"]) == 1 and "Error reading prompts" in capsys.readouterr().err
+    assert main(["x", "--prompts-file", "/nonexistent/prompts.txt"]) == 1 and "Error reading prompts" in capsys.readouterr().err
 
 
 def test_command_line_writes_a_random_model_or_says_why_not(tmp_path, capsys):
