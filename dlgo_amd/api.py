@@ -6,6 +6,7 @@ tokenizers and chat templates are not part of this library.
 """
 from __future__ import annotations
 
+import operator
 from dataclasses import dataclass
 from typing import Callable, List, Optional, Sequence, Union
 
@@ -15,7 +16,7 @@ from .cache import PAGE, tokens_that_fit
 from .config import ModelConfig, build_model, load_config
 from .engine.engine import Engine, EngineError, run_dtype
 from .weights import load_weights
-from .engine.generate import Result, Stats, generate
+from .engine.generate import GenerationError, Result, Stats, generate
 from .sampling import GenerateConfig, Option, Sampler, apply_options
 
 Prompt = Sequence[int]
@@ -51,6 +52,22 @@ class BenchmarkResult:
     step_ms: List[float]
 
 
+def _is_id(x) -> bool:
+    """An integer of any kind (Python's, numpy's, an element of an integer tensor), not a float and not a sequence."""
+    try:
+        operator.index(x)
+        return True
+    except TypeError:
+        return False
+
+
+def _ids(prompt, i: int) -> List[int]:
+    try:
+        return [operator.index(t) for t in prompt]
+    except TypeError:
+        raise GenerationError(f"request {i}: a prompt is a sequence of integer token ids") from None
+
+
 class LLM:
     def __init__(self, engine: Engine, max_batch: int = 64):
         self.engine = engine
@@ -62,6 +79,7 @@ class LLM:
         self.stop_tokens = tuple(eos)
 
     def _run(self, prompts: Sequence[Prompt], opts: Sequence[Option], on_token=None):
+        prompts = [_ids(p, i) for i, p in enumerate(prompts)]
         cfg = apply_options(opts)
         results, stats = generate(self.engine, self.sampler, prompts, [cfg] * len(prompts), self.stop_tokens, on_token,
                                   self.max_batch, sync=torch.cuda.synchronize)
@@ -75,7 +93,7 @@ class LLM:
     def generate(self, prompt: Union[Prompt, Sequence[Prompt]], *opts: Option):
         """One prompt (a list of token ids) -> GenerateResult; a list of prompts -> a list of them, run as
         batches of unequal lengths."""
-        many = len(prompt) > 0 and not isinstance(prompt[0], int)
+        many = len(prompt) > 0 and not _is_id(prompt[0])
         prompts = list(prompt) if many else [prompt]
         results, stats = self._run(prompts, opts)
         out = [self._wrap(r, stats) for r in results]

@@ -483,6 +483,18 @@ def test_options_have_the_reference_defaults_and_meanings():
     assert dlgo_amd.WithMaxTokens is dlgo_amd.with_max_tokens and dlgo_amd.LoadLLM is dlgo_amd.load_llm
 
 
+def test_prompts_are_integer_token_ids():
+    """The entry point takes ids of any integer kind and tells one prompt from a list of prompts by its first element;
+    floats and text are refused rather than cut down to integers."""
+    from dlgo_amd.api import _ids, _is_id
+    assert _ids([1, np.int64(2), torch.tensor(3)], 0) == [1, 2, 3] and _ids(np.array([4, 5]), 0) == [4, 5]
+    assert _is_id(7) and _is_id(np.int32(7)) and _is_id(torch.tensor([7, 8])[0])
+    assert not _is_id([7]) and not _is_id(7.0) and not _is_id("7")
+    for bad in ([1.5, 2.0], "hello", [[1, 2]], [None]):
+        with pytest.raises(GenerationError, match="request 3: a prompt is a sequence of integer token ids"):
+            _ids(bad, 3)
+
+
 def test_command_line_checks_like_the_reference(capsys):
     """examples/simple_chat/main.go:28-39."""
     from dlgo_amd.cli import main
