@@ -8,14 +8,14 @@ from __future__ import annotations
 
 import operator
 from dataclasses import dataclass
-from typing import Callable, List, Optional, Sequence, Union
+from typing import Callable, List, Mapping, Optional, Sequence, Union
 
 import torch
 
 from .cache import PAGE, tokens_that_fit
-from .config import ModelConfig, build_model, load_config
-from .engine.engine import Engine, EngineError, run_dtype
-from .weights import load_weights
+from .config import ModelConfig, build_model, config_from_dict, load_config
+from .engine.engine import Engine, EngineError, recordings_bytes, run_dtype
+from .weights import load_state, load_weights, random_tensors
 from .engine.generate import GenerationError, Result, Stats, generate
 from .sampling import GenerateConfig, Option, Sampler, apply_options
 
@@ -75,8 +75,7 @@ class LLM:
         self.max_seq_len = engine.max_ctx
         self.max_batch = max_batch
         self.sampler = Sampler(engine.vocab, engine.device, max_rows=max_batch)
-        eos = getattr(self.config, "eos_token_ids", ())
-        self.stop_tokens = tuple(eos)
+        self.stop_tokens = tuple(self.config.stop_tokens())
 
     def _run(self, prompts: Sequence[Prompt], opts: Sequence[Option], on_token=None):
         prompts = [_ids(p, i) for i, p in enumerate(prompts)]
@@ -117,32 +116,45 @@ class LLM:
 
     def model_info(self) -> str:
         """dlgo.go:170-185."""
-        c = self.config
-        g = lambda k: getattr(c, k, "?")
-        return (f"{c.architecture} | {g('num_hidden_layers')} layers | {g('hidden_size')} dim | "
-                f"{g('num_attention_heads')} heads ({g('num_key_value_heads')} KV) | {g('intermediate_size')} FFN | "
-                f"vocab {g('vocab_size')} | ctx {self.max_seq_len} | {str(self.engine.dtype).replace('torch.', '')}")
+        return " | ".join([self.config.architecture, *self.config.describe(), f"ctx {self.max_seq_len}",
+                           str(self.engine.dtype).replace('torch.', '')])
 
 
-def load_llm(path: str, max_seq_len: int = 0, dtype: str = "bfloat16", device: str = "cuda:0", max_batch: int = 64,
-             max_tokens: Optional[int] = None, **engine_options) -> LLM:
-    """Load a model folder (config.json, model.safetensors).  max_seq_len <= 0 or beyond the model's
-    context means the model's context (models/llm/generate.go:56-58).  The cache is sized for
-    `max_tokens` tokens over all live sequences; by default for max_batch sequences of max_seq_len, or for as many
-    tokens as the device's free memory holds once the weights are loaded (a fifth of it stays free), if that is less."""
-    config = load_config(path)
-    limit = getattr(config, "max_position_embeddings", None)
+def load_llm(model: Union[str, ModelConfig, Mapping], max_seq_len: int = 0, dtype: str = "bfloat16", device: str = "cuda:0",
+             max_batch: int = 64, max_tokens: Optional[int] = None, random_seed: Optional[int] = None,
+             random_std: Optional[float] = None, **engine_options) -> LLM:
+    """Load a model folder (config.json, model.safetensors), as dlgo.go:37-47 loads a file.  With `random_seed` the
+    weights are drawn for that seed instead of read, and `model` may then also be a config.json file, its contents as
+    a mapping, or a configuration object: nothing is written (a folder given with a seed lends its config.json only).
+    max_seq_len <= 0 or beyond the model's context means the model's context (models/llm/generate.go:56-58).  The
+    cache is sized for `max_tokens` tokens over all live sequences; by default for max_batch sequences of max_seq_len,
+    or for as many tokens as the device's free memory holds once the weights are loaded (a fifth of it stays free,
+    and room for the recordings of steps), if that is less."""
+    if isinstance(model, ModelConfig):
+        config = model
+    elif isinstance(model, Mapping):
+        config = config_from_dict(model)
+    else:
+        config = load_config(model)
+    if random_seed is None and not isinstance(model, str):
+        raise EngineError("load_llm: a configuration without a model folder needs random_seed (there are no weights to read)")
+    limit = config.context_length()
     ctx = max_seq_len if max_seq_len > 0 and (limit is None or max_seq_len <= limit) else limit
     if not torch.cuda.is_available():
         raise EngineError("no HIP device: dlgo_amd runs on an AMD GPU only and has no CPU path")
     rd = run_dtype(dtype)
-    model = build_model(config)
-    load_weights(model, path, device, rd)
+    built = build_model(config)
+    if random_seed is None:
+        load_weights(built, model, device, rd)
+    else:
+        tensors = random_tensors(config, random_seed, rd, random_std, device=device)
+        load_state(built, tensors, device, rd, where="random weights")
+        del tensors
     if max_tokens is None:
         free, _ = torch.cuda.mem_get_info(torch.device(device))
-        fit = tokens_that_fit(model.unit_needs, rd, free)
+        fit = tokens_that_fit(built.unit_needs, rd, free, recordings_bytes(built.vocab, max_batch, **engine_options))
         if fit < PAGE:
             raise EngineError(f"no device memory left for a cache ({free >> 20} MiB free after the weights)")
-        max_tokens = min(max_batch * ctx, fit)
-    engine = Engine(model, rd, device, max_tokens=max_tokens, max_ctx=ctx, **engine_options)
+        max_tokens = fit if ctx is None else min(max_batch * ctx, fit)
+    engine = Engine(built, rd, device, max_tokens=max_tokens, max_ctx=ctx, **engine_options)
     return LLM(engine, max_batch)

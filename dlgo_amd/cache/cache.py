@@ -222,8 +222,21 @@ class Cache:
                 g.table_host[dst, i] = p
             g.dirty.add(dst)
             by_page = g.storage.view(g.pool.n_pages, g.page_stride)
-            by_page[torch.as_tensor(pages, dtype=torch.int64, device=self.device)] = \
-                by_page[torch.as_tensor(src_pages, dtype=torch.int64, device=self.device)]
+            if self.device.type != "cuda":
+                by_page[torch.as_tensor(pages, dtype=torch.int64)] = by_page[torch.as_tensor(src_pages, dtype=torch.int64)]
+                continue
+            # the page numbers travel as the changed table rows do (pinned, in a copy that nothing waits for); the pages
+            # are copied by the library's own kernel
+            from ..kernels import ops
+            k = len(pages)
+            st = self._table_stage(2 * k)
+            st[0].numpy()[:k] = src_pages
+            st[0].numpy()[k:2 * k] = pages
+            st[2][:2 * k].copy_(st[0][:2 * k], non_blocking=True)
+            ops.copy_rows(by_page, by_page, src_rows=st[2][:k], dst_rows=st[2][k:2 * k], n=k)
+            ev = torch.cuda.Event()
+            ev.record()
+            st[4] = ev
         self.lengths[dst] = n
         for t in self.state.values():
             t[dst].copy_(t[src])
@@ -327,9 +340,9 @@ class Cache:
             st[4].synchronize()
         if st is None or st[0].shape[0] < n_rows:
             cap = max(2 * n_rows, 64)
-            st = [torch.empty(cap, dtype=torch.int64, pin_memory=True),
+            st = [torch.empty(cap, dtype=torch.int32, pin_memory=True),
                   torch.empty((cap, self.max_pages_per_seq), dtype=torch.int32, pin_memory=True),
-                  torch.empty(cap, dtype=torch.int64, device=self.device),
+                  torch.empty(cap, dtype=torch.int32, device=self.device),
                   torch.empty((cap, self.max_pages_per_seq), dtype=torch.int32, device=self.device), None]
             self._stages[i] = st
         return st
@@ -352,7 +365,8 @@ class Cache:
             st[1].numpy()[:n] = g.table_host[rows]
             st[2][:n].copy_(st[0][:n], non_blocking=True)
             st[3][:n].copy_(st[1][:n], non_blocking=True)
-            g.table.index_copy_(0, st[2][:n], st[3][:n])
+            from ..kernels import ops
+            ops.copy_rows(st[3], g.table, dst_rows=st[2], n=n)        # table[rows[i]] = the staged row i
             ev = torch.cuda.Event()
             ev.record()
             st[4] = ev
@@ -394,12 +408,13 @@ def kv_bytes_per_token(unit_needs: Sequence[Sequence[CacheNeed]], dtype: torch.d
     return sum(2 * need.kv_heads * need.head_dim * item for needs in unit_needs for need in needs if need.kind == "kv")
 
 
-def tokens_that_fit(unit_needs: Sequence[Sequence[CacheNeed]], dtype: torch.dtype, free_bytes: int, keep_free: float = 0.2,
-                    reserve_bytes: int = 2 << 30) -> int:
+def tokens_that_fit(unit_needs: Sequence[Sequence[CacheNeed]], dtype: torch.dtype, free_bytes: int, recordings_bytes: int = 0,
+                    keep_free: float = 0.2, reserve_bytes: int = 2 << 30) -> int:
     """How many tokens (a whole number of pages) a cache may be sized for when `free_bytes` of device memory are left:
-    a fifth of it and 2 GiB stay free for the step's buffers and the logits."""
+    a fifth of it and 2 GiB stay free for the step's buffers, and `recordings_bytes` for what the recordings of steps
+    will keep (they do not exist yet when the cache is sized)."""
     per_token = kv_bytes_per_token(unit_needs, dtype)
-    budget = int(free_bytes * (1.0 - keep_free)) - reserve_bytes
+    budget = int(free_bytes * (1.0 - keep_free)) - reserve_bytes - int(recordings_bytes)
     if per_token == 0:
         return 1 << 20
     return max(0, budget // (per_token * PAGE)) * PAGE

@@ -4,6 +4,7 @@ path as the positional argument, each checked the same way (> 0, > 0, >= 0).  Pr
 are token ids, since tokenizers are not part of this library.
 
     python -m dlgo_amd [--ctx N] [--max-tokens N] [--temp T] [--prompt-ids 1,2,3 ...] MODEL_DIR
+    python -m dlgo_amd --random-config CONFIG_JSON [--weight-seed S] [...]        (weights drawn for the seed, nothing read or written)
 """
 from __future__ import annotations
 
@@ -33,15 +34,19 @@ def main(argv=None) -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--prompt-ids", action="append", default=[], help="a prompt as token ids, e.g. 1,15,27 (repeatable)")
     ap.add_argument("--prompts-file", help="a file with one prompt of token ids per line")
+    ap.add_argument("--random-config", metavar="CONFIG_JSON",
+                    help="instead of MODEL_DIR: run the model this config.json describes with weights drawn for --weight-seed")
     ap.add_argument("--write-random", metavar="CONFIG_JSON",
                     help="write a model folder with random weights for this config.json into MODEL_DIR, then exit")
-    ap.add_argument("--weight-seed", type=int, default=0, help="seed of --write-random")
+    ap.add_argument("--weight-seed", type=int, default=0, help="seed of --random-config and --write-random")
     ap.add_argument("--weight-std", type=float, default=None,
-                    help="standard deviation of --write-random's matrices (default: the configuration's initializer_range)")
+                    help="standard deviation of the drawn matrices (default: the configuration's initializer_range)")
     ap.add_argument("--info", action="store_true", help="print the model's description and exit")
     args = ap.parse_args(argv)
-    if args.model is None:
-        ap.error("a model folder is required")
+    if (args.model is None) == (args.random_config is None):
+        ap.error("a model folder or --random-config CONFIG_JSON is required (one of them)")
+    if args.write_random and args.model is None:
+        ap.error("--write-random writes into MODEL_DIR")
     if args.ctx <= 0:
         print("Error: --ctx must be > 0", file=sys.stderr)
         return 1
@@ -76,7 +81,12 @@ def main(argv=None) -> int:
                    with_temperature, with_top_k, with_top_p)
     from .api import load_llm
     try:
-        llm = load_llm(args.model, args.ctx, args.dtype, max_batch=max(1, min(64, len(prompts) or 1)))
+        batch = max(1, min(64, len(prompts) or 1))
+        if args.random_config:
+            llm = load_llm(args.random_config, args.ctx, args.dtype, max_batch=batch, random_seed=args.weight_seed,
+                           random_std=args.weight_std)
+        else:
+            llm = load_llm(args.model, args.ctx, args.dtype, max_batch=batch)
     except Exception as e:
         print(f"Error loading model: {e}", file=sys.stderr)
         return 1

@@ -12,7 +12,7 @@ from __future__ import annotations
 import json
 import os
 from dataclasses import dataclass
-from typing import Any, Callable, Dict, Mapping, Type
+from typing import Any, Callable, Dict, List, Mapping, Optional, Tuple, Type
 
 
 class ConfigError(ValueError):
@@ -94,7 +94,10 @@ class KeyReader:
 
 @dataclass(frozen=True)
 class ModelConfig:
-    """What every architecture's configuration offers to the rest of the library."""
+    """What every architecture's configuration offers to the rest of the library.  Engine, entry point, loop and
+    random weights ask these methods and read no key of their own: which keys a config.json has is the
+    architecture's business alone (computerex/dlgo keeps one descriptor per architecture the same way,
+    models/llm/arch.go:17-43)."""
 
     architecture: str
 
@@ -104,6 +107,31 @@ class ModelConfig:
 
     def to_dict(self) -> Dict[str, Any]:
         raise NotImplementedError
+
+    def context_length(self) -> Optional[int]:
+        """The longest sequence the model's positions are defined for; None if nothing in the model bounds it."""
+        return None
+
+    def stop_tokens(self) -> Tuple[int, ...]:
+        """Token ids that end a sequence unless a request says otherwise."""
+        return ()
+
+    def describe(self) -> List[str]:
+        """The sizes worth printing, as short phrases ("16 layers", "2048 dim", ...)."""
+        return []
+
+    def storage_dtype(self) -> str:
+        """The element type a checkpoint of this model is stored in ("bfloat16", "float16" or "float32")."""
+        return "bfloat16"
+
+    def init_std(self) -> Optional[float]:
+        """The standard deviation random matrices are drawn with, if the configuration names one."""
+        return None
+
+    def stored_as(self, dtype_name: str) -> "ModelConfig":
+        """The configuration of the same model whose checkpoint is stored in another element type (an architecture
+        whose config.json does not record the type returns itself)."""
+        return self
 
 
 @dataclass(frozen=True)

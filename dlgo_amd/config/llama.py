@@ -14,8 +14,8 @@ The llama3 `rope_scaling` block has no counterpart in dlgo.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
-from typing import Any, Dict, Mapping, Optional, Tuple
+from dataclasses import dataclass, replace
+from typing import Any, Dict, List, Mapping, Optional, Tuple
 
 from .base import ConfigError, KeyReader, ModelConfig
 
@@ -99,6 +99,27 @@ class LlamaConfig(ModelConfig):
     @property
     def group(self) -> int:
         return self.num_attention_heads // self.num_key_value_heads
+
+    # what the rest of the library asks of any configuration
+    def context_length(self) -> Optional[int]:
+        return self.max_position_embeddings
+
+    def stop_tokens(self) -> Tuple[int, ...]:
+        return self.eos_token_ids
+
+    def describe(self) -> List[str]:
+        return [f"{self.num_hidden_layers} layers", f"{self.hidden_size} dim",
+                f"{self.num_attention_heads} heads ({self.num_key_value_heads} KV)", f"{self.intermediate_size} FFN",
+                f"vocab {self.vocab_size}"]
+
+    def storage_dtype(self) -> str:
+        return self.torch_dtype
+
+    def init_std(self) -> Optional[float]:
+        return self.initializer_range
+
+    def stored_as(self, dtype_name: str) -> "LlamaConfig":
+        return replace(self, torch_dtype=dtype_name)
 
     @classmethod
     def from_dict(cls, raw: Mapping[str, Any]) -> "LlamaConfig":

@@ -870,11 +870,16 @@ extern "C" const char* dlgo_gemm_rmsnorm(const void* W, const float* X, const fl
 }
 
 
-// Whether the two entry points below take a product: up to 16 rows of X, weight rows of 2 to 8 whole kilobytes.
-// scaled: as the consumer (dlgo_gemm_rows_scaled), which takes fewer lengths of rows than the producer.
-extern "C" int dlgo_gemm_rows_streams(int dtype, int Tn, int K, int ldw, int scaled) {
+// Whether the streamed products take a product of Tn rows with a weight [N, K]: up to 16 rows of X, weight rows of whole
+// kilobytes.  role 0: the plain product; 1: as dlgo_gemm_rows_leave_parts, which leaves a share of the sums of squares
+// for every 16 of its N columns; 2: as dlgo_gemm_rows_scaled, which adds up the shares of the K columns it reads.  Both
+// hold at most NORM_PARTS_MAX shares a row, so a normed width beyond 16 * NORM_PARTS_MAX is not theirs.
+extern "C" int dlgo_gemm_rows_streams(int dtype, int N, int Tn, int K, int ldw, int role) {
   int turns = 1;
-  return dtype == DLGO_ELEM && stream_waves<elem_t>(Tn, K, ldw, &turns) > 0 ? 1 : 0;
+  if (dtype != DLGO_ELEM || N <= 0 || stream_waves<elem_t>(Tn, K, ldw, &turns) <= 0) return 0;
+  if (role == 1 && (N + 15) / 16 > NORM_PARTS_MAX) return 0;
+  if (role == 2 && (K + 15) / 16 > NORM_PARTS_MAX) return 0;
+  return role >= 0 && role <= 2 ? 1 : 0;
 }
 
 // residual [T, N] (float32) += X W^T, and for the norm that follows: unscaled [T, N] (run dtype) = new residual * norm_w,

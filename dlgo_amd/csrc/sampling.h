@@ -18,7 +18,12 @@ const char* dlgo_argmax(const float* logits, int ld, int n_rows, int V, void* pa
 // more rows than DLGO_ARGMAX_NOALLOC_ROWS are refused.  Nothing in the array has to start at zero: the first stage
 // writes every entry that the second reads.  All calls on one GPU share the array, so calls that overlap there
 // (two streams, two threads) race; calls on one stream are ordered and safe.
+// The array's address on a device is asked of the runtime (hipGetSymbolAddress) the first time it is wanted there, which
+// is a call that a capturing stream does not take: a caller that captures calls dlgo_argmax_noalloc_init(), or
+// dlgo_argmax_noalloc itself, once on that device before its first capture.  After that the entry point only launches.
 #define DLGO_ARGMAX_NOALLOC_ROWS 256
 const char* dlgo_argmax_noalloc(const float* logits, int ld, int n_rows, int V, int32_t* out, hipStream_t stream);
+// Resolves the array's address for the current device (nothing else); nullptr on success.
+const char* dlgo_argmax_noalloc_init();
 
 }  // extern "C"

@@ -1115,26 +1115,35 @@ static __device__ __align__(256) unsigned char argmax_scratch[DLGO_ARGMAX_NOALLO
 static void* argmax_scratch_ptr[DLGO_MAX_DEVICES];
 static std::mutex argmax_scratch_lock;
 
+// The address of the current device's copy of the array, asked of the runtime the first time it is wanted there.
+static const char* argmax_scratch_here(void** where) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  DLGO_REQUIRE(e == hipSuccess, "argmax: hipGetDevice failed: %s", hipGetErrorString(e));
+  DLGO_REQUIRE(dev >= 0 && dev < DLGO_MAX_DEVICES, "argmax: device %d is beyond the %d this library keeps scratch for", dev, DLGO_MAX_DEVICES);
+  std::lock_guard<std::mutex> hold(argmax_scratch_lock);
+  if (!argmax_scratch_ptr[dev]) {        // this device's copy of the array, with this device current
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(argmax_scratch));
+    DLGO_REQUIRE(e == hipSuccess && p, "argmax: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+    argmax_scratch_ptr[dev] = p;
+  }
+  *where = argmax_scratch_ptr[dev];
+  return nullptr;
+}
+
+extern "C" const char* dlgo_argmax_noalloc_init() {
+  void* p;
+  return argmax_scratch_here(&p);
+}
+
 extern "C" const char* dlgo_argmax_noalloc(const float* logits, int ld, int n_rows, int V, int32_t* out, hipStream_t stream) {
   DLGO_REQUIRE(n_rows >= 0 && V > 0 && ld >= V, "argmax: bad sizes rows=%d V=%d ld=%d", n_rows, V, ld);
   DLGO_REQUIRE(n_rows <= DLGO_ARGMAX_NOALLOC_ROWS, "argmax without allocation: at most %d rows at a time, got %d",
                DLGO_ARGMAX_NOALLOC_ROWS, n_rows);
   DLGO_REQUIRE(logits && out, "argmax: missing argument");
-  int dev = -1;
-  hipError_t e = hipGetDevice(&dev);
-  DLGO_REQUIRE(e == hipSuccess, "argmax: hipGetDevice failed: %s", hipGetErrorString(e));
-  DLGO_REQUIRE(dev >= 0 && dev < DLGO_MAX_DEVICES, "argmax: device %d is beyond the %d this library keeps scratch for", dev, DLGO_MAX_DEVICES);
-  void* partial;
-  {
-    std::lock_guard<std::mutex> hold(argmax_scratch_lock);
-    if (!argmax_scratch_ptr[dev]) {      // this device's copy of the array, with this device current
-      void* p = nullptr;
-      e = hipGetSymbolAddress(&p, HIP_SYMBOL(argmax_scratch));
-      DLGO_REQUIRE(e == hipSuccess && p, "argmax: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
-      argmax_scratch_ptr[dev] = p;
-    }
-    partial = argmax_scratch_ptr[dev];
-  }
+  void* partial = nullptr;
+  if (const char* err = argmax_scratch_here(&partial)) return err;
   if (n_rows == 0) return nullptr;
   hipLaunchKernelGGL(argmax_part_kernel, dim3(ARGMAX_CHUNKS, n_rows), dim3(ARGMAX_THREADS), 0, stream, logits, ld, V, (BestIdx*)partial);
   DLGO_LAUNCH_CHECK("argmax");
@@ -1165,8 +1174,10 @@ extern "C" const char* dlgo_sample(const float* logits, int ld, int n_rows, int 
   if (staged) {
     hipLaunchKernelGGL(topk_part_kernel, dim3(TK_CHUNKS, n_rows), dim3(TK_THREADS), 0, stream, logits, ld, V, work, temperature,
                        top_k, top_p, min_p, penalty, recent, n_recent, recent_rows, counts);
+    DLGO_LAUNCH_CHECK("sample (the rows' parts)");
     hipLaunchKernelGGL(topk_final_kernel, dim3(n_rows), dim3(SAMP_THREADS), 0, stream, logits, ld, V, work, temperature, top_k,
                        top_p, min_p, penalty, recent, n_recent, recent_rows, counts, uniform, out);
+    DLGO_LAUNCH_CHECK("sample (the rows' cuts)");
   }
   hipLaunchKernelGGL(sample_kernel, dim3(n_rows), dim3(SAMP_THREADS), 0, stream, logits, ld, V, work, temperature, top_k, top_p,
                      min_p, penalty, recent, n_recent, recent_rows, counts, uniform, out, staged);

@@ -24,7 +24,7 @@ import numpy as np
 import torch
 
 from .. import models as _models  # noqa: F401  (registers the architectures)
-from ..cache import PAGE, Cache
+from ..cache import PAGE, Cache, CacheError, OutOfPages
 from ..config import ModelConfig, build_model, load_config
 from ..kernels import build as kernel_build
 from ..weights import load_state, load_weights, random_tensors
@@ -47,6 +47,15 @@ def run_dtype(name) -> torch.dtype:
         return _RUN_DTYPES[str(name).lower()]
     except KeyError:
         raise EngineError(f"unknown dtype {name!r}: bfloat16 or float32") from None
+
+
+def recordings_bytes(vocab: int, max_batch: int = 64, graph_max_batch: int = 128, prompt_graph_bytes: int = 1 << 30,
+                     use_graphs: bool = True, **_other_engine_options) -> int:
+    """Device memory that an engine with these options may come to hold for its recorded steps, beyond weights, cache
+    and workspace: the fixed logits of the recorded steps of single tokens, and the logits that the recordings of
+    prompt steps keep (bounded by prompt_graph_bytes).  Whoever sizes a cache from the free memory takes this off first."""
+    fixed = min(graph_max_batch, max(max_batch, 1)) * vocab * 4 if use_graphs else 0
+    return fixed + (prompt_graph_bytes if use_graphs else 0)
 
 
 def _require_gpu() -> None:
@@ -82,16 +91,17 @@ class Engine:
     def __init__(self, model, dtype="bfloat16", device="cuda:0", max_tokens: int = 8192, max_ctx: Optional[int] = None,
                  max_slots: Optional[int] = None, max_step_tokens: int = 8192, logits_rows: int = 1024,
                  use_graphs: bool = True, graph_max_batch: int = 128, prompt_graph_max_tokens: int = 4096,
-                 prompt_graph_limit: int = 32):
+                 prompt_graph_limit: int = 32, prompt_graph_bytes: int = 1 << 30):
         """`model` holds its weights already (see from_folder / from_random).  use_graphs: steps of single tokens are
         recorded per batch size, and steps of fresh prompts of up to prompt_graph_max_tokens rows per shape (the
-        prompt_graph_limit most recently used shapes are kept), the second time a size or shape is seen."""
+        prompt_graph_limit most recently used shapes are kept, as long as the logits they keep stay within
+        prompt_graph_bytes), the second time a size or shape is seen."""
         _require_gpu()
         self.model = model
         self.dtype = run_dtype(dtype)
         self.device = torch.device(device)
         torch.cuda.set_device(self.device)
-        limit = getattr(model.config, "max_position_embeddings", None)
+        limit = model.config.context_length()
         pages_tokens = ((max_tokens + PAGE - 1) // PAGE) * PAGE
         self.max_ctx = min(x for x in (max_ctx, limit, pages_tokens) if x)
         self.max_step_tokens = max(1, min(max_step_tokens, pages_tokens))
@@ -116,12 +126,14 @@ class Engine:
         # recorded steps of fresh prompts, by shape (rows per sequence, wanted places); the least recently used one goes
         self.prompt_graph_max_tokens = prompt_graph_max_tokens
         self.prompt_graph_limit = max(1, prompt_graph_limit)
+        self.prompt_graph_bytes = max(0, prompt_graph_bytes)
         self._prompt_graphs: Dict[tuple, _PromptGraph] = {}
         self._prompt_seen: Dict[tuple, int] = {}
         self._graph_seen: Dict[int, int] = {}
         self._static: Optional[Dict[str, torch.Tensor]] = None
         self._static_logits: Optional[torch.Tensor] = None
         self._meta_dev = torch.empty(0, dtype=torch.int32, device=self.device)
+        self._rows_dev = torch.empty(0, dtype=torch.int32, device=self.device)
         self._staging: List[Tuple[torch.Tensor, Optional[torch.cuda.Event]]] = []
         self._staging_next = 0
         self._logits_piece: Optional[torch.Tensor] = None
@@ -139,7 +151,8 @@ class Engine:
     @classmethod
     def from_random(cls, config: ModelConfig, seed: int, dtype="bfloat16", device="cuda:0", std: Optional[float] = None,
                     norm_jitter: float = 0.0, **kw) -> "Engine":
-        """Random weights drawn on the device and never written (benchmarks)."""
+        """Random weights drawn for the seed (on the host, as a model folder written for the seed would hold them) and
+        never written."""
         _require_gpu()
         model = build_model(config)
         rd = run_dtype(dtype)
@@ -158,7 +171,10 @@ class Engine:
     def fork(self, slot: int, length: Optional[int] = None) -> int:
         """A new sequence that starts as a copy of `slot` (its first `length` tokens; all by default) and goes its own
         way from there: the next step may give the two different tokens."""
-        new = self.cache.copy_slot(slot, length)
+        try:
+            new = self.cache.copy_slot(slot, length)
+        except (CacheError, OutOfPages) as e:
+            raise EngineError(f"fork: {e}") from None
         self.cache.sync_tables()
         return new
 
@@ -217,6 +233,27 @@ class Engine:
         self._staging[idx] = (self._staging[idx][0], ev)
         return {k: dest[offs[k]:offs[k] + len(v)] for k, v in fields.items()}
 
+    def take_rows(self, x: torch.Tensor, rows: Sequence[int]) -> torch.Tensor:
+        """x[rows] for rows given on the host (logits of the sequences that go on, ids of those that are fed): the row
+        numbers go up with the step's arrays, the rows are picked by the library's own kernel; nothing waits."""
+        from ..kernels import ops
+        idx = np.asarray(rows, dtype=np.int64)
+        if idx.size and (idx.min() < 0 or idx.max() >= x.shape[0]):
+            raise EngineError(f"take_rows: rows {rows} of a tensor with {x.shape[0]}")
+        out = torch.empty((len(idx),) + tuple(x.shape[1:]), dtype=x.dtype, device=x.device)
+        if len(idx):
+            stage = self._stage(len(idx))
+            stage.numpy()[:len(idx)] = idx
+            if self._rows_dev.numel() < len(idx):
+                self._rows_dev = torch.empty(max(256, 2 * len(idx)), dtype=torch.int32, device=self.device)
+            self._rows_dev[:len(idx)].copy_(stage[:len(idx)], non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record()
+            i = (self._staging_next - 1) % len(self._staging)
+            self._staging[i] = (self._staging[i][0], ev)
+            ops.copy_rows(x, out, src_rows=self._rows_dev[:len(idx)])
+        return out
+
     # -- the step ----------------------------------------------------------------
     def step(self, entries: Sequence[Entry], sink: Optional[Callable[[int, torch.Tensor], None]] = None) -> Optional[torch.Tensor]:
         """Run the entries' tokens from the cache, as one batch; return float32 logits [wanted, vocab] in the
@@ -274,7 +311,7 @@ class Engine:
         shape = None
         # (a recording keeps its logits: not where those would be more than 64 MB)
         if (self.use_graphs and sink is None and n_out and total <= min(self.max_step_tokens, self.prompt_graph_max_tokens)
-                and n_out * self.vocab * 4 <= (64 << 20) and not any(starts)):
+                and n_out * self.vocab * 4 <= min(64 << 20, self.prompt_graph_bytes) and not any(starts)):
             shape = (tuple(q_lens), tuple(wanted))
         out = None
         if sink is None and (shape is None or shape not in self._prompt_graphs):
@@ -365,9 +402,11 @@ class Engine:
         finally:
             if was_enabled:
                 gc.enable()
-        while len(self._prompt_graphs) >= self.prompt_graph_limit:
-            self._prompt_graphs.pop(next(iter(self._prompt_graphs)))
         self._prompt_graphs[shape] = _PromptGraph(graph, meta, logits, ctx)
+        # the least recently used recordings go when there are too many or their logits take too much
+        held = lambda: sum(p.logits.numel() * 4 for p in self._prompt_graphs.values())
+        while len(self._prompt_graphs) > 1 and (len(self._prompt_graphs) > self.prompt_graph_limit or held() > self.prompt_graph_bytes):
+            self._prompt_graphs.pop(next(iter(self._prompt_graphs)))
         graph.replay()
         return logits.clone()
 
@@ -396,16 +435,10 @@ class Engine:
         overwrites).  `tokens` are ids on the host, or an int32 tensor on the device in the order of `slots`
         (the sampler's output: the ids need not come to the host before the next step starts)."""
         b = len(slots)
-        if b > self.graph_max_batch:
-            # more sequences than the fixed arrays of a recorded step hold: in runs of that many, into a buffer of this call
-            out = torch.empty((b, self.vocab), dtype=torch.float32, device=self.device)
-            for c0 in range(0, b, self.graph_max_batch):
-                c1 = min(b, c0 + self.graph_max_batch)
-                out[c0:c1].copy_(self.decode(slots[c0:c1], tokens[c0:c1], checked))
-            return out
         slot_arr = np.asarray(slots, dtype=np.int64)
         on_device = isinstance(tokens, torch.Tensor)
         if not checked:
+            # the whole call, before anything runs: distinct live slots, token ids, the context, and pages for every sequence
             if b < 1:
                 raise EngineError("decode: no sequences")
             if len(set(slots)) != b or slot_arr.min() < 0 or slot_arr.max() >= self.cache.max_slots \
@@ -419,16 +452,24 @@ class Engine:
                 if tok.shape != (b,) or tok.min() < 0 or tok.max() >= self.vocab:
                     raise EngineError(f"decode: one token id inside the vocabulary of {self.vocab} per slot")
         starts = self.cache.lengths[slot_arr]
+        needs_pages = bool((starts % PAGE == 0).any()) or self.cache.has_windows
         if not checked:
             if (starts + 1 > self.max_ctx).any():
                 raise EngineError(f"decode: a sequence would exceed the context of {self.max_ctx}")
-        if (starts % PAGE == 0).any() or self.cache.has_windows:
-            wants = [(int(s), int(st) + 1) for s, st in zip(slot_arr, starts)]
-            if not checked:
-                why = self.cache.can_reserve(wants)
+            if needs_pages:
+                why = self.cache.can_reserve([(int(s), int(st) + 1) for s, st in zip(slot_arr, starts)])
                 if why:
                     raise EngineError(f"decode: {why}")
-            self.cache.reserve(wants)
+        if b > self.graph_max_batch:
+            # more sequences than the fixed arrays of a recorded step hold: in runs of that many (the call as a whole is
+            # checked by now), into a buffer of this call
+            out = torch.empty((b, self.vocab), dtype=torch.float32, device=self.device)
+            for c0 in range(0, b, self.graph_max_batch):
+                c1 = min(b, c0 + self.graph_max_batch)
+                out[c0:c1].copy_(self.decode(slots[c0:c1], tokens[c0:c1], checked=True))
+            return out
+        if needs_pages:
+            self.cache.reserve([(int(s), int(st) + 1) for s, st in zip(slot_arr, starts)])
             self.cache.sync_tables()
         st = self._static_arrays()
         tok_host = np.zeros(b, dtype=np.int32) if on_device else np.asarray(tokens, dtype=np.int32)

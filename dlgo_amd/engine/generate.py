@@ -92,6 +92,13 @@ def plan_batch(prompt_lens: Sequence[int], max_new: Sequence[int], free_slots: i
     return n
 
 
+def _take(engine, x, rows):
+    """x[rows] for row numbers the host knows: the engine's own row copy where it has one (the rows stay on the
+    device and nothing waits), plain indexing for a stand-in."""
+    take = getattr(engine, "take_rows", None)
+    return take(x, rows) if take is not None else x[rows]
+
+
 def _decode_batch(engine, sampler, live, logits, prompts, results, stats, on_token) -> None:
     """The decode loop of one batch, one step ahead of the host (see the module's text).  `logits` has one row per
     entry of `live`, in order."""
@@ -114,7 +121,7 @@ def _decode_batch(engine, sampler, live, logits, prompts, results, stats, on_tok
         if not keep:
             return
         if len(keep) != len(live):
-            logits = logits[keep]
+            logits = _take(engine, logits, keep)
             live = [live[r] for r in keep]
         ids, wait = sampler.choose_async(logits, [l.config.sampler for l in live],
                                          [uniform(l.seed, l.index, len(l.tokens)) for l in live], keys=[l.slot for l in live])
@@ -122,7 +129,7 @@ def _decode_batch(engine, sampler, live, logits, prompts, results, stats, on_tok
         fed = [row for row, l in enumerate(live) if len(l.tokens) + 1 < l.config.max_tokens and l.pos + 1 < engine.max_ctx - 1]
         next_logits = None
         if fed:
-            next_logits = engine.decode([live[r].slot for r in fed], ids if len(fed) == len(live) else ids[fed])
+            next_logits = engine.decode([live[r].slot for r in fed], ids if len(fed) == len(live) else _take(engine, ids, fed))
             stats.steps += 1
         chosen = wait()
         now = time.perf_counter()
@@ -148,7 +155,7 @@ def _decode_batch(engine, sampler, live, logits, prompts, results, stats, on_tok
         if not still:
             return
         rows = [fed.index(r) for r in still]          # every row in `still` was fed
-        logits = next_logits if len(rows) == len(fed) else next_logits[rows]
+        logits = next_logits if len(rows) == len(fed) else _take(engine, next_logits, rows)
         live = [live[r] for r in still]
 
 

@@ -84,7 +84,7 @@ def _lib(module: str, defines=()):
     lib = _libs.get(key)
     if lib is None:
         lib = build.load(module, defines)
-        for name in ("dlgo_embed", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_accum_norm", "dlgo_gemm_parts", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_gemm_rows_leave_parts", "dlgo_gemm_rows_scaled", "dlgo_gemm_tile_leave", "dlgo_gemm_tile_scaled", "dlgo_attention_rows",
+        for name in ("dlgo_embed", "dlgo_copy_rows", "dlgo_rmsnorm", "dlgo_rope_kv", "dlgo_gemm", "dlgo_gemm_accum_norm", "dlgo_gemm_parts", "dlgo_gemm_rows", "dlgo_gemm_rmsnorm", "dlgo_gemm_rows_leave_parts", "dlgo_gemm_rows_scaled", "dlgo_gemm_tile_leave", "dlgo_gemm_tile_scaled", "dlgo_attention_rows",
                      "dlgo_attention_prefill", "dlgo_attention_prefill_f32", "dlgo_attention_decode", "dlgo_attention_decode_f32", "dlgo_argmax", "dlgo_sample", "dlgo_bias_add", "dlgo_head_rmsnorm"):
             if hasattr(lib, name):
                 getattr(lib, name).restype = ctypes.c_char_p
@@ -103,6 +103,35 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Te
         raise KernelError(f"embed: output {tuple(out.shape)} does not fit {n} tokens of width {d}")
     _check(_lib("embed").dlgo_embed(_ptr(table), dtype_code(table.dtype), _ptr(ids), _ptr(out), n, d, table.shape[0], _stream()))
     return out
+
+
+def copy_rows(src: torch.Tensor, dst: torch.Tensor, src_rows: Optional[torch.Tensor] = None,
+              dst_rows: Optional[torch.Tensor] = None, n: Optional[int] = None) -> torch.Tensor:
+    """dst[dst_rows[i]] = src[src_rows[i]] for i < n (a missing list stands for i itself; n defaults to the lists'
+    length, or to src's rows).  Rows of any element type whose bytes are a multiple of 4; 1-d tensors are rows of one
+    element.  The lists are int32 on the device and hold row numbers inside the two tensors (the caller's duty: they
+    are not read here); source and destination rows must not overlap."""
+    given = dst
+    if src.dim() == 1:
+        src = src.unsqueeze(1)
+    if dst.dim() == 1:
+        dst = dst.unsqueeze(1)
+    _need(src, "rows to copy", dims=2)
+    _need(dst, "copied rows", src.dtype, 2)
+    for name, r in (("source rows", src_rows), ("destination rows", dst_rows)):
+        if r is not None:
+            _need(r, name, torch.int32, 1)
+    if n is None:
+        n = src_rows.shape[0] if src_rows is not None else (dst_rows.shape[0] if dst_rows is not None else src.shape[0])
+    es = src.element_size()
+    if src.shape[1] != dst.shape[1] or (src.shape[1] * es) % 4 or n < 0 \
+            or any(r is not None and r.shape[0] < n for r in (src_rows, dst_rows)) \
+            or (src_rows is None and src.shape[0] < n) or (dst_rows is None and dst.shape[0] < n):
+        raise KernelError(f"copy_rows: {n} rows of {tuple(src.shape)} into {tuple(dst.shape)} (rows of equal width, a multiple of 4 bytes)")
+    _check(_lib("embed").dlgo_copy_rows(_ptr(src), _ptr(src_rows), _ptr(dst), _ptr(dst_rows), n, ctypes.c_longlong(src.shape[1] * es),
+                                        ctypes.c_longlong(_rows(src, "rows to copy") * es), ctypes.c_longlong(_rows(dst, "copied rows") * es),
+                                        _stream()))
+    return given
 
 
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
@@ -311,14 +340,18 @@ class UnscaledNorm:
         self.rows, self.parts, self.n_parts, self.width, self.eps = rows, parts, n_parts, width, eps
 
 
-def streams_few_rows(weight: torch.Tensor, rows: int, scaled: bool = False) -> bool:
+ROLE_PLAIN, ROLE_LEAVES_NORM, ROLE_APPLIES_NORM = 0, 1, 2
+
+
+def streams_few_rows(weight: torch.Tensor, rows: int, role: int = ROLE_PLAIN) -> bool:
     """Whether the streamed products take this weight with this many rows of x: up to 16 rows and weight rows of whole
-    KB."""
+    KB; as the product that leaves a norm (ROLE_LEAVES_NORM) or applies one left to it (ROLE_APPLIES_NORM) also a
+    normed width that its shares of the sums of squares cover."""
     if weight.dim() != 2 or weight.stride(1) != 1 or not (1 <= rows <= 16):
         return False
     lib = _lib("gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),))
     lib.dlgo_gemm_rows_streams.restype = ctypes.c_int
-    return bool(lib.dlgo_gemm_rows_streams(dtype_code(weight.dtype), rows, weight.shape[1], weight.stride(0), int(scaled)))
+    return bool(lib.dlgo_gemm_rows_streams(dtype_code(weight.dtype), weight.shape[0], rows, weight.shape[1], weight.stride(0), int(role)))
 
 
 def _tiles_take_norm(weight: torch.Tensor, rows: int, role: int) -> bool:
@@ -334,12 +367,12 @@ def _tiles_take_norm(weight: torch.Tensor, rows: int, role: int) -> bool:
 
 def can_leave_unscaled(weight: torch.Tensor, rows: int) -> bool:
     """Whether gemm_accum_leave_norm takes this weight with this many rows of x (contiguous rows of x assumed)."""
-    return streams_few_rows(weight, rows) or _tiles_take_norm(weight, rows, 1)
+    return streams_few_rows(weight, rows, ROLE_LEAVES_NORM) or _tiles_take_norm(weight, rows, 1)
 
 
 def can_take_unscaled(weight: torch.Tensor, rows: int) -> bool:
     """Whether gemm_scaled takes this weight with this many rows (contiguous rows assumed)."""
-    return streams_few_rows(weight, rows, scaled=True) or _tiles_take_norm(weight, rows, 2)
+    return streams_few_rows(weight, rows, ROLE_APPLIES_NORM) or _tiles_take_norm(weight, rows, 2)
 
 
 def gemm_accum_leave_norm(weight: torch.Tensor, x: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor, eps: float,

@@ -200,7 +200,7 @@ class Attention(Mixer):
             def leave():
                 shares = ctx.scratch("attention.norm_shares", t * ((self.width + 15) // 16), torch.float32)
                 return ops.gemm_accum_leave_norm(self.w_o, out, residual, then[0].weight, then[0].eps, then[1], shares)
-            if unscaled_ok and ops.streams_few_rows(self.w_o, t):
+            if unscaled_ok and ops.streams_few_rows(self.w_o, t, ops.ROLE_LEAVES_NORM):
                 return leave()
             if ops.gemm_accum_then_norm(self.w_o, out, residual, split, then[0].weight, then[0].eps, then[1]):
                 return True

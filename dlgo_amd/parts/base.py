@@ -38,10 +38,12 @@ class Part:
     #: kernel modules (names under csrc/) this part launches; built before first use
     kernel_modules: Tuple[str, ...] = ()
 
-    #: True if what the part launches for a step of single tokens depends only on the step's device arrays and on the
-    #: number of sequences, so that the launches can be recorded once and replayed with new arrays.  A part that
-    #: reads the step's host-side numbers (ctx.host) to decide what to launch, or launches through anything that cannot
-    #: be recorded, sets this to False; a model with such a part runs every step as it is.
+    #: True if what the part launches for a step depends only on the step's device arrays and on its shape (the number of
+    #: sequences, the rows each brings and the wanted places), so that the launches can be recorded once and replayed
+    #: with new arrays: steps of single tokens per batch size, steps of fresh prompts per shape.  A part that reads the
+    #: step's host-side numbers (ctx.host: lengths, slots) to decide what to launch or where to write, or launches
+    #: through anything that cannot be recorded, sets this to False; a model with such a part runs every step, prompts
+    #: included, as it is.
     graph_safe: bool = True
 
     def tensor_specs(self) -> Dict[str, TensorSpec]:

@@ -56,7 +56,7 @@ class OutputHead(Part):
         return isinstance(norm, RMSNorm) and ops.fused_norm_pays(self.weight, ctx.n_tokens)
 
     def takes_unscaled(self, ctx) -> bool:
-        return ops.streams_few_rows(self.weight, ctx.n_tokens, scaled=True)
+        return ops.streams_few_rows(self.weight, ctx.n_tokens, ops.ROLE_APPLIES_NORM)
 
     def __call__(self, xn, out: torch.Tensor, norm=None) -> torch.Tensor:
         """xn: normed rows (run dtype), or what stands for them (see Part.takes_unscaled), or with `norm` the float32

@@ -15,6 +15,7 @@ rotate-and-store kernel of an attention mixer; None if it rotates nothing).
 from __future__ import annotations
 
 import math
+import weakref
 from dataclasses import dataclass
 from typing import Optional
 
@@ -69,6 +70,33 @@ def rotary_frequencies(width: int, theta: float, scaling=None) -> np.ndarray:
     return out
 
 
+class _Tables:
+    """cos and sin of position * frequency for one recipe of frequencies, [positions, width/2] float32 each."""
+    __slots__ = ("cos", "sin", "__weakref__")
+
+    def __init__(self, cos: torch.Tensor, sin: torch.Tensor):
+        self.cos, self.sin = cos, sin
+
+
+# One pair of tables per distinct recipe (the frequencies themselves, which theta, width and scaling determine) and device,
+# shared by every layer that names the recipe: a model of 16 equal layers holds one, and a decode step reads one.  The
+# entries live as long as a part holds them.
+_TABLES: "weakref.WeakValueDictionary[tuple, _Tables]" = weakref.WeakValueDictionary()
+
+
+def rotary_tables(frequencies: np.ndarray, max_positions: int, device: torch.device) -> _Tables:
+    key = (frequencies.tobytes(), str(torch.device(device)))
+    held = _TABLES.get(key)
+    if held is not None and held.cos.shape[0] >= max_positions:
+        return held
+    angles = np.arange(max_positions, dtype=np.float64)[:, None] * frequencies[None, :]
+    cos = torch.from_numpy(np.cos(angles).astype(np.float32)).to(device)
+    sin = torch.from_numpy(np.sin(angles).astype(np.float32)).to(device)
+    held = _Tables(cos.contiguous(), sin.contiguous())
+    _TABLES[key] = held          # longer tables take the shorter ones' place for whoever asks next
+    return held
+
+
 class Rotary(PositionEncoding):
     kernel_modules = ("rope_kv",)
 
@@ -81,15 +109,14 @@ class Rotary(PositionEncoding):
         self.scaling = scaling
         self.interleaved = interleaved
         self.frequencies = rotary_frequencies(self.width, self.theta, scaling)
+        self._tables: Optional[_Tables] = None
         self._rotation: Optional[Rotation] = None
 
     def prepare(self, max_positions: int, device: torch.device) -> None:
-        if self._rotation is not None and self._rotation.cos.shape[0] >= max_positions and self._rotation.cos.device == device:
+        if self._rotation is not None and self._rotation.cos.shape[0] >= max_positions and self._rotation.cos.device == torch.device(device):
             return
-        angles = np.arange(max_positions, dtype=np.float64)[:, None] * self.frequencies[None, :]
-        cos = torch.from_numpy(np.cos(angles).astype(np.float32)).to(device)
-        sin = torch.from_numpy(np.sin(angles).astype(np.float32)).to(device)
-        self._rotation = Rotation(cos.contiguous(), sin.contiguous(), self.width, self.interleaved)
+        self._tables = rotary_tables(self.frequencies, max_positions, device)
+        self._rotation = Rotation(self._tables.cos, self._tables.sin, self.width, self.interleaved)
 
     def rotation(self) -> Optional[Rotation]:
         if self._rotation is None:

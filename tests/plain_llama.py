@@ -60,6 +60,93 @@ def read_model(folder: str):
 
 
 # ----------------------------------------------------------------------------
+# random weights from (seed, tensor name, element index), written a second time
+# ----------------------------------------------------------------------------
+# The recipe, as the library's documentation states it (the reference draws its fixtures from one seeded stream,
+# testdata/generate.go:45-148; a counter keyed by name and index has no counterpart there):
+#   key = splitmix64(seed ^ fnv1a64(name)); draw(c) = splitmix64(key + c * 0x9E3779B97F4A7C15), c = 1, 2, ...;
+#   u(c) = ((draw(c) >> 11) + 1) / 2^53; normal i = sqrt(-2 ln u(2i+1)) cos(2 pi u(2i+2)); an element is
+#   float32(offset + scale * normal i), then rounded to the stored type (bfloat16: nearest, ties to even).
+# One element at a time with Python integers, so that nothing here resembles the vectorised code it checks.
+
+_M64 = 0xFFFFFFFFFFFFFFFF
+
+
+def _splitmix(z):
+    z &= _M64
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _M64
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _M64
+    return z ^ (z >> 31)
+
+
+def _fnv1a64(text):
+    h = 0xCBF29CE484222325
+    for byte in text.encode("utf-8"):
+        h = ((h ^ byte) * 0x100000001B3) & _M64
+    return h
+
+
+def random_element(seed, name, i, scale, offset=0.0):
+    """Element i (row-major) of tensor `name` for `seed`, as the float32 value before any narrower rounding."""
+    key = _splitmix((seed & _M64) ^ _fnv1a64(name))
+    u1 = ((_splitmix(key + (2 * i + 1) * 0x9E3779B97F4A7C15) >> 11) + 1) / 9007199254740992.0
+    u2 = ((_splitmix(key + (2 * i + 2) * 0x9E3779B97F4A7C15) >> 11) + 1) / 9007199254740992.0
+    normal = float(np.sqrt(-2.0 * np.log(u1)) * np.cos(2.0 * math.pi * u2))
+    return np.float32(offset + scale * normal) if offset else np.float32(scale * normal)
+
+
+def round_to_bf16(x):
+    """float32 -> the float32 value of the nearest bfloat16, ties to even (the rule of quant/bf16.go's inverse; NaNs do
+    not occur here)."""
+    bits = np.asarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    bits = (bits + 0x7FFF + ((bits >> 16) & 1)) & 0xFFFF0000
+    return bits.astype(np.uint32).view(np.float32)
+
+
+def random_tensor(seed, name, shape, scale, offset=0.0, bf16=False):
+    n = int(np.prod(shape))
+    out = np.array([random_element(seed, name, i, scale, offset) for i in range(n)], dtype=np.float32)
+    if bf16:
+        out = round_to_bf16(out)
+    return out.astype(np.float64).reshape(shape)
+
+
+def llama_tensor_shapes(cfg):
+    """name -> (shape, is a norm weight) for a Llama config.json, as a model folder names them."""
+    d, f, L = cfg["hidden_size"], cfg["intermediate_size"], cfg["num_hidden_layers"]
+    H = cfg["num_attention_heads"]
+    KV = cfg.get("num_key_value_heads") or H
+    hd = cfg.get("head_dim") or d // H
+    out = {"model.embed_tokens.weight": ((cfg["vocab_size"], d), False), "model.norm.weight": ((d,), True)}
+    if not cfg.get("tie_word_embeddings", False):
+        out["lm_head.weight"] = ((cfg["vocab_size"], d), False)
+    for l in range(L):
+        p = f"model.layers.{l}."
+        out[p + "input_layernorm.weight"] = ((d,), True)
+        out[p + "post_attention_layernorm.weight"] = ((d,), True)
+        out[p + "self_attn.q_proj.weight"] = ((H * hd, d), False)
+        out[p + "self_attn.k_proj.weight"] = ((KV * hd, d), False)
+        out[p + "self_attn.v_proj.weight"] = ((KV * hd, d), False)
+        out[p + "self_attn.o_proj.weight"] = ((d, H * hd), False)
+        out[p + "mlp.gate_proj.weight"] = ((f, d), False)
+        out[p + "mlp.up_proj.weight"] = ((f, d), False)
+        out[p + "mlp.down_proj.weight"] = ((d, f), False)
+    return out
+
+
+def random_model(cfg, seed, std=None, norm_jitter=0.0, bf16=False):
+    """The weights of a Llama config.json for a seed, computed here: name -> float64 array."""
+    std = cfg["initializer_range"] if std is None else std
+    w = {}
+    for name, (shape, is_norm) in llama_tensor_shapes(cfg).items():
+        if is_norm:
+            w[name] = random_tensor(seed, name, shape, norm_jitter, 1.0, bf16) if norm_jitter else np.ones(shape)
+        else:
+            w[name] = random_tensor(seed, name, shape, std, 0.0, bf16)
+    return w
+
+
+# ----------------------------------------------------------------------------
 # parts
 # ----------------------------------------------------------------------------
 
@@ -312,17 +399,21 @@ def sample_from_logits(logits, r):
     return len(probs) - 1
 
 
+def filtered_logits(logits, temperature, top_k=0, top_p=1.0, min_p=0.0, penalty=1.0, recent=()):
+    """What the draw is taken from: penalty -> temperature -> top-k -> top-p -> min-p (ops/sampling.go:36-47)."""
+    w = apply_repetition_penalty(logits, recent, penalty)
+    w = apply_temperature(w, temperature)
+    w = apply_top_k(w, top_k)
+    w = apply_top_p(w, top_p)
+    return apply_min_p(w, min_p)
+
+
 def sample_token(logits, r, temperature, top_k=0, top_p=1.0, min_p=0.0, penalty=1.0, recent=()):
     """penalty -> temperature -> top-k -> top-p -> min-p -> draw; temperature
     <= 0 is greedy (ops/sampling.go:32-48)."""
     if temperature <= 0:
         return argmax(logits)
-    w = apply_repetition_penalty(logits, recent, penalty)
-    w = apply_temperature(w, temperature)
-    w = apply_top_k(w, top_k)
-    w = apply_top_p(w, top_p)
-    w = apply_min_p(w, min_p)
-    return sample_from_logits(w, r)
+    return sample_from_logits(filtered_logits(logits, temperature, top_k, top_p, min_p, penalty, recent), r)
 
 
 def greedy_generate(cfg, w, prompt, max_tokens, stop_tokens=()):

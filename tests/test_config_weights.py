@@ -244,16 +244,97 @@ def test_attention_bias_is_an_option_of_the_architecture(tiny_a, tmp_path):
 
 def test_random_weights_do_not_depend_on_the_device_and_fill_integer_tables():
     from dlgo_amd.parts import TensorSpec
-    from dlgo_amd.weights.random_weights import _generator, _table
-    t = _table(TensorSpec((3, 17), kind="table"), _generator(5, "x"))
+    from dlgo_amd.weights.random_weights import _table
+    t = _table(5, "x", TensorSpec((3, 17), kind="table"))
     assert t.dtype == torch.int32 and t.shape == (3, 17)
     assert all(sorted(row.tolist()) == list(range(17)) for row in t)
-    assert torch.equal(t, _table(TensorSpec((3, 17), kind="table"), _generator(5, "x")))
-    assert not torch.equal(t, _table(TensorSpec((3, 17), kind="table"), _generator(6, "x")))
-    # the stream is keyed by seed and name and runs on the host: the same call gives the same values
+    assert torch.equal(t, _table(5, "x", TensorSpec((3, 17), kind="table")))
+    assert not torch.equal(t, _table(6, "x", TensorSpec((3, 17), kind="table")))
+    assert not torch.equal(t, _table(5, "y", TensorSpec((3, 17), kind="table")))
+    # a value is a function of seed, name and index, computed on the host: the same call gives the same values
     c = config_from_dict(TINY_A)
     a, b = random_tensors(c, 9), random_tensors(c, 9)
     assert all(torch.equal(a[k], b[k]) for k in a) and not torch.equal(a["model.norm.weight"], random_tensors(c, 9, norm_jitter=0.1)["model.norm.weight"])
+
+
+def test_random_weights_are_a_function_of_seed_name_and_index():
+    """An element does not depend on the tensor's shape, on its neighbours or on how the work was dealt to threads, and
+    the draws are what they claim to be: standard normals, no two tensors alike."""
+    import dlgo_amd.weights.random_weights as rw
+    whole = rw.normal_tensor(3, "some.weight", (700, 300), 1.0)
+    assert torch.equal(rw.normal_tensor(3, "some.weight", (5, 7), 1.0).flatten(), whole.flatten()[:35])
+    old = rw._CHUNK
+    try:
+        rw._CHUNK = 4096                    # many pieces, on the worker threads
+        assert torch.equal(rw.normal_tensor(3, "some.weight", (700, 300), 1.0), whole)
+    finally:
+        rw._CHUNK = old
+    x = whole.double()
+    assert abs(x.mean()) < 0.01 and abs(x.std() - 1) < 0.01 and abs((x ** 3).mean()) < 0.03 and abs((x ** 4).mean() - 3) < 0.1
+    assert abs(torch.corrcoef(torch.stack([x.flatten()[:-1], x.flatten()[1:]]))[0, 1]) < 0.01       # neighbours
+    other = rw.normal_tensor(3, "some.weighu", (700, 300), 1.0).double()
+    assert abs(torch.corrcoef(torch.stack([x.flatten(), other.flatten()]))[0, 1]) < 0.01            # names
+    assert abs(torch.corrcoef(torch.stack([x.flatten(), rw.normal_tensor(4, "some.weight", (700, 300), 1.0).double().flatten()]))[0, 1]) < 0.01
+    # scale and offset are applied in float64 and rounded once
+    import numpy as np
+    assert torch.equal(rw.normal_tensor(3, "some.weight", (9,), 0.02, 1.0),
+                       torch.from_numpy((1.0 + 0.02 * rw._normals(rw.tensor_key(3, "some.weight"), 0, 9)).astype(np.float32)))
+
+
+def test_random_weights_agree_with_the_plain_side_bit_for_bit(tiny_b):
+    """The generator is written twice, here vectorised and in the plain implementation one element at a time with
+    Python integers; for Tiny B, stored as bfloat16 and as float32, both give the same bits for every tensor."""
+    import numpy as np
+    import plain_llama as plain
+    cfg = config_from_dict(tiny_b)
+    for dtype, bf16 in ((torch.bfloat16, True), (torch.float32, False)):
+        ours = random_tensors(cfg, 21, dtype=dtype, norm_jitter=0.1)
+        theirs = plain.random_model(tiny_b, 21, norm_jitter=0.1, bf16=bf16)
+        assert set(ours) == set(theirs)
+        for name, t in ours.items():
+            assert t.dtype == dtype and tuple(t.shape) == theirs[name].shape
+            assert np.array_equal(t.float().numpy().astype(np.float64), theirs[name]), name
+    # and without jitter the norm weights are exactly one on both sides
+    assert torch.equal(random_tensors(cfg, 21)["model.norm.weight"], torch.ones(tiny_b["hidden_size"]))
+    assert np.array_equal(plain.random_model(tiny_b, 21)["model.norm.weight"], np.ones(tiny_b["hidden_size"]))
+
+
+def test_a_model_of_equal_layers_holds_one_rotary_table():
+    """Layers that name the same recipe (width, base, scaling) share the tables of cosines and sines."""
+    from dlgo_amd.parts import rotary_frequencies
+    raw = dict(TINY_B, num_hidden_layers=16)
+    model = build_model(config_from_dict(raw))
+    model.prepare(200, torch.device("cpu"))
+    rotations = [block.mixer.position.rotation() for _, block in model.layers]
+    assert len(rotations) == 16 and len({r.cos.data_ptr() for r in rotations}) == 1 and len({r.sin.data_ptr() for r in rotations}) == 1
+    assert rotations[0].cos.shape == (200, TINY_B["head_dim"] // 2)
+    # another recipe gets tables of its own; a longer context replaces the shared tables for those who ask for it
+    other = build_model(config_from_dict(dict(TINY_B, rope_theta=1234.0)))
+    other.prepare(200, torch.device("cpu"))
+    assert other.layers[0][1].mixer.position.rotation().cos.data_ptr() != rotations[0].cos.data_ptr()
+    longer = build_model(config_from_dict(raw))
+    longer.prepare(300, torch.device("cpu"))
+    assert longer.layers[0][1].mixer.position.rotation().cos.shape[0] == 300
+    assert torch.equal(longer.layers[0][1].mixer.position.rotation().cos[:200], rotations[0].cos)
+
+
+def test_the_library_reads_no_key_of_a_configuration_itself():
+    """Engine, entry point and random weights ask a configuration through its methods; an architecture whose
+    config.json has other key names (no max_position_embeddings, no eos_token_id, no torch_dtype) answers the same
+    questions."""
+    from dataclasses import dataclass
+    from dlgo_amd.config import ModelConfig
+    c = config_from_dict(TINY_B)
+    assert c.context_length() == 512 and c.stop_tokens() == (3, 5) and c.storage_dtype() == "float32" and c.init_std() == 0.02
+    assert c.describe() == ["3 layers", "128 dim", "4 heads (1 KV)", "352 FFN", "vocab 384"]
+    assert c.stored_as("bfloat16").torch_dtype == "bfloat16" and c.torch_dtype == "float32"
+
+    @dataclass(frozen=True)
+    class Bare(ModelConfig):
+        pass
+    b = Bare("BareForCausalLM")
+    assert b.context_length() is None and b.stop_tokens() == () and b.describe() == [] and b.storage_dtype() == "bfloat16"
+    assert b.init_std() is None and b.stored_as("float32") is b
 
 
 def _rewrite_header(path, change):

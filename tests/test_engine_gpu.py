@@ -278,6 +278,50 @@ def test_errors_before_anything_runs(folders):
     assert eng.length(slot) == 3
 
 
+def test_a_decode_call_is_checked_whole_before_any_of_its_runs(folders):
+    """More sequences than a recorded step's fixed arrays hold go in runs of that many; what is wrong with the call (a
+    slot named in two different runs, a token outside the vocabulary in the last run, a sequence at the end of the
+    context) is found before the first run has advanced anything."""
+    from dlgo_amd.engine import EngineError, Entry
+    eng = engine_for(folders["A", "float32"], "float32", max_tokens=1024, graph_max_batch=2)
+    slots = eng.open(5)
+    eng.step([Entry(s, [3, 4, 5], []) for s in slots])
+    lengths = lambda: [eng.length(s) for s in slots]
+    with pytest.raises(EngineError, match="distinct"):
+        eng.decode([slots[0], slots[1], slots[2], slots[0]], [1, 2, 3, 4])       # twice, but once in each run of two
+    assert lengths() == [3] * 5
+    with pytest.raises(EngineError, match="vocabulary"):
+        eng.decode(slots, [1, 2, 3, 4, 256])
+    assert lengths() == [3] * 5
+    with pytest.raises(EngineError, match="in use"):
+        eng.decode(slots[:4] + [77], [1, 2, 3, 4, 5])
+    assert lengths() == [3] * 5
+    out = eng.decode(slots, [1, 2, 3, 4, 5])
+    assert out.shape == (5, 256) and lengths() == [4] * 5
+    eng.close(slots)
+    eng.cache.check_consistent()
+
+
+def test_fork_reports_what_it_cannot_do_as_the_engine_does(folders):
+    from dlgo_amd.engine import EngineError, Entry
+    eng = engine_for(folders["A", "float32"], "float32", max_tokens=3 * 64, max_slots=2)
+    (a,) = eng.open(1)
+    eng.step([Entry(a, list(range(70)), [])])                    # two of the three pages
+    with pytest.raises(EngineError, match="fork: .*pages"):
+        eng.fork(a)                                              # the copy would need two more
+    b = eng.fork(a, 10)                                          # one page: fits
+    with pytest.raises(EngineError, match="fork: .*no free slot"):
+        eng.fork(a, 5)
+    with pytest.raises(EngineError, match="fork: .*holds 70 tokens"):
+        eng.close([b])
+        eng.fork(a, 71)
+    with pytest.raises(EngineError, match="fork: .*not in use"):
+        eng.fork(b)
+    eng.close([a])
+    eng.cache.check_consistent()
+    assert eng.free_slots() == 2 and eng.free_pages() == (3,)
+
+
 def test_sizes_the_kernels_cannot_take_are_refused_at_once(tmp_path):
     """A width that is no multiple of the products' 16-byte loads: a clear error when the engine is made, for the
     dtype it concerns, not a wrong result later."""
@@ -329,7 +373,7 @@ def test_a_model_with_attention_biases(tmp_path, dtype):
     want = [plain.forward(cfg, w, t) for t in seqs]
     # the biases matter: without them the logits are far away
     stripped = {k: v for k, v in w.items() if not k.endswith(".bias")}
-    assert rel_err(plain.forward(cfg, stripped, seqs[1]), want[1]) > 10 * TOL[dtype]
+    assert rel_err(plain.forward(cfg, stripped, seqs[1]), want[1]) > 5 * TOL[dtype]
     eng = Engine.from_folder(folder, dtype, max_tokens=1024)
     slots = eng.open(3)
     out = eng.step([Entry(s, t, list(range(len(t)))) for s, t in zip(slots, seqs)]).cpu().numpy()

@@ -206,6 +206,46 @@ def test_command_line(folder_a):
     assert bad.returncode == 1 and "--temp must be >= 0" in bad.stderr
 
 
+def test_a_model_from_a_configuration_and_a_seed_without_any_file(tmp_path):
+    """load_llm, the command line and the replay program run a model whose weights are drawn for a seed; the plain side
+    computes the same weights itself (its own generator, element by element) and gives the same tokens and logits."""
+    import dlgo_amd
+    from dlgo_amd.config import config_from_dict
+    raw = dict(TINY_B, initializer_range=0.09)
+    w = plain.random_model(raw, 33)
+    prompts = _prompts(TINY_B, [6, 2, 11], seed=12)
+    want = [plain.greedy_generate(raw, w, p, 5) for p in prompts]
+    opts = (dlgo_amd.with_greedy(), dlgo_amd.with_max_tokens(5), dlgo_amd.with_ignore_eos())
+    cfg_file = tmp_path / "b.json"
+    cfg_file.write_text(json.dumps(raw))
+    for source in (raw, config_from_dict(raw), str(cfg_file)):
+        llm = dlgo_amd.load_llm(source, dtype="float32", max_tokens=512, random_seed=33)
+        assert [r.tokens for r in llm.generate(prompts, *opts)] == want
+    assert [r.tokens for r in dlgo_amd.load_llm(raw, dtype="float32", max_tokens=512, random_seed=34).generate(prompts, *opts)] != want
+    with pytest.raises(Exception, match="random_seed"):
+        dlgo_amd.load_llm(raw, dtype="float32", max_tokens=512)
+    # the command line
+    out = subprocess.run([sys.executable, "-m", "dlgo_amd", "--random-config", str(cfg_file), "--weight-seed", "33", "--greedy",
+                          "--max-tokens", "5", "--dtype", "float32", "--ignore-eos"] +
+                         [a for p in prompts for a in ("--prompt-ids", ",".join(map(str, p)))],
+                         cwd=ROOT, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert [json.loads(l)["tokens"] for l in out.stdout.splitlines() if l.startswith("{")] == want
+    both = subprocess.run([sys.executable, "-m", "dlgo_amd", "--random-config", str(cfg_file), str(tmp_path)], cwd=ROOT,
+                          capture_output=True, text=True)
+    assert both.returncode == 2 and "one of them" in both.stderr
+    # the replay program
+    steps = [{"step": 0, "entries": [{"id": "x", "tokens": prompts[2], "want": list(range(len(prompts[2])))}], "end": ["x"]}]
+    text = "".join(json.dumps(s_) + "\n" for s_ in steps)
+    p = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--config", str(cfg_file), "--weight-seed", "33", "--dtype", "float32",
+                        "--out", str(tmp_path / "out"), "--max-tokens", "64"], input=text, capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0 and "done 0" in p.stdout, p.stderr
+    got = np.fromfile(tmp_path / "out" / "0.f32", dtype="<f4").reshape(-1, TINY_B["vocab_size"])
+    ref = plain.forward(raw, w, prompts[2])
+    assert np.abs(got - ref).max() <= 2e-5 * np.abs(ref).max()
+    assert json.load(open(tmp_path / "out" / "index.json"))["weight_seed"] == 33
+
+
 def _replay(folder, dtype, steps, out_dir, max_tokens):
     text = "".join(json.dumps(s) + "\n" for s in steps)
     p = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", str(out_dir),

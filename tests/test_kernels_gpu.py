@@ -332,7 +332,7 @@ def test_norm_left_in_parts_and_applied_by_the_next_product(dtype, _, rel, n1, k
     res = (3 * torch.randn(t, n1, generator=g)).to(DEV)
     nw = (1 + 0.3 * torch.randn(n1, generator=g)).to(DEV)
     eps = 1e-2
-    assert ops.streams_few_rows(w1, t) and ops.streams_few_rows(w2, t, scaled=True)
+    assert ops.streams_few_rows(w1, t, ops.ROLE_LEAVES_NORM) and ops.streams_few_rows(w2, t, ops.ROLE_APPLIES_NORM)
     assert not ops.streams_few_rows(w2[:, :n1 - 8], t) and not ops.streams_few_rows(w1, 17)
     new_res = res.double() + x.double() @ w1.double().T
     xn = new_res / torch.sqrt((new_res * new_res).mean(-1, keepdim=True) + eps) * nw.double()
@@ -360,6 +360,27 @@ def test_norm_left_in_parts_and_applied_by_the_next_product(dtype, _, rel, n1, k
     with pytest.raises(ops.KernelError, match="whole KB"):
         ops.gemm_scaled(w2[:, :n1 - 8].contiguous(), ops.UnscaledNorm(unscaled[:, :n1 - 8].contiguous(), parts, left.n_parts, n1 - 8, eps),
                         torch.empty(t, n2, dtype=dtype, device=DEV))
+
+
+@pytest.mark.parametrize("n1", [5120, 8192])
+def test_norm_hand_off_refuses_widths_beyond_its_shares(n1):
+    """The streamed products keep at most 256 shares of a row's sum of squares, one for every 16 columns: a normed width
+    beyond 4,096 is not theirs, as the product that leaves the norm or as the one that applies it, and the predicates
+    that the parts ask say so, so that such a model takes the norm kernel instead of an error in its first decode step."""
+    ops = _ops()
+    w1 = torch.zeros(n1, 1024, dtype=torch.bfloat16, device=DEV)        # leaves a norm over n1 columns
+    w2 = torch.zeros(64, n1, dtype=torch.bfloat16, device=DEV)          # would apply it
+    for t in (1, 8, 16):
+        assert ops.streams_few_rows(w1, t) and ops.streams_few_rows(w2, t)             # the plain products are streamed
+        assert not ops.streams_few_rows(w1, t, ops.ROLE_LEAVES_NORM) and not ops.can_leave_unscaled(w1, t)
+        assert not ops.streams_few_rows(w2, t, ops.ROLE_APPLIES_NORM) and not ops.can_take_unscaled(w2, t)
+    narrow = torch.zeros(4096, 1024, dtype=torch.bfloat16, device=DEV)
+    assert ops.can_leave_unscaled(narrow, 8) and ops.can_take_unscaled(torch.zeros(64, 4096, dtype=torch.bfloat16, device=DEV), 8)
+    t = 4
+    with pytest.raises(ops.KernelError, match="width of up to 4096"):
+        ops.gemm_accum_leave_norm(w1, torch.zeros(t, 1024, dtype=torch.bfloat16, device=DEV), torch.zeros(t, n1, device=DEV),
+                                  torch.ones(n1, device=DEV), 1e-5, torch.empty(t, n1, dtype=torch.bfloat16, device=DEV),
+                                  torch.empty(t * (n1 // 16), device=DEV))
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
@@ -856,6 +877,44 @@ def test_attention_reference_vectors():
 # ---------------------------------------------------------------------------
 # sampling
 # ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype,width", [(torch.float32, 128256), (torch.float32, 5), (torch.int32, 1), (torch.bfloat16, 6),
+                                         (torch.bfloat16, 2 * 8 * 64 * 80 * 3), (torch.int32, 37)])
+def test_copy_rows_gathers_and_scatters(dtype, width):
+    """dst[dst_rows[i]] = src[src_rows[i]]: rows picked out (the loop's logits and ids), rows put in place (page-table
+    rows), both at once within one tensor (pages copied), for rows of whole 16 bytes and of odd sizes."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(width)
+    n = 9
+    src = (torch.randn(n, width, generator=g) * 100).to(dtype).to(DEV)
+    pick = torch.tensor([7, 0, 0, 3], dtype=torch.int32, device=DEV)
+    out = ops.copy_rows(src, torch.zeros(4, width, dtype=dtype, device=DEV), src_rows=pick)
+    assert torch.equal(out, src[pick.long()])
+    place = torch.tensor([5, 1, 8], dtype=torch.int32, device=DEV)
+    dst = torch.full((n, width), 3, dtype=dtype, device=DEV)
+    ops.copy_rows(src, dst, dst_rows=place)
+    want = torch.full((n, width), 3, dtype=dtype, device=DEV)
+    want[place.long()] = src[:3]
+    assert torch.equal(dst, want)
+    both = src.clone()
+    ops.copy_rows(both, both, src_rows=torch.tensor([0, 4], dtype=torch.int32, device=DEV),
+                  dst_rows=torch.tensor([6, 2], dtype=torch.int32, device=DEV))
+    want = src.clone()
+    want[[6, 2]] = src[[0, 4]]
+    assert torch.equal(both, want)
+    # a strided view (rows of a wider tensor), a 1-d tensor as rows of one element, fewer rows than the lists hold
+    if width >= 4 and dtype != torch.bfloat16:
+        view = src[:, :width // 2 * 2][:, :2]
+        assert torch.equal(ops.copy_rows(view, torch.zeros(2, 2, dtype=dtype, device=DEV), src_rows=pick, n=2), view[pick[:2].long()])
+    if width == 1:
+        flat = src[:, 0].contiguous()
+        assert torch.equal(ops.copy_rows(flat, torch.zeros(4, dtype=dtype, device=DEV), src_rows=pick), flat[pick.long()])
+    with pytest.raises(ops.KernelError):
+        ops.copy_rows(src, torch.zeros(2, width, dtype=dtype, device=DEV), src_rows=pick)             # four rows into two
+    if dtype == torch.bfloat16:
+        with pytest.raises(ops.KernelError):
+            ops.copy_rows(src[:, :3].contiguous(), torch.zeros(4, 3, dtype=dtype, device=DEV), src_rows=pick)   # 6-byte rows
+
+
 def test_argmax_first_maximum():
     ops = _ops()
     x = torch.zeros(3, 70001, device=DEV)

@@ -112,8 +112,10 @@ def test_rotary_tables_follow_the_configuration():
     assert np.array_equal(rot.frequencies, inv)
     table = rot.rotation()
     ang = np.arange(300)[:, None] * inv[None]
-    assert np.array_equal(table.cos.cpu().numpy(), np.cos(ang).astype(np.float32))      # float64 angles, rounded once
-    assert table.cos.shape == (300, 16) and not table.interleaved and table.width == 32
+    # float64 angles, rounded once (the tables are shared by everyone with this recipe, so they may be longer than asked)
+    assert np.array_equal(table.cos.cpu().numpy()[:300], np.cos(ang).astype(np.float32))
+    assert np.array_equal(table.sin.cpu().numpy()[:300], np.sin(ang).astype(np.float32))
+    assert table.cos.shape[0] >= 300 and table.cos.shape[1] == 16 and not table.interleaved and table.width == 32
     plain_rot = Rotary(32, 500000.0, None)
     assert not np.array_equal(plain_rot.frequencies, inv)
 
@@ -279,9 +281,18 @@ def _register_toy():
         eps: float
         decay: float
         window: int
-        max_position_embeddings: int
-        initializer_range: float
-        torch_dtype: str = "float32"
+        table_rows: int              # rows of the learned position table: what bounds a sequence here
+        spread: float
+
+        # what the library asks of a configuration; it reads none of the keys above itself
+        def context_length(self):
+            return self.table_rows
+
+        def storage_dtype(self):
+            return "float32"
+
+        def init_std(self):
+            return self.spread
 
         @classmethod
         def from_dict(cls, raw: Mapping[str, Any]):
@@ -289,8 +300,7 @@ def _register_toy():
             vals = dict(architecture=raw["architectures"][0], vocab_size=r.integer("vocab_size"), width=r.integer("width"),
                         heads=r.integer("heads"), kv_heads=r.integer("kv_heads"), head_dim=r.integer("head_dim"),
                         inner=r.integer("inner"), experts=r.integer("experts"), eps=r.number("eps"), decay=r.number("decay"), window=r.integer("window"),
-                        max_position_embeddings=r.integer("max_position_embeddings"),
-                        initializer_range=r.number("initializer_range"))
+                        table_rows=r.integer("table_rows"), spread=r.number("spread"))
             r.finish()
             return cls(**vals)
 
@@ -318,7 +328,7 @@ def _register_toy():
         order = [LayerRun(0), LayerRun(1), LayerRun(2), LayerRun(1), LayerRun(0, reads_cache_of=0)]
         return DecoderModel(cfg, ("embed", emb), layers, ("final_norm", norm()), ("head", OutputHead(cfg.vocab_size, d, emb)),
                             order=order,
-                            position=("positions", make_part("position", "toy_learned", cfg.max_position_embeddings, d)))
+                            position=("positions", make_part("position", "toy_learned", cfg.table_rows, d)))
 
     register_part("mixer", "toy_decay", DecayMixer)
     register_part("feed_forward", "toy_routed", RoutedFeedForward)
@@ -327,7 +337,7 @@ def _register_toy():
 
 
 TOY = {"architectures": ["ToyForCausalLM"], "vocab_size": 90, "width": 48, "heads": 3, "kv_heads": 1, "head_dim": 16, "inner": 72,
-       "experts": 3, "eps": 1e-4, "decay": 0.8, "window": 20, "max_position_embeddings": 256, "initializer_range": 0.15}
+       "experts": 3, "eps": 1e-4, "decay": 0.8, "window": 20, "table_rows": 256, "spread": 0.15}
 
 
 _EXPERTS_SEEN = set()        # the experts that the plain router chose, over all sequences of the test

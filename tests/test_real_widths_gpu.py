@@ -4,7 +4,9 @@ other in reused slots and pages, and the benchmark's decode shapes, against the 
   1b: Llama 3.2 1B (hidden 2048, 32 heads over 8 kv heads of 64, feed-forward 8192, vocabulary 128256, scaling factor 32)
   3b: Llama 3.2 3B layers (hidden 3072, 24 heads over 8 kv heads of 128: three query heads a group, feed-forward 8192)
   8b: Llama 3.1 8B layers (hidden 4096, 32 heads over 8 kv heads of 128, feed-forward 14336, untied head, factor 8)
-The two larger ones have one layer and a vocabulary of 32003 to keep the plain implementation quick."""
+  wide: a hidden size of 5120 (40 heads over 8 kv heads of 128), wider than the streamed products' hand-off of a norm
+        covers: its decode steps take the norm kernels instead
+The larger ones have one layer and a vocabulary of 32003 to keep the plain implementation quick."""
 import numpy as np
 import pytest
 
@@ -27,7 +29,8 @@ WIDE_3B = dict(WIDE, vocab_size=32003, hidden_size=3072, num_hidden_layers=1, nu
 WIDE_8B = dict(WIDE, vocab_size=32003, hidden_size=4096, num_hidden_layers=1, intermediate_size=14336, head_dim=128,
                tie_word_embeddings=False,
                rope_scaling=dict(WIDE["rope_scaling"], factor=8.0))
-SHAPES = {"1b": WIDE, "3b": WIDE_3B, "8b": WIDE_8B}
+WIDE_5120 = dict(WIDE_3B, hidden_size=5120, num_attention_heads=40, intermediate_size=6144)
+SHAPES = {"1b": WIDE, "3b": WIDE_3B, "8b": WIDE_8B, "wide": WIDE_5120}
 
 
 @pytest.fixture(scope="module")
@@ -104,9 +107,10 @@ def test_real_widths_batches_reuse_slots_and_pages(wide, dtype, tol):
 
 
 # -- the benchmark's own decode shapes ------------------------------------------------------------------------------
-# 8 and 64 sequences of the 1B widths with 2,048 to 2,300 cached keys each, then four single-token steps: the first two
+# 1, 8 and 64 sequences of the 1B widths with 2,048 to 2,300 cached keys each, then four single-token steps: the first two
 # run as they are, the third and fourth as a replayed recording.  At batch 8 the decode attention rotates and stores by
-# itself and its pages are dealt to several blocks whose results a second kernel merges; at batch 64 the rotation kernel
+# itself and its pages are dealt to several blocks whose results a second kernel merges (at batch 1 to many more of
+# them, and the products stream their weights against a single row); at batch 64 the rotation kernel
 # reads the QKV product's unsummed runs and the 64x64 tiles do gate/up.  The plain implementation follows a few of the
 # sequences (each whole, in float64); the first one has 2,048 tokens, so its first decoded token opens a new page.
 BENCH_DECODE_STEPS = 4
@@ -130,7 +134,7 @@ def _bench_plain_rows(folder, i):
 
 
 @pytest.mark.parametrize("dtype,tol", [("float32", 3e-5), ("bfloat16", 3e-2)])
-@pytest.mark.parametrize("batch,checked,max_ctx", [(8, (0, 5), 4096), (64, (0, 5, 40), 4096),
+@pytest.mark.parametrize("batch,checked,max_ctx", [(1, (0,), 4096), (8, (0, 5), 4096), (64, (0, 5, 40), 4096),
                                                    # a recorded step is launched for the longest sequence the cache allows:
                                                    # of the blocks that a context of 32,768 gives a sequence, these use one
                                                    (64, (0, 5, 40), 32768)])
@@ -154,3 +158,53 @@ def test_benchmark_decode_shapes(folder_1b, batch, checked, max_ctx, dtype, tol)
             assert (got[i].argmax(-1) == want.argmax(-1)).all()
     eng.close(slots)
     eng.cache.check_consistent()
+
+
+# -- sampling through the generation loop at the real vocabulary ----------------------------------------------------
+def _draw_is_the_plain_one(logits, tok, u, slack, **options):
+    """Whether `tok` is what the plain pipeline draws from these (plain) logits with the uniform u, give or take `slack`
+    of cumulative probability: the engine's logits differ from the plain ones by rounding, and over 128,256 tokens the
+    steps of the cumulative sum are as small as that difference.  Returns (exactly the plain token, within the slack)."""
+    want = plain.sample_token(logits, u, **options)
+    if tok == want:
+        return True, True
+    kept = plain.filtered_logits(logits, **options)
+    if not np.isfinite(kept[tok]):
+        return False, False
+    cum = np.cumsum(plain.softmax(kept))
+    below = cum[tok - 1] if tok > 0 else 0.0
+    return False, below - slack <= u <= cum[tok] + slack
+
+
+@pytest.mark.parametrize("options", [dict(temperature=0.8, top_k=0, top_p=1.0, penalty=1.0),
+                                     dict(temperature=0.7, top_k=40, top_p=0.9, penalty=1.1)],      # the reference's defaults
+                         ids=["temperature alone", "the default filters"])
+def test_sampled_generation_at_the_real_vocabulary(folder_1b, options):
+    """generate() with a temperature alone (a row of 128,256 that nothing cuts goes to 32 blocks and is drawn from their
+    masses) and with the reference's default filters (top-k over 32 blocks), three requests of unequal lengths: every
+    token is the one the plain pipeline draws from the plain logits of the same history with the same uniform number."""
+    import dlgo_amd
+    from dlgo_amd.sampling import uniform
+    cfg, w = plain.read_model(folder_1b)
+    llm = dlgo_amd.load_llm(folder_1b, dtype="float32", max_tokens=1024, max_batch=4)
+    rng = np.random.default_rng(11)
+    prompts = [rng.integers(0, WIDE["vocab_size"], size=n).tolist() for n in (9, 3, 14)]
+    n_new = 5
+    opts = [dlgo_amd.with_temperature(options["temperature"]), dlgo_amd.with_top_k(options["top_k"]),
+            dlgo_amd.with_top_p(options["top_p"]), dlgo_amd.with_repetition_penalty(options["penalty"]), dlgo_amd.with_seed(99),
+            dlgo_amd.with_max_tokens(n_new), dlgo_amd.with_ignore_eos()]
+    results = llm.generate(prompts, *opts)
+    again = llm.generate(prompts, *opts)
+    assert [r.tokens for r in results] == [r.tokens for r in again]
+    exact = total = 0
+    for i, (p, r) in enumerate(zip(prompts, results)):
+        assert len(r.tokens) == n_new
+        seq = list(p)
+        for step, tok in enumerate(r.tokens):
+            logits = plain.forward(cfg, w, seq, rows=[len(seq) - 1])[0]
+            same, near = _draw_is_the_plain_one(logits, tok, uniform(99, i, step), 3e-5, recent=r.tokens[:step][-64:], **options)
+            assert near, (i, step, tok)
+            exact += same
+            total += 1
+            seq.append(tok)
+    assert exact >= 0.6 * total, f"only {exact} of {total} tokens are the plain ones exactly: the slack decides too often"
