@@ -3,12 +3,15 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--dtype bf16|fp32]
 
-A step is one decode step of the whole batch: greedy choice of the next tokens on
-the device, the step function on those tokens, and the ids' return to the host
-(what the generation loop does per step, in its order).  Random weights, seeded
-uniform-random token ids, no stop tokens.  The K timed steps run as five regions,
-each between two waits for the device; the figures are the median region's.
-Prints ONE JSON line.
+A step is one decode step of the whole batch as the library's own generation loop
+runs it (dlgo_amd.engine.generate): greedy choice of the next tokens on the device,
+the step function on those tokens, the ids' return to the host.  The loop times
+every step itself (Stats.step_ms, as computerex/dlgo's loop does,
+models/llm/generate.go:227-229,275-282): after W warm-up steps the next K steps
+are the timed ones, taken as five regions; the figures are the median region's.
+Random weights, seeded uniform-random token ids, no stop tokens.  Prints ONE JSON
+line.  --breakdown adds "kernels": the time of every launch of one decode step,
+by kind, made one by one between events (gpu_timing_main.go:73-119).
 
 Peaks used for the fractions (MI355X, published): HBM 8 TB/s; dense MFMA bf16
 2.5 PFLOP/s, fp32 157.3 TFLOP/s.
@@ -113,6 +116,48 @@ def ragged(args, cfg, full_layers, elem) -> int:
     return 0
 
 
+def breakdown(eng, sampler, cfg, batch, rng, steps=8):
+    """One decode step of `batch` sequences, launch by launch: the same launches a recorded step replays, made one by
+    one with an event before and after each.  So that the device does not wait for the host between them, every step
+    is queued behind a fill of several gigabytes that keeps the device busy meanwhile (and leaves the caches cold, as
+    the weights of the layers before leave them in a real step); "event_pair" is what two events with nothing between
+    them measure, which is taken off every bracket.  Returns {kind of launch: [microseconds a step, launches a step]},
+    their sum, the launches of a step and the events' share."""
+    import torch
+
+    from dlgo_amd.engine import Entry
+    from dlgo_amd.kernels import ops
+    from dlgo_amd.sampling import SamplerConfig
+    prompts = [rng.integers(0, cfg.vocab_size, size=PROMPT).tolist() for _ in range(batch)]
+    slots = eng.open(batch)
+    greedy = [SamplerConfig(temperature=0.0)] * batch
+    logits = eng.step([Entry(s, p, [PROMPT - 1]) for s, p in zip(slots, prompts)])
+    for _ in range(2):
+        logits = eng.decode(slots, sampler.choose_device(logits, greedy, [0.0] * batch), replay=False)
+    ballast = torch.empty(6 << 30, dtype=torch.uint8, device=eng.device)
+    torch.cuda.synchronize()
+    pairs = []
+    with ops.Timings() as t:
+        for _ in range(steps):
+            ballast.fill_(1)
+            logits = eng.decode(slots, sampler.choose_device(logits, greedy, [0.0] * batch), replay=False)
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            b.record()
+            pairs.append((a, b))
+            torch.cuda.synchronize()
+    us, n = t.microseconds(), t.launches()
+    eng.close(slots)
+    del ballast
+    pair = sum(a.elapsed_time(b) for a, b in pairs) * 1000.0 / len(pairs)
+    # per kind: microseconds a step with the events' own share taken off, and the launches a step
+    out = {k: [round(max(0.0, v / steps - n[k] / steps * pair), 1), n[k] // steps] for k, v in sorted(us.items(), key=lambda kv: -kv[1])}
+    out["sum"] = round(sum(v[0] for v in out.values()), 1)
+    out["launches"] = sum(n.values()) // steps
+    out["event_pair"] = round(pair, 2)
+    return out
+
+
 def main() -> int:
     global PROMPT, CONTEXT
     ap = argparse.ArgumentParser()
@@ -125,6 +170,8 @@ def main() -> int:
     ap.add_argument("--points", default="1,64", help="other batch sizes to report, comma separated ('' = none)")
     ap.add_argument("--point-steps", type=int, default=64)
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--breakdown", action="store_true",
+                    help="add \"kernels\": microseconds of one decode step of --batch by kind of launch, each launch timed between events")
     ap.add_argument("--ragged", default="", metavar="N:LO:HI:NEW:CTX",
                     help="instead of the default run: N requests with prompts of LO..HI tokens (uniform, seeded), NEW "
                          "generated tokens each, context CTX, through the generation loop")
@@ -142,8 +189,10 @@ def main() -> int:
 
     from dlgo_amd import models  # noqa: F401
     from dlgo_amd.config import config_from_dict
-    from dlgo_amd.engine import Engine, Entry
+    from dlgo_amd.engine import Engine
+    from dlgo_amd.engine.generate import generate
     from dlgo_amd.sampling import Sampler, SamplerConfig
+    from dlgo_amd.sampling.options import GenerateConfig
 
     raw = dict(SHAPES[args.shape])
     full_layers = raw["num_hidden_layers"]
@@ -163,37 +212,28 @@ def main() -> int:
                              max_step_tokens=8192, graph_max_batch=max(most, 8))
     sampler = Sampler(eng.vocab, eng.device, max_rows=most)
     rng = np.random.default_rng(0)
-    greedy = SamplerConfig(temperature=0.0)
+
+    def conf(new_tokens):
+        return GenerateConfig(max_tokens=new_tokens, sampler=SamplerConfig(temperature=0.0), seed=1, ignore_eos=True)
 
     def decode(batch, steps, warmup):
+        """`warmup` + `steps` decode steps of `batch` sequences through the generation loop; the loop's own times of the
+        last `steps` of them.  A short run first, so that the step of this batch size is recorded before the run that
+        counts (the loop runs a size as it is twice, then records it)."""
         prompts = [rng.integers(0, cfg.vocab_size, size=PROMPT).tolist() for _ in range(batch)]
-        slots = eng.open(batch)
-        logits = eng.step([Entry(s, p, [PROMPT - 1]) for s, p in zip(slots, prompts)])
-        # the generation loop's own order (engine/generate.py, _decode_batch): choose on the device, queue the next
-        # step with the ids still on the device, then bring the ids of the step before to the host
-        state = {"logits": logits}
-
-        def one():
-            tok_dev, wait = sampler.choose_async(state["logits"], [greedy] * batch, [0.0] * batch)
-            state["logits"] = eng.decode(slots, tok_dev)
-            state["tokens"] = wait()
-        for _ in range(warmup):
-            one()
-        torch.cuda.synchronize()
-        c0 = eng.length(slots[0])
-        # exactly `steps` timed steps, in REGIONS regions of (nearly) equal length, each between two waits for the device;
-        # the figure is the median region's time per step
+        generate(eng, sampler, prompts, [conf(4)] * batch, max_batch=batch, sync=torch.cuda.synchronize)
+        # the first token comes from the prompt step; every further one is a decode step
+        _, st = generate(eng, sampler, prompts, [conf(warmup + steps + 1)] * batch, max_batch=batch, sync=torch.cuda.synchronize)
+        times = st.step_ms[1:]                       # [0] is the prompt step
+        assert len(times) == warmup + steps + 1, (len(times), warmup, steps)
+        timed = times[warmup:warmup + steps]         # the last entry is the loop's final turn, which runs no step
         n_regions = REGIONS if steps >= REGIONS else 1
         sizes = [steps // n_regions + (1 if r < steps % n_regions else 0) for r in range(n_regions)]
-        per_step = []
+        per_step, o = [], 0
         for size in sizes:
-            t0 = time.perf_counter()
-            for _ in range(size):
-                one()
-            torch.cuda.synchronize()
-            per_step.append((time.perf_counter() - t0) / size)
-        eng.close(slots)
-        mean_ctx = c0 + (steps + 1) / 2.0       # keys a step reads per sequence, averaged over the timed steps
+            per_step.append(sum(timed[o:o + size]) / size / 1000.0)
+            o += size
+        mean_ctx = PROMPT + warmup + (steps + 1) / 2.0       # keys a step reads per sequence, averaged over the timed steps
         return statistics.median(per_step), mean_ctx, per_step
 
     # the other batch sizes first: the headline figure is then taken on a device that has been working for a while
@@ -210,18 +250,17 @@ def main() -> int:
     prefill = None
     if not args.no_prefill:
         times = []
-        for i in range(6):
+        for i in range(6):       # the loop's own time of the prompt step (it waits for the device before and after)
             prompt = rng.integers(0, cfg.vocab_size, size=PROMPT).tolist()
-            (slot,) = eng.open(1)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            eng.step([Entry(slot, prompt, [PROMPT - 1])])
-            torch.cuda.synchronize()
-            times.append(time.perf_counter() - t0)
-            eng.close([slot])
+            _, st = generate(eng, sampler, [prompt], [conf(1)], max_batch=1, sync=torch.cuda.synchronize)
+            times.append(st.prefill_ms / 1000.0)
         pt = statistics.median(times[1:])
         prefill = {"value": round(PROMPT / pt, 1), "tokens": PROMPT, "ms": round(pt * 1000.0, 3),
                    "frac": round(prefill_flops(cfg, PROMPT) / pt / FLOP_PEAK[args.dtype], 4)}
+
+    kernels = None
+    if args.breakdown:
+        kernels = breakdown(eng, sampler, cfg, args.batch, rng)
 
     line = {
         "metric": f"decode tok/s @ batch {args.batch} ({args.shape} shape, {PROMPT}-token prompts, context {CONTEXT})",
@@ -233,7 +272,7 @@ def main() -> int:
                    "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
                    "tied_embeddings": cfg.tie_word_embeddings, "global_batch": args.batch, "seq_len": CONTEXT,
                    "prompt_len": PROMPT, "parallelism": "single-gpu", "kv_cache_dtype": args.dtype,
-                   "sampling": "greedy on device, tokens returned to the host each step"},
+                   "sampling": "greedy, through the generation loop"},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK, 4)},
         "points": points,
@@ -241,6 +280,8 @@ def main() -> int:
     }
     if prefill is not None:
         line["prefill"] = prefill
+    if kernels is not None:
+        line["kernels"] = kernels
     print(json.dumps(line))
     return 0
 

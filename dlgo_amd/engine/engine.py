@@ -430,10 +430,12 @@ class Engine:
             "cu_q": np.arange(b + 1, dtype=np.int32),
         }
 
-    def decode(self, slots: Sequence[int], tokens, checked: bool = False) -> torch.Tensor:
+    def decode(self, slots: Sequence[int], tokens, checked: bool = False, replay: bool = True) -> torch.Tensor:
         """One token for each of `slots`, logits [len(slots), vocab] for each (a view that the next decode or step
         overwrites).  `tokens` are ids on the host, or an int32 tensor on the device in the order of `slots`
-        (the sampler's output: the ids need not come to the host before the next step starts)."""
+        (the sampler's output: the ids need not come to the host before the next step starts).  replay=False: the
+        step's launches are made one by one, the same ones a recording of this batch size holds, and nothing is
+        recorded (for timing them)."""
         b = len(slots)
         slot_arr = np.asarray(slots, dtype=np.int64)
         on_device = isinstance(tokens, torch.Tensor)
@@ -466,7 +468,7 @@ class Engine:
             out = torch.empty((b, self.vocab), dtype=torch.float32, device=self.device)
             for c0 in range(0, b, self.graph_max_batch):
                 c1 = min(b, c0 + self.graph_max_batch)
-                out[c0:c1].copy_(self.decode(slots[c0:c1], tokens[c0:c1], checked=True))
+                out[c0:c1].copy_(self.decode(slots[c0:c1], tokens[c0:c1], checked=True, replay=replay))
             return out
         if needs_pages:
             self.cache.reserve([(int(s), int(st) + 1) for s, st in zip(slot_arr, starts)])
@@ -478,7 +480,7 @@ class Engine:
         if on_device:
             arrays["token_ids"].copy_(tokens)
         logits = self._static_logits[:b]
-        g = self._graphs.get(b) if self.use_graphs else None
+        g = self._graphs.get(b) if self.use_graphs and replay else None
         if g is not None:
             g.graph.replay()
         else:
@@ -490,8 +492,8 @@ class Engine:
             x = self.model.hidden(ctx, ctx.token_ids, all_rows_wanted=True)
             self.model.logits(ctx, x, None, logits)
             # the second time a batch size is seen it is worth capturing
-            self._graph_seen[b] = self._graph_seen.get(b, 0) + 1
-            if self.use_graphs and self._graph_seen[b] >= 2:
+            self._graph_seen[b] = self._graph_seen.get(b, 0) + (1 if replay else 0)
+            if self.use_graphs and replay and self._graph_seen[b] >= 2:
                 self._capture(b, ctx, logits)
         self.cache.advance_many(slot_arr, 1)
         self.steps_run += 1

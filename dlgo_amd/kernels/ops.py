@@ -6,8 +6,9 @@ GPU or the compiler they raise.
 from __future__ import annotations
 
 import ctypes
+import functools
 import math
-from typing import Optional, Sequence
+from typing import Dict, List, Optional, Sequence
 
 import torch
 
@@ -691,3 +692,66 @@ def sample(logits: torch.Tensor, work: torch.Tensor, temperature: torch.Tensor, 
                                         _ptr(recent_rows), _ptr(counts), _ptr(uniform), _ptr(out), int(bool(dealt_rows)),
                                         _stream()))
     return out
+
+
+# ---------------------------------------------------------------------------
+# Timing the launches one by one (what computerex/dlgo's gpu_timing_main.go:73-119 does for its operations): inside a
+# `with Timings() as t:` block every face above that launches something is bracketed by two events on the current
+# stream; t.microseconds() then gives, per label, the time between them summed over the block.  A product's label
+# carries its weight's shape, which is what tells the products of a layer apart.  The steps inside the block must run
+# as they are (a replayed recording calls no face).  Outside such a block a face costs one comparison more.
+_recorder: Optional[list] = None
+
+
+class Timings:
+    def __enter__(self) -> "Timings":
+        global _recorder
+        self.events: List[tuple] = []
+        self._outer, _recorder = _recorder, self.events
+        return self
+
+    def __exit__(self, *exc) -> None:
+        global _recorder
+        _recorder = self._outer
+
+    def microseconds(self) -> Dict[str, float]:
+        torch.cuda.synchronize()
+        out: Dict[str, float] = {}
+        for label, start, end in self.events:
+            out[label] = out.get(label, 0.0) + start.elapsed_time(end) * 1000.0
+        return out
+
+    def launches(self) -> Dict[str, int]:
+        out: Dict[str, int] = {}
+        for label, _, _ in self.events:
+            out[label] = out.get(label, 0) + 1
+        return out
+
+
+def _timed(fn):
+    name = fn.__name__
+    by_weight = name.startswith("gemm")
+
+    @functools.wraps(fn)
+    def face(*args, **kwargs):
+        rec = _recorder
+        if rec is None:
+            return fn(*args, **kwargs)
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        result = fn(*args, **kwargs)
+        end.record()
+        if result is False or (result is None and name == "gemm_runs"):
+            return result                # it declined: nothing was launched
+        label = name
+        if by_weight and args and isinstance(args[0], torch.Tensor):
+            label = f"{name}[{args[0].shape[0]}x{args[0].shape[1]}]"
+        rec.append((label, start, end))
+        return result
+    return face
+
+
+for _name in ("embed", "copy_rows", "rmsnorm", "bias_add", "head_rmsnorm", "gemm_accum_then_norm", "gemm_runs", "gemm", "gemm_rmsnorm",
+              "gemm_accum_leave_norm", "gemm_scaled", "rope_kv", "attention", "argmax", "sample"):
+    globals()[_name] = _timed(globals()[_name])
+del _name
