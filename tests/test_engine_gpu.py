@@ -232,6 +232,73 @@ def test_thousands_of_tokens(tmp_path, dtype):
     eng.cache.check_consistent()
 
 
+# -- tens of thousands of tokens ------------------------------------------------------------------------------------
+# Two layers of Tiny B's widths with positions up to 32,768 and a scaling recipe whose original length is 1,024: at
+# 20,000 tokens a sequence holds 313 pages, a decode step deals them to many blocks (more than a context of a few
+# thousand tokens ever gives), and every rotary pair is far into the regime its wavelength puts it in.  Eight
+# sequences of 100 to 20,000 tokens; the plain implementation follows each whole, once: the folder holds bfloat16
+# weights, which a float32 run reads exactly, so both run dtypes have the same model before them.
+FAR = dict(TINY_B, max_position_embeddings=32768, num_hidden_layers=2, num_key_value_heads=2,
+           rope_scaling={"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+                         "original_max_position_embeddings": 1024})
+FAR_LENS = [20000, 100, 300, 1000, 2100, 4200, 8300, 12000]
+FAR_DECODE = 8
+
+
+@pytest.fixture(scope="module")
+def far(tmp_path_factory):
+    folder = make_folder(FAR, seed=6, path=tmp_path_factory.mktemp("far"), dtype="bfloat16", norm_jitter=0.1, std=0.08)
+    cfg, w = plain.read_model(str(folder))
+    rng = np.random.default_rng(14)
+    seqs = [rng.integers(1, FAR["vocab_size"], size=n + FAR_DECODE).tolist() for n in FAR_LENS]
+    for at in (3, 9000, 19990, 20003):          # one rare token far back and near the end: late queries lean on far keys
+        seqs[0][at] = 0
+    # the prompt's last two rows and every decoded row
+    want = [plain.forward(cfg, w, t, rows=range(n - 2, n + FAR_DECODE)) for t, n in zip(seqs, FAR_LENS)]
+    return str(folder), seqs, want
+
+
+def _prompt_then_tokens(eng, slots, seqs, lens, want, tol, what):
+    from dlgo_amd.engine import Entry
+    first = eng.step([Entry(s, t[:n], [n - 2, n - 1]) for s, t, n in zip(slots, seqs, lens)]).cpu().numpy()
+    for j in range(len(slots)):
+        assert rel_err(first[2 * j:2 * j + 2], want[j][:2]) <= tol, (what, "prompt", j)
+    for i in range(FAR_DECODE):          # the first two steps run as they are, the others are a replayed recording
+        out = eng.step([Entry(s, [t[n + i]], [0]) for s, t, n in zip(slots, seqs, lens)]).cpu().numpy()
+        for j in range(len(slots)):
+            assert rel_err(out[j], want[j][2 + i]) <= tol, (what, "token", i, "sequence", j)
+    assert len(slots) in eng._graphs, "the last steps were meant to be replayed"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_one_sequence_of_twenty_thousand_tokens(far, dtype):
+    folder, seqs, want = far
+    tol = 5e-5 if dtype == "float32" else TOL[dtype]
+    eng = engine_for(folder, dtype, max_tokens=20480, max_ctx=24576, max_step_tokens=2048)     # the prompt goes in ten pieces
+    slots = eng.open(1)
+    _prompt_then_tokens(eng, slots, seqs[:1], FAR_LENS[:1], want[:1], tol, dtype)
+    assert eng.length(slots[0]) == 20000 + FAR_DECODE and len(eng.cache.held_pages(slots[0])) == 313
+    eng.close(slots)
+    eng.cache.check_consistent()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_batch_of_lengths_from_a_hundred_to_twenty_thousand(far, dtype):
+    """One launch serves sequences that hold 2 pages and 313: each uses as many of the grid's blocks as its own pages
+    call for.  The sequences are given in an order that is not the order of their lengths."""
+    folder, seqs, want = far
+    tol = 5e-5 if dtype == "float32" else TOL[dtype]
+    held = sum((n + FAR_DECODE + 63) // 64 * 64 for n in FAR_LENS)
+    eng = engine_for(folder, dtype, max_tokens=held, max_ctx=32768, max_step_tokens=4096, max_slots=8)
+    order = [3, 0, 7, 1, 5, 2, 6, 4]
+    slots = eng.open(8)
+    pick = lambda xs: [xs[i] for i in order]
+    _prompt_then_tokens(eng, slots, pick(seqs), pick(FAR_LENS), pick(want), tol, dtype)
+    assert eng.free_pages() == (0,)
+    eng.close(slots)
+    eng.cache.check_consistent()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_more_sequences_than_a_recorded_step_takes(folders, oracle, dtype):
     """150 sequences that start together and go on one token at a time: more than the largest batch for which single
