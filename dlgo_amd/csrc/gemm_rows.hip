@@ -657,17 +657,35 @@ static int stream_waves(int Tn, int K, int ldw, int* turns = nullptr) {
   return 0;
 }
 
+// The compute units of the current device (asked once; 256 on the chip this is written for).
+static int compute_units() {
+  static int cus = 0;
+  if (cus <= 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
+    else cus = 256;
+  }
+  return cus;
+}
+
+// Rows that a wave takes in several turns, or whose kilobytes are 5 or 7, go to the kernel with one group of rows a block.
+static bool stream_is_long(int nw, int turns) { return turns > 1 || nw == 5 || nw == 7; }
+
+// A block takes up to four groups of 16 rows in turn, which share its operands of X (and the work on the norm): as many
+// as leave blocks for at least five eighths of the compute units (a function of N alone).  Measured with 1 to 16 tokens
+// on matrices of 2,048 to 128,256 rows of 4 to 8 KB: fewer blocks than that cost more than the shared work saves; with
+// more, four groups are 5 to 25% faster than one on the wide matrices and two on those of 5,000 to 6,000 rows.
+static int stream_groups(int N, bool is_long) {
+  const int blocks1 = (N + 15) / 16, fill = compute_units() * 5 / 8;
+  return is_long ? 1 : (blocks1 >= 4 * fill ? 4 : (blocks1 >= 2 * fill ? 2 : 1));
+}
+
 template <typename T, int EPI, bool NORM, int MODE = 0>
 static const char* launch_skinny_stream(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K,
                                         int ldw, int ldx, int ldy, int nw, hipStream_t stream, NormParts np = NormParts{},
                                         int turns = 1) {
-  const bool is_long = turns > 1 || nw == 5 || nw == 7;
-  // A block takes up to four groups of 16 rows in turn, which share its operands of X (and the work on the norm): as
-  // many as leave at least 160 blocks, five eighths of the compute units (a function of N alone).  Measured on the
-  // shapes of 1B to 8B Llamas, 1 to 16 tokens: fewer blocks than that cost more than the shared work saves; with more,
-  // four groups are 5 to 25% faster than one on the wide matrices (gate/up, vocabulary) and two on QKV of 5,120 and 6,144 rows.
-  const int blocks1 = (N + 15) / 16;
-  const int groups = is_long ? 1 : (blocks1 >= 4 * 160 ? 4 : (blocks1 >= 2 * 160 ? 2 : 1));
+  const bool is_long = stream_is_long(nw, turns);
+  const int groups = stream_groups(N, is_long);
   dim3 g((N + 16 * groups - 1) / (16 * groups));
   // a wave's LDS: 16 KB of W and, with the norm, a kilobyte of column operands per token
   const int lds = nw * (16384 + (NORM ? Tn * 1024 : 0));
@@ -874,6 +892,20 @@ extern "C" const char* dlgo_gemm_rmsnorm(const void* W, const float* X, const fl
 // kilobytes.  role 0: the plain product; 1: as dlgo_gemm_rows_leave_parts, which leaves a share of the sums of squares
 // for every 16 of its N columns; 2: as dlgo_gemm_rows_scaled, which adds up the shares of the K columns it reads.  Both
 // hold at most NORM_PARTS_MAX shares a row, so a normed width beyond 16 * NORM_PARTS_MAX is not theirs.
+// How the streamed products would take a weight [N, K] with Tn rows of X: waves a block, the kilobytes of a row each wave
+// takes in turn, and the groups of 16 weight rows a block works through (which share its reads of X).  Returns 0, with
+// nothing written, if they do not take it.
+extern "C" int dlgo_gemm_rows_stream_plan(int dtype, int N, int Tn, int K, int ldw, int* waves, int* turns, int* groups) {
+  int t = 1;
+  if (dtype != DLGO_ELEM || N <= 0) return 0;
+  const int nw = stream_waves<elem_t>(Tn, K, ldw, &t);
+  if (nw <= 0) return 0;
+  *waves = nw;
+  *turns = t;
+  *groups = stream_groups(N, stream_is_long(nw, t));
+  return 1;
+}
+
 extern "C" int dlgo_gemm_rows_streams(int dtype, int N, int Tn, int K, int ldw, int role) {
   int turns = 1;
   if (dtype != DLGO_ELEM || N <= 0 || stream_waves<elem_t>(Tn, K, ldw, &turns) <= 0) return 0;

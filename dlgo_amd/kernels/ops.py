@@ -20,7 +20,7 @@ EPI_STORE, EPI_ACCUM_F32, EPI_SWIGLU, EPI_STORE_F32 = 0, 1, 2, 3
 GEMM_AUTO, GEMM_STREAM, GEMM_TILE128, GEMM_TILE64, GEMM_TILE32, GEMM_ROWS16 = 0, 1, 2, 3, 4, 5
 GEMM_FEW_ROWS = 64      # up to this many rows of x the weight-streaming kernels can be chosen
 GEMM_SPLIT_FLOATS = 1 << 22   # scratch that lets gemm() share the inner size of a product out over blocks
-GEMM_VERY_WIDE = 65536   # from this many weight rows on (a vocabulary) the tiled kernel is faster for any number of rows of x
+GEMM_VERY_WIDE = 65536   # from this many weight rows on (a vocabulary: 16 blocks of 16 rows for each of 256 compute units) the tiled kernel is faster for any number of rows of x
 GEMM_FEW_ROWS_WIDE = 16  # ... and up to this many when the weight has very many rows (there the tiled kernel is faster)
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
@@ -178,23 +178,75 @@ def head_rmsnorm(x: torch.Tensor, first_col: int, n_heads: int, head_dim: int, w
     return x
 
 
+_cus: dict = {}
+
+
+def compute_units(device=None) -> int:
+    """Compute units of the device (256 on an MI355X): what the rules below count blocks against."""
+    index = torch.cuda.current_device() if device is None else torch.device(device).index or 0
+    if index not in _cus:
+        _cus[index] = torch.cuda.get_device_properties(index).multi_processor_count
+    return _cus[index]
+
+
+def stream_plan(weight: torch.Tensor, t: int):
+    """(waves a block, kilobytes of a row a wave takes in turn, groups of 16 weight rows a block works through) of the
+    streamed products for this weight and t rows of x, or None if they do not take it."""
+    if weight.dim() != 2 or weight.stride(1) != 1 or not (1 <= t <= 16):
+        return None
+    lib = _lib("gemm_rows", (("DLGO_ELEM", dtype_code(weight.dtype)),))
+    lib.dlgo_gemm_rows_stream_plan.restype = ctypes.c_int
+    waves, turns, groups = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+    ok = lib.dlgo_gemm_rows_stream_plan(dtype_code(weight.dtype), weight.shape[0], t, weight.shape[1], weight.stride(0),
+                                        ctypes.byref(waves), ctypes.byref(turns), ctypes.byref(groups))
+    return (waves.value, turns.value, groups.value) if ok else None
+
+
 def _streams_rows(weight: torch.Tensor, t: int, kind: int, has_scratch: bool, splits: int) -> bool:
-    """Whether a product of t rows with this weight goes to the weight-streaming kernels (else to the tiled ones)."""
+    """Whether a product of t rows with this weight goes to the kernels that stream W against a few rows of x (else to
+    the tiled ones).  The rules count bytes, blocks and rows, not the sizes of a model:
+
+      row_bytes  what a block reads of one weight row; in 128-byte pieces the tiles can load it straight into LDS, and
+                 from 32 pieces (4 KB) on they can share k out over blocks, given scratch (`can_split`);
+      blocks16   blocks of the streamed kernels (16 weight rows each), tiles64 those of the small tiles (64 rows each),
+                 both against the device's compute units.
+
+    Up to 16 rows stream, except: (a) so few blocks that compute units stay idle and rows long enough to share out
+    (the split tiles use every unit); (b) rows that a wave takes in several turns, from 8 rows of x on, where k can be
+    shared out (the streamed kernel for such rows has one group of weight rows a block, and every block reads all of
+    x again: with 10 KB rows and 8 rows of x the split tiles are 10 to 30% faster, with 40 KB rows also for one row);
+    (c) a matrix with 16 and more blocks a unit (a vocabulary), which streams only with up to 8 rows and a wave per
+    kilobyte of a row, or when the tiles cannot load its rows.  17 to 64 rows go to the kernel that reads W into
+    registers only where the tiles are few and cannot split."""
     n, k = weight.shape
-    # k in 128-byte pieces, if it is a whole number of them (what the kernels that load tiles straight into LDS take)
-    piece = 128 // weight.element_size()
-    nk = k // piece if k % piece == 0 else 0
-    can_split = has_scratch and splits != 1 and nk >= 32
+    es = weight.element_size()
+    row_bytes = k * es
+    pieces = row_bytes // 128 if row_bytes % 128 == 0 else 0
+    can_split = has_scratch and splits != 1 and pieces >= 32
     if kind != GEMM_AUTO or splits > 1:
         return kind in (GEMM_STREAM, 5, 6, 7, 8, 9, 10, 11)
-    if t <= GEMM_FEW_ROWS_WIDE:         # measured on the shapes of a 1B Llama: a long inner size is better split,
-        row_kb = k * weight.element_size() / 1024.0
-        if t <= 8 and n >= GEMM_VERY_WIDE and row_kb in (2.0, 3.0, 4.0, 6.0, 8.0):
-            return True                 # a vocabulary of rows that go through LDS whole: streamed faster than tiled
-        return not (can_split and n <= 4096 and nk >= 64) and not (n >= GEMM_VERY_WIDE and nk > 0)   # else a vocabulary is better tiled
-    if t <= GEMM_FEW_ROWS:              # measured on the shapes of 1B, 3B and 8B Llamas: up to 128 tiles of 64x64 split k
-        return n < 16384 and not (can_split and n <= 8192 and (nk >= 48 or t >= 24)) and (t <= 40 or nk == 0)
+    cus = compute_units(weight.device)
+    blocks16, tiles64 = (n + 15) // 16, (n + 63) // 64
+    very_wide = blocks16 >= 16 * cus
+    if t <= GEMM_FEW_ROWS_WIDE:
+        plan = stream_plan(weight, t)
+        waves, turns, groups = plan if plan is not None else (0, 1, 1)
+        if very_wide:                                                                       # (c)
+            return pieces == 0 or (t <= 8 and plan is not None and turns == 1 and waves not in (5, 7))
+        if can_split and blocks16 <= cus and pieces >= 64:                                  # (a)
+            return False
+        if can_split and plan is not None and turns > 1 and (t >= 8 or pieces >= 256):      # (b)
+            return False
+        return True
+    if t <= GEMM_FEW_ROWS:
+        return blocks16 < 4 * cus and not (can_split and tiles64 <= cus // 2 and (pieces >= 48 or t >= 24)) and (t <= 40 or pieces == 0)
     return False
+
+
+def gemm_streams(weight: torch.Tensor, rows: int, has_scratch: bool = True) -> bool:
+    """Which family gemm() gives a product of `rows` rows of x with this weight when the choice is its own: the kernels
+    that stream W against a few rows (True) or the tiled ones (False).  The rules are _streams_rows'."""
+    return _streams_rows(weight, rows, GEMM_AUTO, has_scratch, 0)
 
 
 def gemm_accum_then_norm(weight: torch.Tensor, x: torch.Tensor, residual: torch.Tensor, scratch: Optional[torch.Tensor],
@@ -510,13 +562,17 @@ def attention_rows(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, 
 
 
 def attention_fuses_rotation(dtype: torch.dtype, head_dim: int, group: int, max_q_len: int, rot_width: int,
-                             n_seq: int = 1) -> bool:
+                             n_seq: int = 1, n_kv: int = 8) -> bool:
     """True if attention() should rotate the queries and take in the new keys and values itself for such a step:
-    one row per sequence, bfloat16, a rotated width that is a multiple of 16 or no rotation at all, few enough
-    sequences that a kernel launch costs more than the rotation repeated in every wave, and heads small enough that
-    the kernel keeps eight waves to a block (measured: at a head size of 128 the kernel of its own is faster)."""
-    return (dtype == torch.bfloat16 and head_dim <= 64 and group <= 128 and max_q_len == 1 and rot_width % 16 == 0
-            and n_seq <= 32)
+    one row per sequence, bfloat16, a rotated width that is a multiple of 16 or no rotation at all; at most one
+    (sequence, kv head) pair for every compute unit, so that a kernel launch costs more than the rotation repeated in
+    every wave (with 8 kv heads on 256 units: up to 32 sequences; measured at 64: 62 against 9 + 52 us), and no more
+    than 32 sequences whatever the heads (the largest step the fused variant is tested with); and heads small enough
+    that eight waves of a block each keep a page (keys and values of 64 tokens) in 128 KB of LDS (at a head size of 128
+    the kernel of its own is faster)."""
+    page_bytes = 2 * PAGE * head_dim * 2
+    return (dtype == torch.bfloat16 and 8 * page_bytes <= 128 * 1024 and group <= 128 and max_q_len == 1 and rot_width % 16 == 0
+            and n_seq * n_kv * ((group + 15) // 16) <= compute_units() and n_seq <= 32)
 
 
 def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, positions: torch.Tensor,

@@ -162,7 +162,7 @@ class Attention(Mixer):
         rot = self.position.rotation()
         # a step of single tokens: the attention kernel rotates and stores by itself; else a kernel of its own does
         fused = not self._between and ops.attention_fuses_rotation(ctx.dtype, self.head_dim, self.n_heads // self.n_kv_heads,
-                                                                   ctx.max_q_len, rot.width if rot else 0, ctx.n_seq)
+                                                                   ctx.max_q_len, rot.width if rot else 0, ctx.n_seq, self.n_kv_heads)
         unsummed = None
         if isinstance(xn, ops.UnscaledNorm):   # the norm's factor is applied to the product's sums
             ops.gemm_scaled(self.w_qkv[:cols], xn, qkv[:, :cols])

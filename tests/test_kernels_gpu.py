@@ -428,6 +428,44 @@ def test_norm_left_and_applied_by_tiled_products(dtype, _, rel, n1, k1, n2, t):
         ops.gemm_scaled(w2, left, torch.empty(t, n2, device=DEV), ops.EPI_STORE_F32)
 
 
+# the products of decoders with hidden sizes of 2,048 (a vocabulary of 128,256), 2,560 and 5,120, the latter two being
+# widths the kernels were not tuned on: rows of 5 KB (five waves a block), 10, 20 and 40 KB (several turns a wave)
+CHOICES = [
+    # n, k, rows of x, streamed?
+    (3072, 2048, 8, True), (2048, 2048, 16, True), (16384, 2048, 16, True),
+    (2048, 8192, 8, False),            # few blocks and 16 KB rows: k is shared out over the split tiles
+    (128256, 2048, 8, True), (128256, 2048, 9, False),
+    (3840, 2560, 8, True), (2560, 2560, 16, True), (20480, 2560, 8, True),
+    (2560, 10240, 1, False),           # few blocks, 20 KB rows
+    (128256, 2560, 1, False),          # a vocabulary streams only with a wave per kilobyte of a row
+    (7680, 5120, 4, True), (7680, 5120, 8, False), (5120, 5120, 16, False),     # 10 KB rows: from 8 rows of x on, tiles
+    (5120, 20480, 1, False),           # 40 KB rows: tiles for any number of rows
+    (40960, 5120, 8, False), (40960, 5120, 1, True),
+    (128256, 5120, 1, False),
+    (3072, 2048, 32, False), (2056, 1032, 32, True),      # 17 to 64 rows: tiles, unless they cannot load the rows
+]
+
+
+@pytest.mark.parametrize("n,k,t,streamed", CHOICES)
+def test_the_choice_of_product_kernel_follows_bytes_and_blocks(n, k, t, streamed):
+    """gemm()'s own choice between streaming W and tiles, stated for the products of three decoders, two of them of
+    widths no kernel was tuned on; and whatever it chooses is the product."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(n + k + t)
+    w = (torch.randn(n, k, generator=g) * 0.05).to(torch.bfloat16).to(DEV)
+    x = torch.randn(t, k, generator=g).to(torch.bfloat16).to(DEV)
+    assert ops.compute_units(DEV) == 256, "the table above is for 256 compute units"
+    assert ops.gemm_streams(w, t) is streamed
+    scratch = torch.empty(ops.GEMM_SPLIT_FLOATS, device=DEV)
+    out = torch.empty(t, n, device=DEV)
+    ops.gemm(w, x, out, ops.EPI_STORE_F32, scratch=scratch)
+    want = x.double() @ w.double().T
+    close(out, want, 2e-3, "the chosen kernel")
+    acc = torch.ones(t, n, device=DEV)
+    ops.gemm(w, x, acc, ops.EPI_ACCUM_F32, scratch=scratch)
+    close(acc, want + 1.0, 2e-3, "the chosen kernel, adding")
+
+
 def test_gemm_reference_vectors():
     """blas/blas_test.go:21-64: identity, [[1,2],[3,4]]·[1,1] = [3,7], batch layout out[p*rows + r]."""
     ops = _ops()
