@@ -1004,19 +1004,39 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_lds_kernel(
     const int d0 = ks * 32 + G * 8 < HD ? ks * 32 + G * 8 : 0;
     qin[ks] = FUSED ? rot8_load(qrow, d0, cs, sn, rot, interleaved) : Rot8In{*(const uint4*)(qrow + d0)};
   }
+  const int own = pos % PAGE;          // the token's own row in its page
+  const int own_t = 2 * (own >> 5) + ((own >> 2) & 1), own_j = 4 * ((own >> 3) & 3) + (own & 3);     // where it sits in the score tiles
+  // The wave that will take the sequence's last page also takes in the token's own key and value from the step's row:
+  // it asks for them here, with the queries, so that they are in when the page is (asked for when the page is reached
+  // they would be one more trip to memory in the middle of the kernel).
+  const bool takes_own = FUSED && new_kv && pg1 == last_pg && (last_pg - pg0) % NWV == wave;
+  Rot8In kin[KS];
+  bf16_t v_own[DT];
+  if (takes_own) {
+    const bf16_t* row = q + (size_t)seq * ldq;
+    const bf16_t* krow_new = row + k_col + (size_t)kvh * HD;
+    const bf16_t* vrow_new = row + v_col + (size_t)kvh * HD;
+    if (j == own_j) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        if (ks * 32 + G * 8 < HD) kin[ks] = rot8_load(krow_new, ks * 32 + G * 8, cs, sn, rot, interleaved);
+    }
+    if (G == ((own >> 3) & 3)) {
+#pragma unroll
+      for (int d = 0; d < DT; ++d) v_own[d] = vrow_new[d * 16 + j];
+    }
+  }
   int pg = pg0 + wave;
   int page_cur = pg <= pg1 ? __builtin_amdgcn_readfirstlane(my_pages[pg]) : -1;
   int page_next = pg + NWV <= pg1 ? my_pages[pg + NWV] : -1;
   if (page_cur >= 0) issue(page_cur);
 
-  uint4 qf[KS];
+  uint4 qf[KS], k_own[KS];
   bool have_q = false;
   f32x4_t o[DT];
 #pragma unroll
   for (int d = 0; d < DT; ++d) o[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m = -INFINITY, l = 0.f;
-  const int own = pos % PAGE;          // the token's own row in its page
-  const int own_t = 2 * (own >> 5) + ((own >> 2) & 1), own_j = 4 * ((own >> 3) & 3) + (own & 3);     // where it sits in the score tiles
 
   for (; pg <= pg1; pg += NWV) {
     const int page = page_cur;
@@ -1057,12 +1077,14 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_lds_kernel(
       for (int ks = 0; ks < KS; ++ks)
         qf[ks] = !(head_ok && ks * 32 + G * 8 < HD) ? make_uint4(0, 0, 0, 0)
                  : rot8_apply(qin[ks], ks * 32 + G * 8, FUSED && cs != nullptr, rot, interleaved);
+      if (takes_own && j == own_j) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+          if (ks * 32 + G * 8 < HD) k_own[ks] = rot8_apply(kin[ks], ks * 32 + G * 8, cs != nullptr, rot, interleaved);
+      }
     }
     if (FUSED && new_kv && pg == last_pg) {
       // the token's own key and value come from the step's row, not from the cache; head block 0 stores them
-      const bf16_t* row = q + (size_t)seq * ldq;
-      const bf16_t* krow_new = row + k_col + (size_t)kvh * HD;
-      const bf16_t* vrow_new = row + v_col + (size_t)kvh * HD;
       if (j == own_j) {
 #pragma unroll
         for (int t = 0; t < 4; ++t)
@@ -1070,7 +1092,7 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_lds_kernel(
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks)
               if (ks * 32 + G * 8 < HD) {
-                kf[t][ks] = rotated8(krow_new, ks * 32 + G * 8, cs, sn, rot, interleaved);
+                kf[t][ks] = k_own[ks];
                 if (hb == 0) *(uint4*)(kpage + (size_t)own * HD + ks * 32 + G * 8) = kf[t][ks];
               }
           }
@@ -1081,7 +1103,7 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_lds_kernel(
           if (u == (own >> 5)) {
 #pragma unroll
             for (int d = 0; d < DT; ++d) {
-              const bf16_t val = vrow_new[d * 16 + j];
+              const bf16_t val = v_own[d];
               uint32_t w4[4] = {vf[u][d].x, vf[u][d].y, vf[u][d].z, vf[u][d].w};
               const int e = own & 7;
 #pragma unroll

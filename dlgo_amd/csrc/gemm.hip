@@ -498,12 +498,13 @@ __global__ __launch_bounds__(256) void split_sum_norm_kernel(const float* __rest
   float ss = 0.f;
   // the first eight runs of every piece of the row and the old values are all asked for before anything is added:
   // one trip to memory for the whole row (the last run stands in for those beyond it, and is not added twice)
-  float4 old[NCH], x[NCH][8];
+  float4 old[NCH], x[NCH][8], nw[NCH];        // (the norm's weights too: asked for after the sum they would be a second trip)
 #pragma unroll
   for (int c = 0; c < NCH; ++c) {
     const int n = (c * 256 + threadIdx.x) * 4;
     const int nn = n < N ? n : 0;
     old[c] = *(const float4*)(y + nn);
+    nw[c] = *(const float4*)(norm_w + nn);
 #pragma unroll
     for (int i = 0; i < 8; ++i) x[c][i] = *(const float4*)(p + nn + (size_t)(i < runs ? i : runs - 1) * run_stride);
   }
@@ -545,7 +546,7 @@ __global__ __launch_bounds__(256) void split_sum_norm_kernel(const float* __rest
   for (int c = 0; c < NCH; ++c) {
     const int n = (c * 256 + threadIdx.x) * 4;
     if (n < N) {
-      const float4 w = *(const float4*)(norm_w + n);
+      const float4 w = nw[c];
       T* o = normed + (size_t)t * ldn + n;
       Elem<T>::store(o, row[c].x * scale * w.x);
       Elem<T>::store(o + 1, row[c].y * scale * w.y);

@@ -331,13 +331,38 @@ struct NormShares {
   }
 };
 
+// Mode 1 reads, besides W and X, the residual values it adds to and the norm's weights.  They are asked for at the
+// kernel's start (by wave 0, which runs the epilogue), so that they arrive while W streams in: asked for after the
+// product they would cost the kernel one more trip to memory, a quarter of what a product of a few megabytes takes.
+struct ResidualAhead {
+  float y[4], w[4];
+};
+template <int MODE>
+__device__ __forceinline__ ResidualAhead residual_ahead(const void* __restrict__ Y, int ldy, int N, int n_first, bool tok, int t_row,
+                                                        const NormParts& np) {
+  ResidualAhead a;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) a.y[q] = a.w[q] = 0.f;
+  if (MODE != 1 || (threadIdx.x >> 6) != 0 || !tok) return a;
+  const int n = n_first + 4 * ((threadIdx.x & 63) >> 4);
+  const float* y = (const float*)Y + (size_t)t_row * ldy + n;
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+    if (n + q < N) {
+      a.y[q] = y[q];
+      a.w[q] = np.norm_w[n + q];
+    }
+  return a;
+}
+
 // The end of a streamed product for one group of 16 rows: the waves' partial sums go through LDS (the rows' place, once
 // every wave is done with them, which the caller's barrier has made sure of); wave 0 adds them in wave order and runs the
 // epilogue.  lane: token t_row (the block's token lane % 16), rows 4 G + v of the group.  part_index: where this
 // group's share goes (mode 1).
 template <typename T, int NW, int EPI, int MODE>
 __device__ __forceinline__ void stream_finish(float* red, const f32x4_t& acc, void* __restrict__ Y, int ldy, int N, int n_first,
-                                              bool tok, float sc, const NormParts& np, int part_index, int t_row) {
+                                              bool tok, float sc, const NormParts& np, int part_index, int t_row,
+                                              const ResidualAhead& ahead) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = lane & 15, G = lane >> 4;
 #pragma unroll
@@ -363,10 +388,10 @@ __device__ __forceinline__ void stream_finish(float* red, const f32x4_t& acc, vo
 #pragma unroll
       for (int q = 0; q < 4; ++q)
         if (n + q < N) {
-          const float x = y[q] + v[q];
+          const float x = ahead.y[q] + v[q];
           y[q] = x;
           p = fmaf(x, x, p);
-          Elem<T>::store(u + q, x * np.norm_w[n + q]);
+          Elem<T>::store(u + q, x * ahead.w[q]);
         }
     }
     p += __shfl_xor(p, 16, WAVE);
@@ -402,6 +427,9 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __rest
   __shared__ float sumsq[16];
   NormShares<NW, MODE> shares;                 // mode 2: asked for here, in front of W's loads
   shares.ask(np, Tn);
+  ResidualAhead ahead[R];                      // mode 1: likewise
+#pragma unroll
+  for (int r = 0; r < R; ++r) ahead[r] = residual_ahead<MODE>(Y, ldy, N, n0 + r * 16, tok, j, np);
   // load c brings row c's kilobyte of a group; the lane fetches the piece that belongs at its slot.  Rows beyond N repeat the last.
   const char* base = (const char*)uniform_ptr(W + (size_t)n0 * ldw + wave * CH);
   const uint32_t last_row = (uint32_t)(N - 1 - n0);
@@ -444,7 +472,7 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __rest
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     if (r) __syncthreads();                    // wave 0 has read the group before
-    stream_finish<T, NW, EPI, MODE>(red, acc[r], Y, ldy, N, n0 + r * 16, tok, sc, np, blockIdx.x * R + r, j);
+    stream_finish<T, NW, EPI, MODE>(red, acc[r], Y, ldy, N, n0 + r * 16, tok, sc, np, blockIdx.x * R + r, j, ahead[r]);
   }
 }
 
@@ -496,6 +524,7 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_long_kernel(const T* _
   __shared__ float sumsq[16];
   NormShares<NW, MODE> shares;
   shares.ask(np, Tn);
+  const ResidualAhead ahead = residual_ahead<MODE>(Y, ldy, N, n0, tok, j, np);
   uint4 b0[STEPS], b1[STEPS];
   ask(0, b0);
   for (int turn = 0; turn < turns; turn += 2) {
@@ -505,7 +534,7 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_long_kernel(const T* _
   shares.leave(sumsq);
   __syncthreads();
   const float sc = MODE == 2 ? 1.0f / sqrtf(sumsq[j] / (float)np.width + np.eps) : 1.f;
-  stream_finish<T, NW, EPI, MODE>((float*)lds_raw, acc, Y, ldy, N, n0, tok, sc, np, blockIdx.x, j);
+  stream_finish<T, NW, EPI, MODE>((float*)lds_raw, acc, Y, ldy, N, n0, tok, sc, np, blockIdx.x, j, ahead);
 }
 
 // The same with the RMSNorm of the float32 residual rows riding in the product (see skinny_kernel).  A wave needs the
