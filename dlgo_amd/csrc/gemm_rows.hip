@@ -703,7 +703,10 @@ static bool stream_is_long(int nw, int turns) { return turns > 1 || nw == 5 || n
 // A block takes up to four groups of 16 rows in turn, which share its operands of X (and the work on the norm): as many
 // as leave blocks for at least five eighths of the compute units (a function of N alone).  Measured with 1 to 16 tokens
 // on matrices of 2,048 to 128,256 rows of 4 to 8 KB: fewer blocks than that cost more than the shared work saves; with
-// more, four groups are 5 to 25% faster than one on the wide matrices and two on those of 5,000 to 6,000 rows.
+// more, four groups are 5 to 25% faster than one on the wide matrices and two on those of 5,000 to 6,000 rows.  (Where
+// two blocks share a compute unit's LDS, rows of 4 KB, one group a block is 5% faster for the plain product of 16,384
+// rows with up to 8 rows of X, 15.8 against 16.5 us; the product that applies a norm left to it adds up the norm's
+// shares once per block and loses that again, 1.020 against 1.011 ms a step, so the rule has no such exception.)
 static int stream_groups(int N, bool is_long) {
   const int blocks1 = (N + 15) / 16, fill = compute_units() * 5 / 8;
   return is_long ? 1 : (blocks1 >= 4 * fill ? 4 : (blocks1 >= 2 * fill ? 2 : 1));
@@ -712,9 +715,9 @@ static int stream_groups(int N, bool is_long) {
 template <typename T, int EPI, bool NORM, int MODE = 0>
 static const char* launch_skinny_stream(const void* W, const void* X, const float* norm_w, float eps, void* Y, int N, int Tn, int K,
                                         int ldw, int ldx, int ldy, int nw, hipStream_t stream, NormParts np = NormParts{},
-                                        int turns = 1) {
+                                        int turns = 1, int force_groups = 0) {
   const bool is_long = stream_is_long(nw, turns);
-  const int groups = stream_groups(N, is_long);
+  const int groups = force_groups && !is_long ? force_groups : stream_groups(N, is_long);     // forced: tuning and tests
   dim3 g((N + 16 * groups - 1) / (16 * groups));
   // a wave's LDS: 16 KB of W and, with the norm, a kilobyte of column operands per token
   const int lds = nw * (16384 + (NORM ? Tn * 1024 : 0));
@@ -808,8 +811,9 @@ static const char* launch_skinny(const void* W, const void* X, const float* norm
   int turns = 1;
   int sw = stream_waves<T>(Tn, K, ldw, NORM ? nullptr : &turns);
   if (NORM && sw * (16384 + Tn * 1024) > 160 * 1024) sw = 0;      // the tokens' operands have to fit in LDS beside W
-  if (sw && (force_nw == 32 || force_nw == 0)) {
-    return launch_skinny_stream<T, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, sw, stream, NormParts{}, turns);
+  if (sw && (force_nw == 32 || force_nw == 0 || force_nw == 33 || force_nw == 34 || force_nw == 36)) {
+    return launch_skinny_stream<T, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, sw, stream, NormParts{}, turns,
+                                              force_nw > 32 ? force_nw - 32 : 0);
   }
   if (force_nw && force_nw < 32) nw = force_nw;
   // many rows: each block takes 2 or 4 groups of 16, which divides the traffic of X (a function of N alone)
@@ -840,13 +844,13 @@ static const char* dispatch_rows(const void* W, const void* X, void* Y, int N, i
                                  hipStream_t stream) {
   // kind: 0 = the MFMA kernels, 1 = the vector kernel (at most 8 rows), 6..9 = the MFMA kernel that reads W into registers,
   // with 1, 2, 4, 8 waves per block, 10 = the MFMA kernel that sends W through LDS (where it applies, else as 0),
-  // 11 = never that one
+  // 11 = never that one, 15..17 = as 10 with 1, 2, 4 groups of weight rows a block
   if (kind == 1) {
     launch_gemv<T, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
     return nullptr;
   }
   return launch_skinny<T, EPI, false>(W, X, nullptr, 0.f, Y, N, Tn, K, ldw, ldx, ldy, stream,
-                                      kind == 0 ? 0 : (kind == 10 ? 32 : (kind == 11 ? 64 : 1 << (kind - 6))));
+                                      kind == 0 ? 0 : (kind == 10 ? 32 : (kind == 11 ? 64 : (kind >= 15 ? 32 + (1 << (kind - 15)) : 1 << (kind - 6)))));
 }
 
 template <typename T>
@@ -875,7 +879,7 @@ extern "C" const char* dlgo_gemm_rows(const void* W, const void* X, void* Y, int
   DLGO_REQUIRE(((uintptr_t)Y & 3) == 0 || (dtype == DLGO_DTYPE_BF16 && ((uintptr_t)Y & 1) == 0), "gemm: Y must be aligned to its elements");
   DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm: SwiGLU epilogue needs an even N and ldy >= N/2");
   DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm: ldy %d shorter than N %d", ldy, N);
-  DLGO_REQUIRE(kind == 0 || kind == 1 || (kind >= 6 && kind <= 11), "gemm_rows: unknown kernel choice %d", kind);
+  DLGO_REQUIRE(kind == 0 || kind == 1 || (kind >= 6 && kind <= 11) || (kind >= 15 && kind <= 17), "gemm_rows: unknown kernel choice %d", kind);
   DLGO_REQUIRE(kind != 1 || Tn <= 8, "gemm: the vector kernel takes at most 8 rows, got %d", Tn);
   if (Tn == 0) return nullptr;
   const char* err = rows_by_epilogue<elem_t>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, kind, stream);

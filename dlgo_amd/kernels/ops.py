@@ -224,7 +224,7 @@ def _streams_rows(weight: torch.Tensor, t: int, kind: int, has_scratch: bool, sp
     pieces = row_bytes // 128 if row_bytes % 128 == 0 else 0
     can_split = has_scratch and splits != 1 and pieces >= 32
     if kind != GEMM_AUTO or splits > 1:
-        return kind in (GEMM_STREAM, 5, 6, 7, 8, 9, 10, 11)
+        return kind in (GEMM_STREAM, 5, 6, 7, 8, 9, 10, 11, 15, 16, 17)
     cus = compute_units(weight.device)
     blocks16, tiles64 = (n + 15) // 16, (n + 63) // 64
     very_wide = blocks16 >= 16 * cus

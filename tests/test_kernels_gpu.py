@@ -126,11 +126,11 @@ GEMM_SHAPES = [(200, 37, 96), (130, 5, 40), (64, 1, 64), (388, 130, 352), (34, 8
 
 
 @pytest.mark.parametrize("dtype,_,rel", DT)
-@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 14])
+@pytest.mark.parametrize("kind", [0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 14, 15, 16, 17])
 @pytest.mark.parametrize("n,t,k", GEMM_SHAPES)
 def test_gemm_store_and_accumulate(dtype, _, rel, kind, n, t, k):
     ops = _ops()
-    if (kind == 1 and t > 8) or (5 <= kind <= 11 and t > 64):
+    if (kind == 1 and t > 8) or ((5 <= kind <= 11 or kind >= 15) and t > 64):
         pytest.skip("the streaming kernels take a few rows only")
     if dtype == torch.bfloat16 and k % 8:
         pytest.skip("bfloat16 rows come in 16-byte pieces")
