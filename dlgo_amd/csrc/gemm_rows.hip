@@ -362,7 +362,7 @@ __device__ __forceinline__ ResidualAhead residual_ahead(const void* __restrict__
 template <typename T, int NW, int EPI, int MODE>
 __device__ __forceinline__ void stream_finish(float* red, const f32x4_t& acc, void* __restrict__ Y, int ldy, int N, int n_first,
                                               bool tok, float sc, const NormParts& np, int part_index, int t_row,
-                                              const ResidualAhead& ahead) {
+                                              const ResidualAhead& ahead, int rows_here = 16) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = lane & 15, G = lane >> 4;
 #pragma unroll
@@ -374,6 +374,7 @@ __device__ __forceinline__ void stream_finish(float* red, const f32x4_t& acc, vo
 #pragma unroll
     for (int q = 0; q < 4; ++q) v[q] += red[(w * 16 + 4 * G + q) * 17 + j];
   const int n = n_first + 4 * G;
+  if (4 * G >= rows_here) tok = false;         // a block of 8 rows: the other half of the tile is nobody's
   if (MODE == 2) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) v[q] *= sc;
@@ -405,7 +406,9 @@ __device__ __forceinline__ void stream_finish(float* red, const f32x4_t& acc, vo
 template <typename T, int NW, int R, int EPI, int MODE>
 __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __restrict__ W, const void* __restrict__ Xv,
                                                                   void* __restrict__ Y, int N, int Tn, int K, int ldw, int ldx,
-                                                                  int ldy, NormParts np) {
+                                                                  int ldy, NormParts np, int rows) {
+  // rows: 16, or (R == 1 only) 8: a block takes half a tile's rows, so that a matrix of few rows still gives every
+  // compute unit a block; the tile's other half is computed on whatever LDS holds and dropped
   constexpr int EPC = 16 / sizeof(T);          // elements of a 16-byte operand
   constexpr int CH = 1024 / sizeof(T);         // elements of a row's kilobyte
   constexpr int STEPS = 16;                    // MFMA steps of a kilobyte: four 16-byte pieces each
@@ -415,7 +418,7 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __rest
   const uint32_t wbase = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)wbuf);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = lane & 15, G = lane >> 4;
-  const int n0 = blockIdx.x * 16 * R;          // the block's R groups of 16 rows take the wave's operands of X in turn
+  const int n0 = R == 1 ? blockIdx.x * rows : blockIdx.x * 16 * R;    // the block's R groups of 16 rows take the wave's operands of X in turn
   const bool tok = j < Tn;
   // the lane's operands of X, once for all the groups: token j, the wave's kilobyte of k
   uint4 b[STEPS];
@@ -436,6 +439,7 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __rest
   auto issue = [&](int r) {
 #pragma unroll
     for (int c = 0; c < 16; ++c) {
+      if (R == 1 && c >= rows) break;
       const uint32_t row = (uint32_t)(16 * r + c) < last_row ? (uint32_t)(16 * r + c) : last_row;
       row_to_lds(base, row * (uint32_t)ldw * (uint32_t)sizeof(T) + (uint32_t)((lane ^ c) << 4), wbase + c * 1024);
     }
@@ -472,7 +476,7 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __rest
 #pragma unroll
   for (int r = 0; r < R; ++r) {
     if (r) __syncthreads();                    // wave 0 has read the group before
-    stream_finish<T, NW, EPI, MODE>(red, acc[r], Y, ldy, N, n0 + r * 16, tok, sc, np, blockIdx.x * R + r, j, ahead[r]);
+    stream_finish<T, NW, EPI, MODE>(red, acc[r], Y, ldy, N, n0 + r * 16, tok, sc, np, blockIdx.x * R + r, j, ahead[r], R == 1 ? rows : 16);
   }
 }
 
@@ -707,6 +711,17 @@ static bool stream_is_long(int nw, int turns) { return turns > 1 || nw == 5 || n
 // two blocks share a compute unit's LDS, rows of 4 KB, one group a block is 5% faster for the plain product of 16,384
 // rows with up to 8 rows of X, 15.8 against 16.5 us; the product that applies a norm left to it adds up the norm's
 // shares once per block and loses that again, 1.020 against 1.011 ms a step, so the rule has no such exception.)
+// Rows of W a block of one group takes: 16, a whole MFMA tile, or 8 where tiles of 16 would give at most half of the
+// compute units a block (an output projection of 2,048 rows: 128 blocks on 256 units; 4.3 to 4.9 against 4.5 to 5.3 us
+// with 1 to 16 rows of X, a matrix of 1,024 rows 3.8 against 4.3 us) and, for the product that leaves a norm's shares,
+// the shares of twice as many blocks still fit.  With more blocks than that, halves lose: 3,072 rows of 4 KB take 5.5
+// to 7.3 us in blocks of 8 and 5.0 to 5.6 in blocks of 16, rows of 6 KB 8.2 against 6.2 us.
+static int stream_rows(int N, bool is_long, int groups, int mode) {
+  if (is_long || groups != 1 || (N + 15) / 16 > compute_units() / 2) return 16;
+  if (mode == 1 && (N + 7) / 8 > NORM_PARTS_MAX) return 16;
+  return 8;
+}
+
 static int stream_groups(int N, bool is_long) {
   const int blocks1 = (N + 15) / 16, fill = compute_units() * 5 / 8;
   return is_long ? 1 : (blocks1 >= 4 * fill ? 4 : (blocks1 >= 2 * fill ? 2 : 1));
@@ -717,8 +732,9 @@ static const char* launch_skinny_stream(const void* W, const void* X, const floa
                                         int ldw, int ldx, int ldy, int nw, hipStream_t stream, NormParts np = NormParts{},
                                         int turns = 1, int force_groups = 0) {
   const bool is_long = stream_is_long(nw, turns);
-  const int groups = force_groups && !is_long ? force_groups : stream_groups(N, is_long);     // forced: tuning and tests
-  dim3 g((N + 16 * groups - 1) / (16 * groups));
+  const int groups = force_groups && !is_long ? (force_groups > 0 ? force_groups : 1) : stream_groups(N, is_long);     // forced: tuning and tests
+  const int rows = NORM || is_long ? 16 : (force_groups == -8 ? 8 : (force_groups == -16 ? 16 : stream_rows(N, is_long, groups, MODE)));
+  dim3 g(groups == 1 ? (N + rows - 1) / rows : (N + 16 * groups - 1) / (16 * groups));
   // a wave's LDS: 16 KB of W and, with the norm, a kilobyte of column operands per token
   const int lds = nw * (16384 + (NORM ? Tn * 1024 : 0));
 #define STREAM_RAISE(LIMIT_, ...)                                                                                               \
@@ -758,7 +774,7 @@ static const char* launch_skinny_stream(const void* W, const void* X, const floa
       auto k4 = skinny_stream_kernel<T, NW_, 4, EPI, MODE>;                                                  \
       STREAM_RAISE(NW_ * 16384, (const void*)k1, (const void*)k2, (const void*)k4);                                             \
       auto kernel = groups == 4 ? k4 : (groups == 2 ? k2 : k1);                                                                 \
-      hipLaunchKernelGGL(kernel, g, dim3(NW_* WAVE), lds, stream, (const T*)W, X, Y, N, Tn, K, ldw, ldx, ldy, np);              \
+      hipLaunchKernelGGL(kernel, g, dim3(NW_* WAVE), lds, stream, (const T*)W, X, Y, N, Tn, K, ldw, ldx, ldy, np, rows);        \
     }                                                                                                                           \
   } while (0)
   if (is_long) {
@@ -811,9 +827,10 @@ static const char* launch_skinny(const void* W, const void* X, const float* norm
   int turns = 1;
   int sw = stream_waves<T>(Tn, K, ldw, NORM ? nullptr : &turns);
   if (NORM && sw * (16384 + Tn * 1024) > 160 * 1024) sw = 0;      // the tokens' operands have to fit in LDS beside W
-  if (sw && (force_nw == 32 || force_nw == 0 || force_nw == 33 || force_nw == 34 || force_nw == 36)) {
-    return launch_skinny_stream<T, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, sw, stream, NormParts{}, turns,
-                                              force_nw > 32 ? force_nw - 32 : 0);
+  if (sw && (force_nw == 32 || force_nw == 0 || force_nw == 33 || force_nw == 34 || force_nw == 36 || force_nw == 40 || force_nw == 41)) {
+    // 33, 34, 36: 1, 2, 4 groups of rows a block; 40, 41: one group, of 8 or 16 rows
+    const int force = force_nw == 40 ? -8 : (force_nw == 41 ? -16 : (force_nw > 32 ? force_nw - 32 : 0));
+    return launch_skinny_stream<T, EPI, NORM>(W, X, norm_w, eps, Y, N, Tn, K, ldw, ldx, ldy, sw, stream, NormParts{}, turns, force);
   }
   if (force_nw && force_nw < 32) nw = force_nw;
   // many rows: each block takes 2 or 4 groups of 16, which divides the traffic of X (a function of N alone)
@@ -844,13 +861,13 @@ static const char* dispatch_rows(const void* W, const void* X, void* Y, int N, i
                                  hipStream_t stream) {
   // kind: 0 = the MFMA kernels, 1 = the vector kernel (at most 8 rows), 6..9 = the MFMA kernel that reads W into registers,
   // with 1, 2, 4, 8 waves per block, 10 = the MFMA kernel that sends W through LDS (where it applies, else as 0),
-  // 11 = never that one, 15..17 = as 10 with 1, 2, 4 groups of weight rows a block
+  // 11 = never that one, 15..17 = as 10 with 1, 2, 4 groups of weight rows a block, 18 and 19 = as 10 with one group of 8 or 16 rows
   if (kind == 1) {
     launch_gemv<T, EPI>(W, X, Y, N, Tn, K, ldw, ldx, ldy, stream);
     return nullptr;
   }
   return launch_skinny<T, EPI, false>(W, X, nullptr, 0.f, Y, N, Tn, K, ldw, ldx, ldy, stream,
-                                      kind == 0 ? 0 : (kind == 10 ? 32 : (kind == 11 ? 64 : (kind >= 15 ? 32 + (1 << (kind - 15)) : 1 << (kind - 6)))));
+                                      kind == 0 ? 0 : (kind == 10 ? 32 : (kind == 11 ? 64 : (kind >= 18 ? 22 + kind : (kind >= 15 ? 32 + (1 << (kind - 15)) : 1 << (kind - 6))))));
 }
 
 template <typename T>
@@ -879,7 +896,7 @@ extern "C" const char* dlgo_gemm_rows(const void* W, const void* X, void* Y, int
   DLGO_REQUIRE(((uintptr_t)Y & 3) == 0 || (dtype == DLGO_DTYPE_BF16 && ((uintptr_t)Y & 1) == 0), "gemm: Y must be aligned to its elements");
   DLGO_REQUIRE(epilogue != EPI_SWIGLU || (N % 2 == 0 && ldy >= N / 2), "gemm: SwiGLU epilogue needs an even N and ldy >= N/2");
   DLGO_REQUIRE(epilogue == EPI_SWIGLU || ldy >= N, "gemm: ldy %d shorter than N %d", ldy, N);
-  DLGO_REQUIRE(kind == 0 || kind == 1 || (kind >= 6 && kind <= 11) || (kind >= 15 && kind <= 17), "gemm_rows: unknown kernel choice %d", kind);
+  DLGO_REQUIRE(kind == 0 || kind == 1 || (kind >= 6 && kind <= 11) || (kind >= 15 && kind <= 19), "gemm_rows: unknown kernel choice %d", kind);
   DLGO_REQUIRE(kind != 1 || Tn <= 8, "gemm: the vector kernel takes at most 8 rows, got %d", Tn);
   if (Tn == 0) return nullptr;
   const char* err = rows_by_epilogue<elem_t>(W, X, Y, N, Tn, K, ldw, ldx, ldy, epilogue, kind, stream);
@@ -961,8 +978,12 @@ extern "C" const char* dlgo_gemm_rows_leave_parts(const void* W, const void* X, 
   const int epc = dtype == DLGO_DTYPE_F32 ? 4 : 8;
   DLGO_REQUIRE(ldw % epc == 0 && ldx % epc == 0 && ((uintptr_t)W & 15) == 0 && ((uintptr_t)X & 15) == 0,
                "gemm_rows_leave_parts: W and X must be 16-byte aligned with row strides that keep them so");
-  const int np_ = (N + 15) / 16;
-  DLGO_REQUIRE(np_ <= NORM_PARTS_MAX, "gemm_rows_leave_parts: a width of up to %d, got %d", 16 * NORM_PARTS_MAX, N);
+  DLGO_REQUIRE((N + 15) / 16 <= NORM_PARTS_MAX, "gemm_rows_leave_parts: a width of up to %d, got %d", 16 * NORM_PARTS_MAX, N);
+  // a share for every block of one group of rows (16 rows, or 8: stream_rows), or for every group of a block of several
+  const bool is_long = stream_is_long(sw, turns);
+  const int groups = stream_groups(N, is_long);
+  const int rows = stream_rows(N, is_long, groups, 1);
+  const int np_ = groups == 1 ? (N + rows - 1) / rows : (N + 15) / 16;
   DLGO_REQUIRE(residual && norm_w && unscaled && parts && parts_elems >= (long long)Tn * np_, "gemm_rows_leave_parts: missing operand or scratch too small");
   *n_parts = np_;
   if (Tn == 0) return nullptr;

@@ -224,7 +224,7 @@ def _streams_rows(weight: torch.Tensor, t: int, kind: int, has_scratch: bool, sp
     pieces = row_bytes // 128 if row_bytes % 128 == 0 else 0
     can_split = has_scratch and splits != 1 and pieces >= 32
     if kind != GEMM_AUTO or splits > 1:
-        return kind in (GEMM_STREAM, 5, 6, 7, 8, 9, 10, 11, 15, 16, 17)
+        return kind in (GEMM_STREAM, 5, 6, 7, 8, 9, 10, 11, 15, 16, 17, 18, 19)
     cus = compute_units(weight.device)
     blocks16, tiles64 = (n + 15) // 16, (n + 63) // 64
     very_wide = blocks16 >= 16 * cus
@@ -431,7 +431,7 @@ def can_take_unscaled(weight: torch.Tensor, rows: int) -> bool:
 def gemm_accum_leave_norm(weight: torch.Tensor, x: torch.Tensor, residual: torch.Tensor, norm_weight: torch.Tensor, eps: float,
                           unscaled: torch.Tensor, parts: torch.Tensor) -> UnscaledNorm:
     """residual += x @ weight.T, and of rmsnorm(residual) * norm_weight of the new rows what UnscaledNorm describes
-    (unscaled: [T, N] in the run dtype; parts: float32 scratch of at least T * ceil(N / 16) elements).  For weights
+    (unscaled: [T, N] in the run dtype; parts: float32 scratch of at least T * ceil(N / 8) elements).  For weights
     and rows that can_leave_unscaled accepts: few rows go to the streamed product, many to tiles."""
     _need(weight, "gemm weight", dims=2)
     _need(x, "gemm input", weight.dtype, 2)

@@ -198,7 +198,7 @@ class Attention(Mixer):
             unscaled_ok = len(then) > 2 and then[2] is not None and then[2].takes_unscaled(ctx)
 
             def leave():
-                shares = ctx.scratch("attention.norm_shares", t * ((self.width + 15) // 16), torch.float32)
+                shares = ctx.scratch("attention.norm_shares", t * ((self.width + 7) // 8), torch.float32)
                 return ops.gemm_accum_leave_norm(self.w_o, out, residual, then[0].weight, then[0].eps, then[1], shares)
             if unscaled_ok and ops.streams_few_rows(self.w_o, t, ops.ROLE_LEAVES_NORM):
                 return leave()

@@ -79,7 +79,7 @@ class GatedFeedForward(FeedForward):
             t = residual.shape[0]
             if t > 16 and len(then) > 2 and then[2] is not None and then[2].takes_unscaled(ctx) \
                     and ops.can_leave_unscaled(self.w_down, t):
-                shares = ctx.scratch("feed_forward.norm_shares", t * ((self.width + 15) // 16), torch.float32)
+                shares = ctx.scratch("feed_forward.norm_shares", t * ((self.width + 7) // 8), torch.float32)
                 return ops.gemm_accum_leave_norm(self.w_down, hid, residual, then[0].weight, then[0].eps, then[1], shares)
         ops.gemm(self.w_down, hid, residual, ops.EPI_ACCUM_F32, scratch=split)
         return False
