@@ -88,6 +88,12 @@ class KVGroup:
         self.table_host = np.full((max_slots, max_pages_per_seq), -1, dtype=np.int32)
         self.table = torch.full((max_slots, max_pages_per_seq), -1, dtype=torch.int32, device=device)
         self.dirty: set = set()
+        self.version = 0             # counts the changes of table_host: who keeps a copy of some rows knows when it is stale
+
+    def touch(self, slot: int) -> None:
+        """Row `slot` of the page table changed on the host."""
+        self.dirty.add(slot)
+        self.version += 1
 
     def unit_view(self, index_in_group: int) -> torch.Tensor:
         """Storage from the first element of this unit's part of page 0."""
@@ -180,7 +186,7 @@ class Cache:
             g.pool.give(list(held.values()))
             if held:
                 g.table_host[slot, list(held.keys())] = -1
-                g.dirty.add(slot)
+                g.touch(slot)
             held.clear()
         self._live[slot] = False
         self.lengths[slot] = 0
@@ -220,7 +226,7 @@ class Cache:
             for i, p in zip(idx, pages):
                 self._held[dst][gi][i] = p
                 g.table_host[dst, i] = p
-            g.dirty.add(dst)
+            g.touch(dst)
             by_page = g.storage.view(g.pool.n_pages, g.page_stride)
             if self.device.type != "cuda":
                 by_page[torch.as_tensor(pages, dtype=torch.int64)] = by_page[torch.as_tensor(src_pages, dtype=torch.int64)]
@@ -300,7 +306,7 @@ class Cache:
                 for i, p in zip(idx, pages):
                     self._held[slot][gi][i] = p
                     g.table_host[slot, i] = p
-                g.dirty.add(slot)
+                g.touch(slot)
 
     def advance(self, slot: int, n_tokens: int) -> None:
         """The slot now holds n_tokens more; pages no later token can see go back to their pool."""
@@ -315,7 +321,7 @@ class Cache:
             if gone:
                 g.pool.give([held.pop(i) for i in gone])
                 g.table_host[slot, gone] = -1
-                g.dirty.add(slot)
+                g.touch(slot)
 
     @property
     def has_windows(self) -> bool:
@@ -375,7 +381,7 @@ class Cache:
     def kv_view(self, unit: int) -> "KVView":
         gi, ui = self.unit_group[unit]
         g = self.groups[gi]
-        return KVView(g.unit_view(ui), g.page_stride, g.v_off, g.table, g.spec.kv_heads, g.spec.head_dim, g.spec.window)
+        return KVView(g.unit_view(ui), g.page_stride, g.v_off, g.table, g.spec.kv_heads, g.spec.head_dim, g.spec.window, gi)
 
     def state_of(self, unit: int) -> torch.Tensor:
         return self.state[unit]
@@ -430,3 +436,4 @@ class KVView:
     kv_heads: int
     head_dim: int
     window: Optional[int]
+    group: int = 0             # index of the storage group (its page table is shared by the group's units)

@@ -943,7 +943,11 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_lds_kernel(
     const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, const int32_t* __restrict__ page_table,
     int max_pages, bf16_t* __restrict__ cache, long long page_stride, long long v_off, int n_heads, int group,
     int head_blocks, SplitPlan sp, int window, float scale_log2e, const float* __restrict__ cos_t,
-    const float* __restrict__ sin_t, int rot, int interleaved, int new_kv, int k_col, int v_col) {
+    const float* __restrict__ sin_t, int rot, int interleaved, int new_kv, int k_col, int v_col,
+    const int32_t* __restrict__ seq_pages) {
+  // seq_pages (may be null): the page numbers of the step's sequences by their place in the step, [n_seq, max_pages]:
+  // row seq is row slots[seq] of page_table.  With it nothing here waits for the slot, and the number of a wave's first
+  // page is asked for together with the position instead of after it (below).
   constexpr int HD = HEAD_DIM;
   constexpr int KS = (HD + 31) / 32;   // k steps of K Q^T (16x16x32)
   constexpr int DT = HD / 16;          // 16-row tiles of the output's head dimension
@@ -956,6 +960,16 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_lds_kernel(
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int split = blockIdx.z, seq = blockIdx.y;         // as attn_decode_kernel
   const int kvh = blockIdx.x / head_blocks, hb = blockIdx.x % head_blocks;
+  // Which page a wave takes first depends on the sequence's length, which is a trip to memory away.  With the pages
+  // listed by sequence their place is known at once, so every lane asks for a candidate now: lane s - 1 for the page the
+  // wave would start at if the block's share were s pages (split * s + wave, without a window), and the one that the
+  // position then calls for is picked from the lanes.  That makes position and page number one trip instead of two.
+  const int first_wave = (int)(threadIdx.x >> 6);
+  int candidate = -1;
+  if (seq_pages != nullptr && window == 0) {
+    const long long at = (long long)split * ((int)(threadIdx.x & 63) + 1) + first_wave;
+    if (at < max_pages) candidate = seq_pages[(size_t)seq * max_pages + at];
+  }
   const int pos = positions[seq];
   const int lo = window > 0 && pos - window + 1 > 0 ? pos - window + 1 : 0;
   const int first_pg = lo / PAGE, last_pg = pos / PAGE;
@@ -964,13 +978,12 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_lds_kernel(
   const int pg0 = first_pg + split * span;
   const int pg1 = pg0 + span - 1 < last_pg ? pg0 + span - 1 : last_pg;
   if (pg0 > pg1) return;               // the whole block: fewer pages than splits
-  const int slot = slots[seq];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, j = lane & 15, G = lane >> 4;
   const int hig = hb * 16 + j;                    // head within the group
   const int heads_here = group - hb * 16 < 16 ? group - hb * 16 : 16;
   const bool head_ok = j < heads_here;
   const int head = kvh * group + hig;
-  const int32_t* my_pages = page_table + (size_t)slot * max_pages;
+  const int32_t* my_pages = seq_pages != nullptr ? seq_pages + (size_t)seq * max_pages : page_table + (size_t)slots[seq] * max_pages;
 
   typedef __attribute__((address_space(3))) char lds_char;
   lds_char* wbuf = (lds_char*)lds + (size_t)wave * (KBYTES + VBYTES);      // this wave's page: keys, then values
@@ -1027,7 +1040,11 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_lds_kernel(
     }
   }
   int pg = pg0 + wave;
-  int page_cur = pg <= pg1 ? __builtin_amdgcn_readfirstlane(my_pages[pg]) : -1;
+  int page_cur;
+  if (seq_pages != nullptr && window == 0 && span <= WAVE)        // the candidate of lane span - 1 is page split * span + wave
+    page_cur = pg <= pg1 ? __builtin_amdgcn_readlane(candidate, span - 1) : -1;
+  else
+    page_cur = pg <= pg1 ? __builtin_amdgcn_readfirstlane(my_pages[pg]) : -1;
   int page_next = pg + NWV <= pg1 ? my_pages[pg + NWV] : -1;
   if (page_cur >= 0) issue(page_cur);
 
@@ -1566,7 +1583,8 @@ extern "C" const char* dlgo_attention_prefill_f32(const void* q, int ldq, void* 
 // bfloat16, one row per sequence.  With cos_t/sin_t ([table_rows, rot/2]) the rows q are unrotated and are rotated
 // here; with new_kv they are [q | k | v] rows whose key (rotated) and value enter the product and the cache here.
 // max_pages_used bounds the pages of any sequence of the step (a recorded
-// launch passes the context's bound).  part: float32 scratch, used when the pages are split over several
+// launch passes the context's bound).  seq_pages (may be null): [n_seq, max_pages], row i = row slots[i] of page_table;
+// the kernel that takes pages through LDS then reads the pages' numbers by sequence (see there).  part: float32 scratch, used when the pages are split over several
 // blocks: n_seq * n_heads * n_splits * (hd + 4) with n_splits = dlgo_attention_decode_splits(...).
 static void decode_plan(int n_pairs, int group, int max_pages_used, bool fused, bool through_lds, int* nwv, SplitPlan* plan) {
   const int heads_here = group < 16 ? group : 16;
@@ -1615,7 +1633,8 @@ extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, 
                                              const int32_t* slots, const int32_t* page_table, int max_pages,
                                              int max_pages_used, void* cache, long long page_stride, long long v_off,
                                              int window, float scale, const float* cos_t, const float* sin_t, int table_rows,
-                                             int rot, int interleaved, int new_kv, int variant, hipStream_t stream) {
+                                             int rot, int interleaved, int new_kv, int variant, const int32_t* seq_pages,
+                                             hipStream_t stream) {
   DLGO_REQUIRE(head_dim == HEAD_DIM, "attention: this library is built for head size %d, got %d", HEAD_DIM, head_dim);
   DLGO_REQUIRE(HEAD_DIM <= 256, "attention: the split kernel takes head sizes up to 256");
   DLGO_REQUIRE(variant >= 0 && variant <= 2, "attention: unknown variant %d of the split kernel", variant);
@@ -1663,7 +1682,7 @@ extern "C" const char* dlgo_attention_decode(const void* q, int ldq, void* out, 
     hipLaunchKernelGGL(kernel, grid, dim3(W_* WAVE), lds_bytes, stream, (const bf16_t*)q, ldq, (bf16_t*)out, ldo, part,        \
                        positions, slots, page_table, max_pages, (bf16_t*)cache, page_stride, v_off, n_heads, group,            \
                        head_blocks, plan, window, scale* LOG2E, cos_t, sin_t, rot, interleaved, new_kv,                    \
-                       n_heads* head_dim, (n_heads + n_kv) * head_dim);                                                        \
+                       n_heads* head_dim, (n_heads + n_kv) * head_dim, seq_pages);                                             \
   } while (0)
     if (fused) {
       if (nwv == 16) DECODE_LDS_GO(16, true);

@@ -87,6 +87,9 @@ class StepContext:
 
         #: pages any sequence of this step may hold (a captured step must allow for the whole context)
         self.max_pages_used: Optional[int] = None
+        #: steps of single tokens: for each storage group of the cache, the sequences' page-table rows in the order of
+        #: the step ([>= n_seq, the table's width], row i = the row of slots[i]), kept current by the engine
+        self.seq_pages: Dict[int, torch.Tensor] = {}
 
     def buffer(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
         return self.engine.workspace.get(name, shape, dtype)

@@ -134,6 +134,10 @@ class Engine:
         self._static_logits: Optional[torch.Tensor] = None
         self._meta_dev = torch.empty(0, dtype=torch.int32, device=self.device)
         self._rows_dev = torch.empty(0, dtype=torch.int32, device=self.device)
+        # steps of single tokens: the sequences' page-table rows by their place in the step, per storage group, at fixed
+        # addresses; (slots, version of the group's table) of what each holds
+        self._seq_pages: Dict[int, torch.Tensor] = {}
+        self._seq_pages_of: Dict[int, tuple] = {}
         self._staging: List[Tuple[torch.Tensor, Optional[torch.cuda.Event]]] = []
         self._staging_next = 0
         self._logits_piece: Optional[torch.Tensor] = None
@@ -253,6 +257,30 @@ class Engine:
             self._staging[i] = (self._staging[i][0], ev)
             ops.copy_rows(x, out, src_rows=self._rows_dev[:len(idx)])
         return out
+
+    def _sync_seq_pages(self, slot_arr: np.ndarray) -> Dict[int, torch.Tensor]:
+        """The page-table rows of these slots, in this order, on the device (one table per storage group of the cache):
+        what the attention of a step of single tokens reads instead of going through the slots.  Rows go up only when
+        the slots or a table changed since the last step (a new page every 64 tokens a sequence)."""
+        b = len(slot_arr)
+        for gi, g in enumerate(self.cache.groups):
+            dev = self._seq_pages.get(gi)
+            if dev is None:
+                dev = torch.full((max(self.graph_max_batch, 1), g.table_host.shape[1]), -1, dtype=torch.int32, device=self.device)
+                self._seq_pages[gi] = dev
+            key = (g.version, slot_arr.tobytes())
+            if self._seq_pages_of.get(gi) == key:
+                continue
+            rows = g.table_host[slot_arr]
+            stage = self._stage(rows.size)
+            stage.numpy()[:rows.size] = rows.reshape(-1)
+            dev[:b].view(-1).copy_(stage[:rows.size], non_blocking=True)
+            ev = torch.cuda.Event()
+            ev.record()
+            i = (self._staging_next - 1) % len(self._staging)
+            self._staging[i] = (self._staging[i][0], ev)
+            self._seq_pages_of[gi] = key
+        return self._seq_pages
 
     # -- the step ----------------------------------------------------------------
     def step(self, entries: Sequence[Entry], sink: Optional[Callable[[int, torch.Tensor], None]] = None) -> Optional[torch.Tensor]:
@@ -473,6 +501,7 @@ class Engine:
         if needs_pages:
             self.cache.reserve([(int(s), int(st) + 1) for s, st in zip(slot_arr, starts)])
             self.cache.sync_tables()
+        seq_pages = self._sync_seq_pages(slot_arr)
         st = self._static_arrays()
         tok_host = np.zeros(b, dtype=np.int32) if on_device else np.asarray(tokens, dtype=np.int32)
         fields = self._decode_fields(tok_host, starts, slot_arr)
@@ -487,6 +516,7 @@ class Engine:
             host = {"q_lens": np.ones(b, dtype=np.int64), "start_pos": starts.astype(np.int64), "slots": slot_arr}
             ctx = StepContext(self, b, b, arrays, host)
             ctx.is_decode = True
+            ctx.seq_pages = seq_pages
             if self.use_graphs:
                 ctx.max_pages_used = self.cache.max_pages_per_seq     # the recorded launch must cover any later length
             x = self.model.hidden(ctx, ctx.token_ids, all_rows_wanted=True)

@@ -581,7 +581,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
               scale: Optional[float] = None, cu_q: Optional[torch.Tensor] = None,
               start_pos_dev: Optional[torch.Tensor] = None, scratch=None,
               max_pages_used: Optional[int] = None, kernel: str = "auto", rotation=None, new_kv: bool = False,
-              split_variant: int = 0) -> torch.Tensor:
+              split_variant: int = 0, seq_pages: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of a step's query rows over the cache, with the kernel chosen by the step's shape and dtype.
 
     q_lens, start_pos: per sequence, on the host (rows of the step, and the length before it).  cu_q and
@@ -594,6 +594,9 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
     token's own key and value from its row and writes them to the cache (what rope_kv() does otherwise).
     split_variant (bfloat16 split kernel): 0 or 2 = a page goes through LDS in whole 1 KB runs, 1 = it is read straight
     into the operands' registers.
+    seq_pages (steps of single tokens): the sequences' rows of page_table in the order of the step, [>= n_seq, the table's
+    width]: row i holds what row slots[i] of page_table holds.  The bfloat16 split kernel then finds a sequence's pages
+    without waiting for its slot, and asks for its first page's number together with the position.
     """
     n_seq = len(q_lens)
     max_q = int(max(q_lens)) if n_seq else 0
@@ -647,6 +650,10 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
             _need(sin, "sin table", torch.float32, 2)
             if cos.shape != sin.shape or cos.shape[1] != rot_width // 2 or not cos.is_contiguous() or not sin.is_contiguous():
                 raise KernelError(f"attention: tables {tuple(cos.shape)} do not fit a rotated width of {rot_width}")
+        if seq_pages is not None:
+            _need(seq_pages, "pages by sequence", torch.int32, 2)
+            if seq_pages.shape[0] < n_seq or seq_pages.shape[1] != max_pages or not seq_pages.is_contiguous():
+                raise KernelError(f"attention: pages by sequence {tuple(seq_pages.shape)} do not fit {n_seq} sequences and a table {max_pages} wide")
         lib.dlgo_attention_decode_splits.restype = ctypes.c_int
         variant = split_variant if q.dtype == torch.bfloat16 else 1
         n_splits = lib.dlgo_attention_decode_splits(n_seq, n_heads, n_kv, max_pages_used, int(rotation is not None or new_kv), variant)
@@ -667,7 +674,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, n_heads: int, n_kv: int, head_
                                          head_dim, _ptr(positions), _ptr(slots), _ptr(page_table), max_pages, max_pages_used,
                                          _ptr(cache), ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(window),
                                          ctypes.c_float(scale), _ptr(cos), _ptr(sin), cos.shape[0] if cos is not None else 0,
-                                         int(rot_width), int(interleaved), int(new_kv), int(variant), _stream()))
+                                         int(rot_width), int(interleaved), int(new_kv), int(variant), _ptr(seq_pages), _stream()))
         return out
     if kernel != "tiled":
         raise KernelError(f"attention: unknown kernel {kernel!r}")

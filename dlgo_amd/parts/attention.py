@@ -216,4 +216,5 @@ class Attention(Mixer):
                       kv.page_table, kv.cache, kv.page_stride, kv.v_off, ctx.host["q_lens"], ctx.host["start_pos"],
                       window=self.window or 0, scale=self.scale, cu_q=ctx.cu_q, start_pos_dev=ctx.start_pos,
                       scratch=lambda n: ctx.scratch("attention.partials", n, torch.float32),
-                      max_pages_used=ctx.max_pages_used, rotation=rotation, new_kv=new_kv)
+                      max_pages_used=ctx.max_pages_used, rotation=rotation, new_kv=new_kv,
+                      seq_pages=getattr(ctx, "seq_pages", {}).get(kv.group) if ctx.max_q_len == 1 else None)

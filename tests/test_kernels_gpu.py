@@ -763,14 +763,15 @@ def _wider(table, bound):
 
 
 @pytest.mark.parametrize("bound", [None, 3000])
-@pytest.mark.parametrize("variant", [0, 1])
+@pytest.mark.parametrize("variant", [0, 1, "pages by sequence"])
 @pytest.mark.parametrize("H,KV,hd,rot,inter,window", [(4, 2, 16, 16, False, 0), (32, 8, 64, 64, False, 0), (6, 3, 48, 32, True, 0),
                                                        (40, 2, 32, 32, False, 0), (8, 8, 128, 128, True, 50), (4, 1, 80, 0, False, 0),
                                                        (6, 2, 80, 48, False, 0), (2, 1, 256, 256, False, 0)])
 def test_decode_attention_that_rotates_and_stores_by_itself(H, KV, hd, rot, inter, window, variant, bound):
     """One row per sequence: the split kernel given unrotated [q | k | v] rows against the two-kernel way
     (rotate and store, then attend): the same output, the same cache afterwards.  Also with a launch sized for
-    sequences of 3,000 pages, of whose blocks a short sequence uses a few."""
+    sequences of 3,000 pages, of whose blocks a short sequence uses a few; and with the sequences' page numbers given
+    by their place in the step, where the fused kernel must not look at the table by slot (which then holds nonsense)."""
     ops = _ops()
     from dlgo_amd.parts import rotary_frequencies
     dtype = torch.bfloat16
@@ -796,10 +797,16 @@ def test_decode_attention_that_rotates_and_stores_by_itself(H, KV, hd, rot, inte
         store = storage.clone().to(DEV)
         rows = qkv.clone().to(DEV)
         out = torch.empty(len(lens), H * hd, dtype=dtype, device=DEV)
-        common = dict(q_lens=[1] * len(lens), start_pos=[n - 1 for n in lens], window=window, kernel="split", split_variant=variant)
+        by_seq = variant == "pages by sequence"
+        common = dict(q_lens=[1] * len(lens), start_pos=[n - 1 for n in lens], window=window, kernel="split",
+                      split_variant=0 if by_seq else variant)
         if fused:
-            ops.attention(rows, out, H, KV, hd, positions, tok_seq, dslots, table.to(DEV), store[unit_off:], page_stride, v_off,
-                          rotation=(cos, sin, rot, inter) if rot else None, new_kv=True, **common)
+            extra, by_slot = {}, table.to(DEV)
+            if by_seq:
+                extra = dict(seq_pages=table[torch.tensor(slots, dtype=torch.long)].contiguous().to(DEV))
+                by_slot = torch.zeros_like(by_slot)          # every entry names page 0: of no use to anyone
+            ops.attention(rows, out, H, KV, hd, positions, tok_seq, dslots, by_slot, store[unit_off:], page_stride, v_off,
+                          rotation=(cos, sin, rot, inter) if rot else None, new_kv=True, **common, **extra)
         else:
             ops.rope_kv(rows, H, KV, hd, rot, inter, cos, sin, positions, tok_seq, dslots, table.to(DEV), store[unit_off:],
                         page_stride, v_off)
@@ -824,7 +831,7 @@ def _fill_pages(storage, table, slot, k, v, KV, hd, page_stride, unit_off, v_off
             storage[ov:ov + hd * PAGE].view(hd, PAGE)[:, :p1 - p0] = v[p0:p1, kvh * hd:(kvh + 1) * hd].T
 
 
-@pytest.mark.parametrize("kernel", ["bfloat16", "bfloat16 registers", "float32"])
+@pytest.mark.parametrize("kernel", ["bfloat16", "bfloat16 registers", "bfloat16 pages by sequence", "float32"])
 @pytest.mark.parametrize("H,KV,hd,bound,lens", [
     # 288 (sequence, kv head) pairs fill the chip by themselves: a sequence gets a second block from about 12,000 tokens
     (8, 8, 64, 400, [12500, 8200, 4097, 64, 65, 1] + [3 + 7 * i for i in range(30)]),
@@ -878,9 +885,13 @@ def test_decode_attention_of_short_sequences_in_a_launch_sized_for_long_ones(H, 
         q[:, :, axis] = 60.0
         q = q.reshape(n, H * hd).to(dtype).to(DEV)
         out = torch.full((n, H * hd), float("nan"), dtype=dtype, device=DEV)
-        ops.attention(q, out, H, KV, hd, positions, tok_seq, dslots, dtable, store[unit_off:], page_stride, v_off,
+        extra, by_slot = {}, dtable
+        if kernel == "bfloat16 pages by sequence":      # the pages' numbers by place in the step; the table by slot is not to be read
+            extra = dict(seq_pages=dtable[dslots.long()].contiguous())
+            by_slot = torch.zeros_like(dtable)
+        ops.attention(q, out, H, KV, hd, positions, tok_seq, dslots, by_slot, store[unit_off:], page_stride, v_off,
                       q_lens=[1] * n, start_pos=[x - 1 for x in lens], kernel="split", max_pages_used=bound,
-                      split_variant=1 if kernel == "bfloat16 registers" else 0)
+                      split_variant=1 if kernel == "bfloat16 registers" else 0, **extra)
         got = out.float().cpu().view(n, H, hd)
         for i in range(n):
             t = marks[i][axis]
