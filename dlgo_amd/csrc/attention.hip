@@ -885,24 +885,25 @@ struct Rot8In {
 };
 __device__ __forceinline__ Rot8In rot8_load(const bf16_t* __restrict__ vec, int d0, const float* __restrict__ cs,
                                             const float* __restrict__ sn, int rot, int interleaved) {
+  // Every load is made whatever the piece needs, from a place that can be read (the piece itself where nothing is
+  // wanted): with the loads under conditions the compiler waits for each before it goes on to the next, which made
+  // the queries four trips to memory instead of one.
   Rot8In r;
+  const bool turn = cs != nullptr && d0 < rot;
+  const int half = rot / 2;
+  const bool low = d0 < half;
+  const bool halves = turn && !interleaved;
+  const int partner = halves ? (low ? d0 + half : d0 - half) : d0;
+  const int i0 = !turn ? 0 : (interleaved ? d0 / 2 : (low ? d0 : d0 - half));
+  const int i1 = halves ? i0 + 4 : i0;
+  const float* c = turn ? cs : (const float*)vec;
+  const float* sp = turn ? sn : (const float*)vec;
   r.x = *(const uint4*)(vec + d0);
-  r.p = r.x;
-  r.c0 = r.c1 = r.s0 = r.s1 = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (cs == nullptr || d0 >= rot) return r;
-  if (interleaved) {
-    r.c0 = *(const float4*)(cs + d0 / 2);
-    r.s0 = *(const float4*)(sn + d0 / 2);
-  } else {
-    const int half = rot / 2;
-    const bool low = d0 < half;
-    const int i0 = low ? d0 : d0 - half;
-    r.p = *(const uint4*)(vec + (low ? d0 + half : d0 - half));
-    r.c0 = *(const float4*)(cs + i0);
-    r.c1 = *(const float4*)(cs + i0 + 4);
-    r.s0 = *(const float4*)(sn + i0);
-    r.s1 = *(const float4*)(sn + i0 + 4);
-  }
+  r.p = *(const uint4*)(vec + partner);
+  r.c0 = *(const float4*)(c + i0);
+  r.s0 = *(const float4*)(sp + i0);
+  r.c1 = *(const float4*)(c + i1);
+  r.s1 = *(const float4*)(sp + i1);
   return r;
 }
 __device__ __forceinline__ void unpack8(const uint4& u, float* f) {
@@ -1024,20 +1025,20 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_lds_kernel(
   // they would be one more trip to memory in the middle of the kernel).
   const bool takes_own = FUSED && new_kv && pg1 == last_pg && (last_pg - pg0) % NWV == wave;
   Rot8In kin[KS];
-  bf16_t v_own[DT];
-  if (takes_own) {
+  uint32_t v_own[DT];
+  if (FUSED) {
+    // (every lane of every wave makes these loads, a wave that does not take the token's own from the queries' row:
+    // loads under a condition would each be waited for in turn)
     const bf16_t* row = q + (size_t)seq * ldq;
-    const bf16_t* krow_new = row + k_col + (size_t)kvh * HD;
-    const bf16_t* vrow_new = row + v_col + (size_t)kvh * HD;
-    if (j == own_j) {
+    const bf16_t* krow_new = takes_own ? row + k_col + (size_t)kvh * HD : qrow;
+    const bf16_t* vrow_new = takes_own ? row + v_col + (size_t)kvh * HD : qrow;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks)
-        if (ks * 32 + G * 8 < HD) kin[ks] = rot8_load(krow_new, ks * 32 + G * 8, cs, sn, rot, interleaved);
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d0 = ks * 32 + G * 8 < HD ? ks * 32 + G * 8 : 0;
+      kin[ks] = rot8_load(krow_new, d0, cs, sn, rot, interleaved);
     }
-    if (G == ((own >> 3) & 3)) {
 #pragma unroll
-      for (int d = 0; d < DT; ++d) v_own[d] = vrow_new[d * 16 + j];
-    }
+    for (int d = 0; d < DT; ++d) v_own[d] = vrow_new[d * 16 + j];
   }
   int pg = pg0 + wave;
   int page_cur;
@@ -1120,7 +1121,7 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_lds_kernel(
           if (u == (own >> 5)) {
 #pragma unroll
             for (int d = 0; d < DT; ++d) {
-              const bf16_t val = v_own[d];
+              const bf16_t val = (bf16_t)v_own[d];
               uint32_t w4[4] = {vf[u][d].x, vf[u][d].y, vf[u][d].z, vf[u][d].w};
               const int e = own & 7;
 #pragma unroll
