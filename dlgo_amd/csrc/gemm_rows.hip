@@ -303,6 +303,9 @@ struct NormShares {
   float share[TOK_TURNS][SHARES];
   __device__ __forceinline__ void ask(const NormParts& np, int Tn) {
     if (MODE != 2) return;
+    // every load is made, from a place that holds a share (the row's first) where none is wanted, and what is not
+    // wanted is left out when the shares are added up: a load under a condition is waited for before the code after
+    // it goes on, and W's loads, which stand behind these, would start a trip to memory late
 #pragma unroll
     for (int turn = 0; turn < TOK_TURNS; ++turn) {
       const int t = turn * TOK_STEP + (threadIdx.x >> 4);
@@ -310,22 +313,22 @@ struct NormShares {
 #pragma unroll
       for (int u = 0; u < SHARES; ++u) {
         const int i = u * 16 + (threadIdx.x & 15);
-        share[turn][u] = t < Tn && i < np.n_parts ? p[i] : 0.f;
+        share[turn][u] = p[i < np.n_parts ? i : 0];
       }
     }
   }
-  __device__ __forceinline__ void leave(float* sumsq) const {
+  __device__ __forceinline__ void leave(float* sumsq, const NormParts& np, int Tn) const {
     if (MODE != 2) return;
 #pragma unroll
     for (int turn = 0; turn < TOK_TURNS; ++turn) {
+      const int t = turn * TOK_STEP + (threadIdx.x >> 4);
       float sh = 0.f;
 #pragma unroll
-      for (int u = 0; u < SHARES; ++u) sh += share[turn][u];
+      for (int u = 0; u < SHARES; ++u) sh += (t < Tn && u * 16 + (int)(threadIdx.x & 15) < np.n_parts) ? share[turn][u] : 0.f;
       sh += __shfl_xor(sh, 1, WAVE);
       sh += __shfl_xor(sh, 2, WAVE);
       sh += __shfl_xor(sh, 4, WAVE);
       sh += __shfl_xor(sh, 8, WAVE);
-      const int t = turn * TOK_STEP + (threadIdx.x >> 4);
       if ((threadIdx.x & 15) == 0 && t < 16) sumsq[t] = sh;
     }
   }
@@ -469,7 +472,7 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_kernel(const T* __rest
       for (int s_ = 0; s_ < STEPS; ++s_) Mma16<T>::run(aop[s_], b[s_], acc[r]);
     }
   }
-  shares.leave(sumsq);
+  shares.leave(sumsq, np, Tn);
   __syncthreads();
   const float sc = MODE == 2 ? 1.0f / sqrtf(sumsq[j] / (float)np.width + np.eps) : 1.f;
   float* red = (float*)lds_raw;                // [NW][16][17]
@@ -535,7 +538,7 @@ __global__ __launch_bounds__(NW* WAVE) void skinny_stream_long_kernel(const T* _
     multiply(turn, b0, b1);
     if (turn + 1 < turns) multiply(turn + 1, b1, b0);
   }
-  shares.leave(sumsq);
+  shares.leave(sumsq, np, Tn);
   __syncthreads();
   const float sc = MODE == 2 ? 1.0f / sqrtf(sumsq[j] / (float)np.width + np.eps) : 1.f;
   stream_finish<T, NW, EPI, MODE>((float*)lds_raw, acc, Y, ldy, N, n0, tok, sc, np, blockIdx.x, j, ahead);
