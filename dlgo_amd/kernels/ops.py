@@ -484,12 +484,15 @@ def rope_kv(qkv: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, rot: int,
             cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], positions: torch.Tensor,
             tok_seq: Optional[torch.Tensor], slots: Optional[torch.Tensor], page_table: Optional[torch.Tensor],
             cache: Optional[torch.Tensor], page_stride: int, v_off: int, write_kv: bool = True,
-            unsummed: Optional[UnsummedRows] = None, single_tokens: bool = False) -> None:
+            unsummed: Optional[UnsummedRows] = None, single_tokens: bool = False,
+            seq_pages: Optional[torch.Tensor] = None) -> None:
     """Rotate the query heads of qkv [T, (H+2KV)*hd] in place; rotate the key heads and copy the value heads
     into the cache page of each token (cache: the first element of this layer's pages).  unsummed: the rows are not
     in qkv yet but in the runs that gemm_runs left (see rope_takes_unsummed); the rotated queries are written to qkv.
     single_tokens: every row is a sequence of its own (a hint for how the transposed values are best stored; the
-    result is the same)."""
+    result is the same).  seq_pages: for such a step, the sequences' page-table rows in the order of the rows
+    ([>= T, the table's width], row i = page_table[slots[tok_seq[i]]]); the kernel then reads a row's page from there
+    without going through its sequence and slot."""
     _need(qkv, "qkv rows", dims=2)
     _need(positions, "positions", torch.int32, 1)
     t = qkv.shape[0]
@@ -511,6 +514,13 @@ def rope_kv(qkv: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, rot: int,
         if tok_seq.shape[0] != t or not page_table.is_contiguous():
             raise KernelError("rope_kv: one sequence index per row and a contiguous page table")
         max_pages = page_table.shape[1]
+    by_row = write_kv and seq_pages is not None
+    if by_row:
+        _need(seq_pages, "pages by sequence", torch.int32, 2)
+        if not single_tokens or seq_pages.shape[0] < t or seq_pages.shape[1] != max_pages or not seq_pages.is_contiguous():
+            raise KernelError(f"rope_kv: pages by sequence {tuple(seq_pages.shape)} do not fit {t} single-token rows "
+                              f"and a table {max_pages} wide")
+        page_table = seq_pages
     part = (_ptr(None), 0, ctypes.c_longlong(0), 0)
     if unsummed is not None:
         if unsummed.rows != t or unsummed.cols < (n_heads + (2 * n_kv if write_kv else 0)) * head_dim:
@@ -520,7 +530,7 @@ def rope_kv(qkv: torch.Tensor, n_heads: int, n_kv: int, head_dim: int, rot: int,
                                         rot, int(interleaved), _ptr(cos), _ptr(sin), table_rows, _ptr(positions),
                                         _ptr(tok_seq), _ptr(slots), _ptr(page_table), max_pages, _ptr(cache),
                                         ctypes.c_longlong(page_stride), ctypes.c_longlong(v_off), int(write_kv), *part,
-                                        int(single_tokens), _stream()))
+                                        int(single_tokens), int(by_row), _stream()))
 
 
 def rope_takes_unsummed(dtype: torch.dtype, head_dim: int, rot: int) -> bool:

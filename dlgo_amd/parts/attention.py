@@ -184,7 +184,8 @@ class Attention(Mixer):
             ops.rope_kv(qkv, self.n_heads, n_kv, self.head_dim, rot.width if rot else 0, rot.interleaved if rot else False,
                         rot.cos if rot else None, rot.sin if rot else None, ctx.positions,
                         ctx.tok_seq, ctx.slots, kv.page_table, kv.cache, kv.page_stride, kv.v_off, write_kv=owns_cache,
-                        unsummed=unsummed, single_tokens=ctx.max_q_len == 1)
+                        unsummed=unsummed, single_tokens=ctx.max_q_len == 1,
+                        seq_pages=getattr(ctx, "seq_pages", {}).get(kv.group) if ctx.max_q_len == 1 else None)
         out = ctx.buffer("attention.out", (t, self.q_dim), ctx.dtype)
         self.attend(qkv, out, ctx, kv, rotation=(rot.cos, rot.sin, rot.width, rot.interleaved) if fused and rot else None,
                     new_kv=fused and owns_cache)

@@ -607,6 +607,43 @@ def test_rope_kv_from_unsummed_runs(dtype, _, rel, H, KV, hd, rot, inter, write)
         assert torch.equal(torch.nan_to_num(got[0][1].float(), nan=-77.0), torch.nan_to_num(other[1].float(), nan=-77.0)), "pages"
 
 
+@pytest.mark.parametrize("dtype,_,rel", DT)
+@pytest.mark.parametrize("H,KV,hd,rot,inter", [(4, 2, 16, 16, False), (6, 3, 48, 32, True), (8, 1, 128, 128, False), (3, 1, 6, 6, False)])
+def test_rope_kv_of_single_tokens_finds_the_pages_by_row(dtype, _, rel, H, KV, hd, rot, inter):
+    """A step of single tokens with the sequences' page-table rows given in the order of the rows writes the pages that
+    the way through sequence and slot writes, bit for bit.  The table by slot is then not read: it holds holes only."""
+    ops = _ops()
+    from dlgo_amd.parts import rotary_frequencies
+    lens = [70, 3, 129, 64, 65]
+    table, slots, storage, page_stride, unit_off, v_off = _paged_setup(dtype, lens, KV, hd)
+    T = len(lens)
+    g = torch.Generator().manual_seed(11)
+    rows = torch.randn(T, (H + 2 * KV) * hd, generator=g)
+    positions = torch.tensor([l - 1 for l in lens], dtype=torch.int32).to(DEV)
+    order = [3, 0, 4, 1, 2]                                    # the rows' sequences, not in the order of the rows
+    tok_seq = torch.tensor(order, dtype=torch.int32).to(DEV)
+    positions = positions[tok_seq.long()]
+    freqs = rotary_frequencies(rot, 10000.0)
+    ang = np.arange(200)[:, None] * freqs[None]
+    cos, sin = torch.from_numpy(np.cos(ang).astype(np.float32)).to(DEV), torch.from_numpy(np.sin(ang).astype(np.float32)).to(DEV)
+    slot_t = torch.tensor(slots, dtype=torch.int32, device=DEV)
+    by_row = torch.full((T + 3, table.shape[1]), -1, dtype=torch.int32)
+    by_row[:T] = table[torch.tensor(slots)[torch.tensor(order)]]
+    got = []
+    for pages, by_slot in ((None, table), (by_row.to(DEV), torch.full_like(table, -1))):
+        dq = rows.to(dtype).to(DEV)
+        store = storage.clone().to(DEV)
+        ops.rope_kv(dq, H, KV, hd, rot, inter, cos, sin, positions, tok_seq, slot_t, by_slot.to(DEV), store[unit_off:], page_stride,
+                    v_off, single_tokens=True, seq_pages=pages)
+        got.append((dq[:, :H * hd].cpu(), store.cpu()))
+    assert (~torch.isnan(got[0][1].float())).sum().item() == T * 2 * KV * hd
+    assert torch.equal(got[0][0], got[1][0]), "rotated queries"
+    assert torch.equal(torch.nan_to_num(got[0][1].float(), nan=-77.0), torch.nan_to_num(got[1][1].float(), nan=-77.0)), "pages"
+    with pytest.raises(ops.KernelError, match="pages by sequence"):
+        ops.rope_kv(rows.to(dtype).to(DEV), H, KV, hd, rot, inter, cos, sin, positions, tok_seq, slot_t, table.to(DEV),
+                    storage.clone().to(DEV)[unit_off:], page_stride, v_off, single_tokens=True, seq_pages=by_row[:T - 1].to(DEV))
+
+
 def _attention_ref(q, k, v, H, KV, hd, pos_of_q, lo_of_q):
     """q [n, H*hd]; k, v [len, KV*hd] for one sequence; row i attends keys lo..pos."""
     g = H // KV
