@@ -141,3 +141,41 @@ def test_functions_that_return_a_message_are_told_so():
             assert name in listed, f"{name} returns a message but `_lib` does not set its return type"
         else:
             assert name not in listed, f"{name} returns {decl[name][1]}, not a message"
+
+
+def test_the_choice_of_product_kernel_is_made_on_the_host(monkeypatch):
+    """The rules that choose between the streamed and the tiled products count bytes, blocks and rows and ask the
+    library's own planning functions, none of which touches a device: the table that the GPU test checks together with
+    the products' results holds here too, for tensors that have a shape and nothing else, given 256 compute units."""
+    import torch
+
+    from dlgo_amd.kernels import ops
+    from test_kernels_gpu import CHOICES
+    monkeypatch.setattr(ops, "_cus", {0: 256})
+    for n, k, t, streamed in CHOICES:
+        w = torch.empty(n, k, dtype=torch.bfloat16, device="meta")
+        assert ops.gemm_streams(w, t) is streamed, (n, k, t)
+    # float32 rows are twice as long: the same widths fall on the other side of a rule
+    w = torch.empty(2048, 4096, dtype=torch.float32, device="meta")
+    assert ops.gemm_streams(w, 8) is ops.gemm_streams(torch.empty(2048, 8192, dtype=torch.bfloat16, device="meta"), 8)
+
+
+def test_the_decode_attention_plans_its_splits_within_the_pages():
+    """How many blocks share a sequence's pages in a step of single tokens is planned on the host from counts alone:
+    for every shape there is at least one block, never more blocks than the longest sequence may have pages, and a
+    step with many sequences does not split at all without long sequences to balance."""
+    import ctypes
+
+    from dlgo_amd.kernels import build
+    for head_dim in (64, 128):
+        lib = build.load("attention", (("HEAD_DIM", head_dim),))
+        lib.dlgo_attention_decode_splits.restype = ctypes.c_int
+        for n_seq in (1, 2, 8, 31, 64, 300):
+            for n_heads, n_kv in ((32, 8), (24, 8), (6, 3), (40, 40), (64, 2)):
+                for pages in (1, 3, 33, 64, 512, 2048):
+                    for fused in (0, 1):
+                        for variant in (0, 1):
+                            s = lib.dlgo_attention_decode_splits(n_seq, n_heads, n_kv, pages, fused, variant)
+                            assert 1 <= s <= pages, (head_dim, n_seq, n_heads, n_kv, pages, fused, variant, s)
+                            if n_seq * n_kv >= 256 and pages <= 64:
+                                assert s == 1, (head_dim, n_seq, n_heads, n_kv, pages, fused, variant, s)
