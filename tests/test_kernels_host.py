@@ -1,8 +1,12 @@
-"""The launches in `dlgo_amd/kernels/ops.py` against the `extern "C"` declarations they call, read from the sources:
+"""What can be said of the kernels without a device.
+
+The launches in `dlgo_amd/kernels/ops.py` against the `extern "C"` declarations they call, read from the sources:
 the number of arguments, and for every argument whose kind can be told from the call's text (a pointer, a stream, a
 64-bit integer, a float) that the C parameter at its place is of that kind.  ctypes checks none of this without
 declared argument types: a call with one argument too few, or a 64-bit count passed as a plain int, runs and reads
-garbage.  Needs neither GPU nor compiler."""
+garbage.  Then what the libraries decide on the host alone: which product kernel a shape gets, how the decode
+attention splits a sequence's pages, which widths the norm's hand-off covers, and what the launchers refuse before
+they touch a device.  These need the compiler (the libraries are built at first use) but no GPU."""
 import ast
 import re
 from pathlib import Path
@@ -179,3 +183,55 @@ def test_the_decode_attention_plans_its_splits_within_the_pages():
                             assert 1 <= s <= pages, (head_dim, n_seq, n_heads, n_kv, pages, fused, variant, s)
                             if n_seq * n_kv >= 256 and pages <= 64:
                                 assert s == 1, (head_dim, n_seq, n_heads, n_kv, pages, fused, variant, s)
+
+
+def test_the_norm_hand_off_of_few_rows_knows_its_width():
+    """A streamed product that leaves a norm keeps a share of every row's sum of squares per block of weight rows, and
+    the product that applies the norm reads as many: beyond the widths those shares cover (256 of them), both say no,
+    so that a model of hidden size 5,120 or 8,192 takes the norm kernel instead of a hand-off that cannot hold it."""
+    import torch
+
+    from dlgo_amd.kernels import ops
+
+    def w(n, k):
+        return torch.empty(n, k, dtype=torch.bfloat16, device="meta")
+    for width in (2048, 3072, 4096):
+        assert ops.streams_few_rows(w(width, width), 8, ops.ROLE_LEAVES_NORM), width
+        assert ops.streams_few_rows(w(4 * width, width), 8, ops.ROLE_APPLIES_NORM), width
+    for width in (5120, 8192):
+        assert ops.streams_few_rows(w(width, width), 8, ops.ROLE_PLAIN), width
+        assert not ops.streams_few_rows(w(width, width), 8, ops.ROLE_LEAVES_NORM), width
+        assert not ops.streams_few_rows(w(4 * width, width), 8, ops.ROLE_APPLIES_NORM), width
+    assert not ops.streams_few_rows(w(2048, 2048), 17, ops.ROLE_PLAIN)       # more rows than the streamed kernels take
+    assert not ops.streams_few_rows(w(2048, 2040), 8, ops.ROLE_PLAIN)        # weight rows that are no whole kilobytes
+
+
+def test_launchers_refuse_what_their_kernels_do_not_take():
+    """Argument checks of the launchers come before anything touches a device, so the refusals can be read here: each
+    names what was wrong."""
+    import ctypes
+
+    from dlgo_amd.kernels import build
+    null, i64 = ctypes.c_void_p(0), ctypes.c_longlong
+    rope = build.load("rope_kv")
+    rope.dlgo_rope_kv.restype = ctypes.c_char_p
+
+    def rope_kv(hd=64, rot=64, ld=None, n_heads=4, n_kv=2, write_kv=0):
+        ld = (n_heads + 2 * n_kv) * hd if ld is None else ld
+        return rope.dlgo_rope_kv(null, 1, 3, ld, n_heads, n_kv, hd, rot, 0, null, null, 0, null, null, null, null, 0, null, i64(0),
+                                 i64(0), write_kv, null, 0, i64(0), 0, 0, 0, null)
+    assert b"rotated width" in rope_kv(rot=63) and b"rotated width" in rope_kv(rot=80)
+    assert b"row stride" in rope_kv(ld=100)
+    assert b"cache arguments missing" in rope_kv(write_kv=1)
+    att = build.load("attention", (("HEAD_DIM", 64),))
+    att.dlgo_attention_decode.restype = ctypes.c_char_p
+
+    def decode(head_dim=64, n_heads=32, n_kv=8, max_pages=4, used=4, variant=0, ldq=2048):
+        return att.dlgo_attention_decode(null, ldq, null, 2048, null, i64(0), 2, n_heads, n_kv, head_dim, null, null, null, max_pages,
+                                         used, null, i64(0), i64(0), 0, ctypes.c_float(0.125), null, null, 0, 0, 0, 0, variant,
+                                         null, null)
+    assert b"built for head size 64, got 128" in decode(head_dim=128)
+    assert b"bad sizes" in decode(n_heads=30)
+    assert b"bound on the pages" in decode(used=5)
+    assert b"unknown variant" in decode(variant=7)
+    assert b"row strides" in decode(ldq=100)
