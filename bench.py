@@ -11,7 +11,8 @@ models/llm/generate.go:227-229,275-282): after W warm-up steps the next K steps
 are the timed ones, taken as five regions; the figures are the median region's.
 Random weights, seeded uniform-random token ids, no stop tokens.  Prints ONE JSON
 line.  --breakdown adds "kernels": the time of every launch of one decode step,
-by kind, made one by one between events (gpu_timing_main.go:73-119).
+by kind, made one by one between events (gpu_timing_main.go:73-119), and
+"prefill_kernels": the same for one prompt step.
 
 Peaks used for the fractions (MI355X, published): HBM 8 TB/s; dense MFMA bf16
 2.5 PFLOP/s, fp32 157.3 TFLOP/s.
@@ -158,6 +159,38 @@ def breakdown(eng, sampler, cfg, batch, rng, steps=8):
     return out
 
 
+def prefill_breakdown(eng, cfg, rng, tokens):
+    """One prompt step of `tokens` rows, launch by launch between events, as `breakdown` does for a decode step.  The
+    prompt is one token shorter than the benchmark's, a shape the engine has not seen, so the step is made of its
+    launches and not replayed from a recording; its kernels are long enough that the device does not wait for the host
+    between them.  Returns {kind of launch: [microseconds, launches]}, their sum, the launches and the events' share."""
+    import torch
+
+    from dlgo_amd.engine import Entry
+    from dlgo_amd.kernels import ops
+    prompt = rng.integers(0, cfg.vocab_size, size=tokens).tolist()
+    slots = eng.open(1)
+    torch.cuda.synchronize()
+    with ops.Timings() as t:
+        eng.step([Entry(slots[0], prompt, [tokens - 1])])
+        pairs = []
+        for _ in range(8):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            b.record()
+            pairs.append((a, b))
+        torch.cuda.synchronize()
+    us, n = t.microseconds(), t.launches()
+    eng.close(slots)
+    pair = sum(a.elapsed_time(b) for a, b in pairs) * 1000.0 / len(pairs)
+    out = {k: [round(max(0.0, v - n[k] * pair), 1), n[k]] for k, v in sorted(us.items(), key=lambda kv: -kv[1])}
+    out["sum"] = round(sum(v[0] for v in out.values()), 1)
+    out["launches"] = sum(n.values())
+    out["event_pair"] = round(pair, 2)
+    out["tokens"] = tokens
+    return out
+
+
 def main() -> int:
     global PROMPT, CONTEXT
     ap = argparse.ArgumentParser()
@@ -171,7 +204,8 @@ def main() -> int:
     ap.add_argument("--point-steps", type=int, default=64)
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--breakdown", action="store_true",
-                    help="add \"kernels\": microseconds of one decode step of --batch by kind of launch, each launch timed between events")
+                    help="add \"kernels\": microseconds of one decode step of --batch by kind of launch, each launch timed between events, "
+                         "and \"prefill_kernels\": the same for one prompt step")
     ap.add_argument("--ragged", default="", metavar="N:LO:HI:NEW:CTX",
                     help="instead of the default run: N requests with prompts of LO..HI tokens (uniform, seeded), NEW "
                          "generated tokens each, context CTX, through the generation loop")
@@ -258,9 +292,14 @@ def main() -> int:
         prefill = {"value": round(PROMPT / pt, 1), "tokens": PROMPT, "ms": round(pt * 1000.0, 3),
                    "frac": round(prefill_flops(cfg, PROMPT) / pt / FLOP_PEAK[args.dtype], 4)}
 
-    kernels = None
+    kernels = prefill_kernels = None
     if args.breakdown:
         kernels = breakdown(eng, sampler, cfg, args.batch, rng)
+        if not args.no_prefill and PROMPT > 1:
+            try:
+                prefill_kernels = prefill_breakdown(eng, cfg, rng, PROMPT - 1)
+            except Exception as e:      # the line's other figures are measured by now: say what went wrong beside them
+                prefill_kernels = {"error": f"{type(e).__name__}: {e}"}
 
     line = {
         "metric": f"decode tok/s @ batch {args.batch} ({args.shape} shape, {PROMPT}-token prompts, context {CONTEXT})",
@@ -282,6 +321,8 @@ def main() -> int:
         line["prefill"] = prefill
     if kernels is not None:
         line["kernels"] = kernels
+    if prefill_kernels is not None:
+        line["prefill_kernels"] = prefill_kernels
     print(json.dumps(line))
     return 0
 
