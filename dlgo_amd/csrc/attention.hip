@@ -962,8 +962,8 @@ __global__ __launch_bounds__(NWV* WAVE) void attn_decode_lds_kernel(
   const int split = blockIdx.z, seq = blockIdx.y;         // as attn_decode_kernel
   // The kv head of a block turns with its sequence and its share of the pages.  A block runs on the XCD that its linear
   // number mod 8 names; with the kv head straight from blockIdx.x and eight kv heads, an XCD would read one head for
-  // good, and a head's keys and values lie at the same 8 KB (head size 64) of every 64 KB of the cache: of the address
-  // bits that spread reads over an L2's channels, that XCD would only ever see one value.
+  // good, and a head's keys and values lie at the same 8 KB (head size 64) of every 64 KB of the cache.  Whatever
+  // address bits an L2 spreads its reads by, every XCD now sees all of them; the reads and sums are the same.
   const int kvh = (int)((blockIdx.x / head_blocks + seq + split) % (gridDim.x / head_blocks)), hb = blockIdx.x % head_blocks;
   // Which page a wave takes first depends on the sequence's length, which is a trip to memory away.  With the pages
   // listed by sequence their place is known at once, so every lane asks for a candidate now: lane s - 1 for the page the
