@@ -520,6 +520,23 @@ def test_command_line_writes_a_random_model_or_says_why_not(tmp_path, capsys):
     assert main(["--write-random", str(tmp_path / "nope.json"), out]) == 1 and "no such file" in capsys.readouterr().err
 
 
+def test_command_line_takes_a_folder_or_a_configuration_to_draw_weights_for(tmp_path, capsys):
+    """Exactly one of MODEL_DIR and --random-config; without a GPU either ends in one line that says so, no traceback."""
+    import json
+    from conftest import TINY_A
+    from dlgo_amd.cli import main
+    (tmp_path / "c.json").write_text(json.dumps(TINY_A))
+    for argv in ([], ["x", "--random-config", str(tmp_path / "c.json")]):
+        with pytest.raises(SystemExit) as e:
+            main(argv)
+        assert e.value.code == 2 and "one of them" in capsys.readouterr().err
+    if not torch.cuda.is_available():
+        assert main(["--random-config", str(tmp_path / "c.json"), "--weight-seed", "3", "--prompt-ids", "1,2"]) == 1
+        err = capsys.readouterr().err
+        assert err.startswith("Error loading model:") and "no HIP device" in err and "Traceback" not in err
+    assert main(["--random-config", str(tmp_path / "missing.json")]) == 1 and "Error loading model" in capsys.readouterr().err
+
+
 def test_engine_refuses_to_run_without_a_gpu(tmp_path):
     if torch.cuda.is_available():
         pytest.skip("a GPU is present")
