@@ -537,6 +537,32 @@ def test_command_line_takes_a_folder_or_a_configuration_to_draw_weights_for(tmp_
     assert main(["--random-config", str(tmp_path / "missing.json")]) == 1 and "Error loading model" in capsys.readouterr().err
 
 
+def test_replay_program_checks_its_arguments_before_anything_else(tmp_path):
+    """bin/trace_run takes exactly one of --model and --config and a positive --max-tokens; a model that cannot be
+    loaded (here: no GPU) ends in one line and status 1, an empty input in status 0 only after a model is there."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+    from conftest import TINY_A
+    prog = str(Path(__file__).resolve().parents[1] / "bin" / "trace_run")
+    (tmp_path / "c.json").write_text(json.dumps(TINY_A))
+    common = ["--dtype", "float32", "--out", str(tmp_path / "out"), "--max-tokens", "64"]
+
+    def run(*argv):
+        return subprocess.run([sys.executable, prog, *argv], input="", capture_output=True, text=True, timeout=300)
+    r = run(*common)
+    assert r.returncode == 2 and "one of --model DIR and --config FILE" in r.stderr
+    r = run("--model", str(tmp_path), "--config", str(tmp_path / "c.json"), *common)
+    assert r.returncode == 2 and "one of --model DIR and --config FILE" in r.stderr
+    r = run("--config", str(tmp_path / "c.json"), "--dtype", "float32", "--out", str(tmp_path / "out"), "--max-tokens", "0")
+    assert r.returncode == 2 and "--max-tokens must be > 0" in r.stderr
+    if not torch.cuda.is_available():
+        r = run("--config", str(tmp_path / "c.json"), "--weight-seed", "3", *common)
+        assert r.returncode == 1 and "trace_run: cannot load" in r.stderr and "no HIP device" in r.stderr
+        assert "Traceback" not in r.stderr
+
+
 def test_engine_refuses_to_run_without_a_gpu(tmp_path):
     if torch.cuda.is_available():
         pytest.skip("a GPU is present")
